@@ -1,0 +1,175 @@
+"""Pins the decode-GEMM oracle (decode_gemm.py:368-401, gemm.py:393-400,450-456,1575-1617,
+common.py:98-114) and the integer routing helpers (model.py:451-491,557).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import clib
+from oracle import lyra_oracle as O
+
+
+def test_expert_ids_and_padding_rule():
+    np.testing.assert_array_equal(O.expert_ids([2, 0, 3], 5), [0, 0, 2, 2, 2])
+    np.testing.assert_array_equal(O.expert_ids([1, 1], 2), [0, 1])
+    # rows beyond sum(group_sizes): every group start <= the sum, so the gather lands on G-1
+    np.testing.assert_array_equal(O.expert_ids([2, 0, 0], 4), [0, 0, 2, 2])
+    np.testing.assert_array_equal(O.expert_ids([1, 0, 1, 0], 4), [0, 2, 3, 3])
+
+
+def test_normalize_bias_shapes():
+    assert O.normalize_bias(None, 3, 8).shape == (3, 1, 8)
+    assert O.normalize_bias(np.ones((3, 8)), 3, 8).shape == (3, 1, 8)
+    with pytest.raises(ValueError):
+        O.normalize_bias(np.ones((3, 2, 8)), 3, 8)
+
+
+def test_swiglu_closed_forms():
+    # zero gate -> 0 whatever the linear half
+    assert O.swiglu(np.array([[0.0, 5.0]], np.float32))[0, 0] == 0.0
+    # gate clamp at 7 (min only), linear clamp at +-7, +1 shift
+    x = np.array([[100.0, 100.0], [100.0, -100.0], [-100.0, 3.0], [2.0, -1.0]], np.float32)
+    y = O.swiglu(x)
+    sig7 = 1.0 / (1.0 + np.exp(-1.702 * 7.0))
+    np.testing.assert_allclose(y[0, 0], (7.0 + 1.0) * 7.0 * sig7, rtol=1e-6)
+    np.testing.assert_allclose(y[1, 0], (-7.0 + 1.0) * 7.0 * sig7, rtol=1e-6)
+    np.testing.assert_allclose(y[2, 0], (3.0 + 1.0) * -100.0 / (1.0 + np.exp(170.2)), rtol=1e-5, atol=1e-30)
+    assert y[3, 0] == 0.0  # lin = -1 -> (lin + 1) = 0
+    # first half gates, second half is linear (split, not interleave): common.py:109
+    z = O.swiglu(np.array([[1.0, 2.0, 10.0, 20.0]], np.float32))
+    sig = lambda g: 1.0 / (1.0 + np.exp(-1.702 * g))
+    np.testing.assert_allclose(z[0], [(7.0 + 1) * 1.0 * sig(1.0), (7.0 + 1) * 2.0 * sig(2.0)], rtol=1e-6)
+    # against torch's own sigmoid
+    rng = np.random.default_rng(0)
+    a = (rng.standard_normal((5, 64)) * 4).astype(np.float32)
+    t = torch.from_numpy(a)
+    g, l = t[:, :32].clamp(max=7.0), t[:, 32:].clamp(-7.0, 7.0)
+    np.testing.assert_allclose(O.swiglu(a), ((l + 1) * g * torch.sigmoid(1.702 * g)).numpy(), rtol=2e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("sizes,M", [([3, 0, 2, 1], 6), ([0, 0, 4, 0], 4), ([1, 1, 1, 1], 4), ([2, 1, 0, 0], 5)])
+def test_grouped_gemm_is_per_group_matmul(sizes, M):
+    rng = np.random.default_rng(1)
+    G, K, N = len(sizes), 32, 16
+    lhs = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    rhs = O.bf16_round(rng.standard_normal((G, K, N)).astype(np.float32))
+    bias = rng.standard_normal((G, N)).astype(np.float32)
+    got = O.grouped_gemm_reference(lhs, rhs, np.array(sizes), bias=bias)
+    want = np.zeros((M, N), np.float32)
+    row = 0
+    for g, n in enumerate(sizes):
+        for _ in range(n):
+            want[row] = (torch.from_numpy(lhs[row]).double() @ torch.from_numpy(rhs[g]).double()).float().numpy() + bias[g]
+            row += 1
+    for r in range(row, M):  # padding rows: zero product + bias of expert G-1
+        want[r] = bias[G - 1]
+    np.testing.assert_allclose(got, want, atol=1e-5, rtol=1e-5)
+
+
+def test_brute_force_tiny_with_swiglu():
+    rng = np.random.default_rng(2)
+    M, G, K, N = 3, 2, 4, 6
+    lhs = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    rhs = O.bf16_round(rng.standard_normal((G, K, N)).astype(np.float32))
+    sizes = np.array([1, 2])
+    got = O.decode_gemm_reference(lhs, rhs, sizes, fused_swiglu=True)
+    ids = [0, 1, 1]
+    for r in range(M):
+        t = [sum(float(lhs[r, k]) * float(rhs[ids[r], k, n]) for k in range(K)) for n in range(N)]
+        for j in range(N // 2):
+            glu, lin = min(t[j], 7.0), max(-7.0, min(7.0, t[N // 2 + j]))
+            want = (lin + 1.0) * glu / (1.0 + np.exp(-1.702 * glu))
+            np.testing.assert_allclose(got[r, j], want, rtol=1e-5, atol=1e-6)
+
+
+def test_fp8_weights_dequantise_to_bf16_first():
+    rng = np.random.default_rng(3)
+    M, G, K, N = 5, 3, 512, 256
+    lhs = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    w = (rng.standard_normal((G, K, N)) * 0.02).astype(np.float32)
+    sizes = np.array([2, 0, 3])
+    for block in ((256, 256), (K, 1)):
+        q, s = O.quantize(w, block)
+        wd = O.dequantize(q, s, block, to_bf16=True)
+        a = O.decode_gemm_reference(lhs, (q, s), sizes, block=block, mode="ref")
+        b = O.grouped_gemm_reference(lhs, wd, sizes, mode="ref")
+        np.testing.assert_array_equal(a, b)
+        f = O.decode_gemm_reference(lhs, (q, s), sizes, block=block, mode="fp32")
+        assert np.abs(f - a).max() < 2e-2
+    assert O.default_weight_block(2048, 4096) == (256, 256) and O.default_weight_block(2880, 2880) == (64, 64)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_c_oracle_matches_numpy_oracle(fp8, swiglu):
+    rng = np.random.default_rng(4)
+    M, G, K, N = 9, 4, 512, 256
+    lhs = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    w = (rng.standard_normal((G, K, N)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal((G, N)).astype(np.float32)
+    sizes = np.array([4, 0, 1, 3], np.int32)  # one padding row
+    for mode in ("fp32", "ref"):
+        if fp8:
+            q, s = O.quantize(w, (256, 256))
+            want = O.decode_gemm_reference(lhs, (q, s), sizes, block=(256, 256), bias=bias, fused_swiglu=swiglu, mode=mode)
+            got = clib.decode_gemm(O.bf16_bits(lhs), q, s, (256, 256), sizes, bias, fused_swiglu=swiglu, ref_rounding=(mode == "ref"))
+        else:
+            wb = O.bf16_round(w)
+            want = O.decode_gemm_reference(lhs, wb, sizes, bias=bias, fused_swiglu=swiglu, mode=mode)
+            got = clib.decode_gemm(O.bf16_bits(lhs), O.bf16_bits(wb), None, None, sizes, bias, fused_swiglu=swiglu, ref_rounding=(mode == "ref"))
+        tol = 3e-5 if mode == "fp32" else 1.6e-2
+        np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
+
+
+def test_routing_topk_softmax_bincount():
+    logits = np.array([[0.1, 2.0, 2.0, -1.0, 0.5], [3.0, -2.0, 0.0, 3.0, 3.0]], np.float32)
+    scores, active, groups = O.route_tokens(logits, 3, 5, 1)
+    # stable top-k: ties resolve to the lower index (lax.top_k)
+    np.testing.assert_array_equal(active.reshape(2, 4), [[1, 2, 4, 5], [0, 3, 4, 5]])
+    np.testing.assert_allclose(scores[0, :3], torch.softmax(torch.tensor([2.0, 2.0, 0.5]), 0).numpy(), rtol=1e-6)
+    np.testing.assert_array_equal(scores[:, 3], [1.0, 1.0])  # shared expert joins with score 1 (model.py:476)
+    np.testing.assert_array_equal(groups, [1, 1, 1, 1, 2, 2])
+
+
+def test_bpermute_is_stable_counting_sort():
+    # input vector of the reference's tests/test_combine.py:13-15
+    assignments = np.array([0, 2, 4, 7, 1, 3, 4, 7], np.int32)
+    groups = np.bincount(assignments, minlength=8)
+    perm, dest = O.bpermute(assignments, groups, 8)
+    np.testing.assert_array_equal(perm, np.argsort(assignments, kind="stable"))
+    np.testing.assert_array_equal(perm, [0, 4, 1, 5, 2, 6, 3, 7])
+    np.testing.assert_array_equal(dest[perm], np.arange(8))
+    rng = np.random.default_rng(5)
+    for _ in range(20):
+        a = rng.integers(0, 6, 40)
+        perm, dest = O.bpermute(a, np.bincount(a, minlength=6), 6)
+        np.testing.assert_array_equal(perm, np.argsort(a, kind="stable"))
+        np.testing.assert_array_equal(np.argsort(perm), dest)
+
+
+def test_combine_weighted_sum():
+    rng = np.random.default_rng(6)
+    F, k, C, E = 4, 3, 8, 5
+    a = rng.integers(0, E, F * k)
+    perm, dest = O.bpermute(a, np.bincount(a, minlength=E), E)
+    tokens = rng.standard_normal((F, C)).astype(np.float32)
+    rows = tokens[perm // k]  # model.py:521
+    scores = rng.random((F, k)).astype(np.float32)
+    got = O.combine(rows, scores, dest)
+    np.testing.assert_allclose(got, tokens * scores.sum(-1, keepdims=True), rtol=1e-5, atol=1e-6)
+
+
+def test_rms_norm_and_rotate_against_torch():
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((3, 64)).astype(np.float32)
+    w = rng.standard_normal(64).astype(np.float32)
+    want = torch.nn.functional.rms_norm(torch.from_numpy(x), (64,), torch.from_numpy(w), eps=1e-5).numpy()
+    np.testing.assert_allclose(O.rms_norm(x, w, 1e-5), want, rtol=2e-6, atol=1e-6)
+    cos, sin = O.rope_tables(16, 64)
+    assert cos.shape == (16, 32) and cos[0].min() == 1.0 and np.abs(sin[0]).max() == 0.0
+    # rotation by angle theta of the pair (x1_i, x2_i) = (x_i, x_{i+H/2}) preserves its norm
+    r = O.rotate(x[:1], cos[5], sin[5])
+    np.testing.assert_allclose(r[0, :32] ** 2 + r[0, 32:] ** 2, x[0, :32] ** 2 + x[0, 32:] ** 2, rtol=1e-5)
+    z = (x[0, :32] + 1j * x[0, 32:]) * np.exp(1j * np.arange(5, 6) * (1.0 / 150000.0 ** (np.arange(0, 64, 2) / 64)))
+    np.testing.assert_allclose(r[0, :32], z.real, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r[0, 32:], z.imag, rtol=1e-4, atol=1e-5)
