@@ -1,0 +1,105 @@
+/*
+ * liblyra_hip - C ABI of the MI355X (gfx950) decode kernels.
+ *
+ * The reference (ibbyml/lyra) has no FFI: its plugin seam is two Python callables chosen in
+ * lyra/kernels/op.py:18-27.  Each entry point below names the reference callable it stands
+ * behind.  All pointers are device pointers unless stated otherwise; every call is
+ * asynchronous on `stream`, never synchronises, never allocates and keeps no state, so it is
+ * re-entrant from any host thread.  Return value: 0 on success, a negative LYRA_E_* code
+ * otherwise (nothing has been launched in that case).
+ */
+#ifndef LYRA_HIP_H
+#define LYRA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LYRA_ABI_VERSION 1
+
+/* element types of buffers that cross the ABI */
+#define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
+#define LYRA_DTYPE_E4M3FN 1 /* OCP FP8 E4M3 (finite, max 448), 1 byte; needs scales */
+#define LYRA_DTYPE_F32 2    /* float32 (outputs only) */
+
+#define LYRA_OK 0
+#define LYRA_E_BADARG (-1)      /* null pointer, non-positive size, N % K != 0 ... */
+#define LYRA_E_UNSUPPORTED (-2) /* a shape or dtype the kernels do not cover */
+#define LYRA_E_WORKSPACE (-3)   /* workspace pointer missing or too small */
+#define LYRA_E_LAUNCH (-4)      /* the HIP runtime refused the launch */
+
+typedef void* lyra_stream_t; /* a hipStream_t; NULL = the default stream */
+
+int lyra_abi_version(void);
+const char* lyra_strerror(int code);
+
+/*
+ * Decode attention: one query token per sequence against the KV cache.
+ * Stands behind lyra.kernels.decode_attention.decode_attention
+ * (lyra/kernels/decode_attention.py:364-415; maths of decode_attention_reference :311-361
+ * and sliding_decode :263-308).
+ *
+ *   q        [B,N,H] bf16                      (the reference's [B,N,1,H])
+ *   k, v     [B,K,S,H] bf16 or e4m3fn, contiguous; kv head of query head n is n / (N/K)
+ *   k_scale, v_scale   [B,K,S] float32, one per cached token and kv head (QArray block (1,H),
+ *            lyra/model.py:225); NULL iff kv_dtype == LYRA_DTYPE_BF16
+ *   sinks    [N] float32 learned sink logits (a virtual key with value 0)
+ *   position int32; element b*position_stride is the index of the newest token of row b; keys
+ *            0..position are visible (minus the window).  position_stride 0 = one scalar for the
+ *            whole batch (the reference's only mode), 1 = ragged batch.
+ *   gate     [B,N] bf16 or NULL; out = bf16(bf16(attn) * gate)  (lyra/model.py:343-347)
+ *   out      [B,N,H] out_dtype (bf16 or float32)
+ *   sliding_window  0 = global layer; w > 0 = only keys j with position-w < j <= position
+ *   sm_scale        multiplies q.k (the reference passes H**-0.5)
+ *   workspace       at least lyra_decode_attention_workspace(...) bytes, 256-byte aligned; holds
+ *                   split partials for the duration of the call only
+ * Supported: H in {64,128}; 1 <= N/K <= 16; any B, S >= 1.
+ */
+int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                          const float* sinks, const int32_t* position, int position_stride, const void* gate,
+                          void* out, void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
+                          float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream);
+
+size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sliding_window);
+
+/*
+ * Decode grouped matmul: out[r,:] = epilogue(lhs[r,:] @ rhs[e(r)]) with rows sorted by group.
+ * Stands behind lyra.kernels.decode_gemm.decode_gemm (lyra/kernels/decode_gemm.py:404-474;
+ * maths of grouped_gemm_reference, lyra/kernels/gemm.py:1575-1617) and, with G == 1, behind
+ * lyra.nn.quant.dot for the dense projections (lyra/nn/quant.py:106-108).
+ *
+ *   lhs         [M,K] bf16
+ *   rhs         [G,K,N] bf16 or e4m3fn, contiguous
+ *   rhs_scale   [G,K/bk,N/bn] float32 block scales (QArray block (bk,bn)); NULL iff rhs is bf16.
+ *               bk == K, bn == 1 is the per-output-channel layout.
+ *   group_sizes [G] int32 on the device; rows of group g are [sum(sizes[:g]), +sizes[g]).
+ *               Experts with no rows are never read.  Rows at or beyond sum(sizes) produce
+ *               epilogue(0) with the bias of group G-1 (lax.ragged_dot + gemm.py:450-456).
+ *   bias        [G,N] float32 or NULL, added in float32 before SwiGLU
+ *   fused_swiglu  out[:, j] = (clip(t[:, N/2+j], +-limit) + 1) * g * sigmoid(beta*g),
+ *               g = min(t[:, j], limit)  (lyra/kernels/common.py:98-114); out is then [M,N/2]
+ *   out         [M,N] or [M,N/2], out_dtype (bf16 or float32)
+ *   workspace   at least lyra_decode_gemm_workspace(...) bytes, 256-byte aligned
+ * Supported: K % 32 == 0, N % 128 == 0 (N % 256 == 0 with fused_swiglu), fp8 blocks with
+ * bk % 32 == 0 or bk == K, and bn % 128 == 0 or bn == 1.
+ */
+int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
+                     const int32_t* group_sizes, const float* bias, void* out, void* workspace,
+                     size_t workspace_bytes, int M, int G, int K, int N, int rhs_dtype, int out_dtype,
+                     int fused_swiglu, float swiglu_beta, float swiglu_limit, lyra_stream_t stream);
+
+size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu);
+
+/*
+ * Self-check of the matrix-core register layouts and FP8 conversions the kernels rely on.
+ * `report` (device, >= 8 int32) receives mismatch counts; all zeros = pass.  Test hook only.
+ */
+int lyra_selftest(int32_t* report, lyra_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LYRA_HIP_H */

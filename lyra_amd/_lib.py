@@ -1,0 +1,71 @@
+"""ctypes binding of liblyra_hip.so.  There is no fallback: a missing library is an error."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
+
+DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
+ABI_VERSION = 1
+
+_c = ctypes
+SIGNATURES = {
+    "lyra_abi_version": (_c.c_int, []),
+    "lyra_strerror": (_c.c_char_p, [_c.c_int]),
+    "lyra_decode_attention": (
+        _c.c_int,
+        [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
+    "lyra_decode_attention_workspace": (_c.c_size_t, [_c.c_int] * 6),
+    "lyra_decode_gemm": (
+        _c.c_int,
+        [_c.c_void_p] * 3 + [_c.c_int] * 2 + [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 7 + [_c.c_float] * 2 + [_c.c_void_p],
+    ),
+    "lyra_decode_gemm_workspace": (_c.c_size_t, [_c.c_int] * 5),
+    "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
+}
+
+
+class LyraHipError(RuntimeError):
+    pass
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise LyraHipError(
+            f"{LIB_PATH} is missing: build it with `python -m lyra_amd.build` (hipcc, gfx950). "
+            "lyra_amd has no non-HIP code path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here means a stale library
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.lyra_abi_version() != ABI_VERSION:
+        raise LyraHipError(f"liblyra_hip.so has ABI {lib.lyra_abi_version()}, bindings expect {ABI_VERSION}: rebuild it")
+    return lib
+
+
+lib = _load()
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        raise LyraHipError(f"{what}: {lib.lyra_strerror(code).decode()} ({code})")
+
+
+_WORKSPACES: dict[tuple[int, int], "object"] = {}
+
+
+def workspace(device, stream_ptr: int, nbytes: int):
+    """A reusable device scratch buffer per (device, stream); grows, never shrinks."""
+    import torch
+
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    buf = _WORKSPACES.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = buf
+    return buf

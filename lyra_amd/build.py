@@ -1,0 +1,37 @@
+"""Builds liblyra_hip.so (the gfx950 decode kernels + C ABI) in-tree with hipcc."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
+SOURCES = ("abi.hip", "decode_attention.hip", "decode_gemm.hip")
+HIPCC_FLAGS = (
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # keep the compiler from forming packed-FP32 VALU instructions out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+)
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, *(os.path.join(CSRC, s) for s in SOURCES), "-o", LIB_PATH]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"  # host pass does not know the device feature
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,117 @@
+// ABI housekeeping and a device self-check of the hardware behaviours the kernels assume.
+#include "lyra_device.h"
+
+namespace lyra {
+
+// e4m3fn code -> float by the format's definition (s.eeee.mmm, bias 7, no infinities)
+__device__ float e4m3fn_by_definition(int code) {
+    const float sign = (code & 0x80) ? -1.f : 1.f;
+    const int e = (code >> 3) & 0xF, m = code & 7;
+    if (e == 0xF && m == 7) return __builtin_nanf("");
+    if (e == 0) return sign * ldexpf((float)m / 8.f, -6);
+    return sign * ldexpf(1.f + (float)m / 8.f, e - 7);
+}
+
+__global__ __launch_bounds__(64) void selftest_kernel(int32_t* report) {
+    const int lane = threadIdx.x;
+    const int x = lane & 15, kb = lane >> 4;
+    int bad_mfma = 0, bad_cvt = 0, bad_cvt_bf16 = 0, bad_pack = 0, bad_perm = 0, bad_denorm = 0;
+
+    // [0] accumulator layout of the 16x16x32 bf16 tile: A[i][k] = (i+1) if k == 0 else 0,
+    //     B[k][j] = (j+1) if k == 0 else 0  ->  D[i][j] = (i+1)(j+1); slot 0 of k-group 0 plays k == 0.
+    {
+        Pack8 a, b;
+        for (int i = 0; i < 4; ++i) a.u[i] = b.u[i] = 0u;
+        if (kb == 0) {
+            a.u[0] = pack_bf16((float)(x + 1), 0.f);
+            b.u[0] = pack_bf16((float)(x + 1), 0.f);
+        }
+        f32x4 d = mfma_16x16x32(a.v, b.v, f32x4{0.f, 0.f, 0.f, 0.f});
+        for (int r = 0; r < 4; ++r) bad_mfma += d[r] != (float)((4 * kb + r + 1) * (x + 1));
+    }
+    // [1] every k slot contributes once, with the same slot pairing in A and B:
+    //     A[i][slot] = 1, B[slot][j] = w(slot) distinct powers of two -> D = sum of all w
+    {
+        Pack8 a, b;
+        float want = 0.f;
+        for (int g = 0; g < 4; ++g)
+            for (int i = 0; i < 8; ++i) want += ldexpf(1.f, (8 * g + i) % 8 - 3) * (float)(g + 1);
+        for (int i = 0; i < 4; ++i) {
+            a.u[i] = pack_bf16(1.f, 1.f);
+            b.u[i] = pack_bf16(ldexpf(1.f, (2 * i) % 8 - 3) * (float)(kb + 1), ldexpf(1.f, (2 * i + 1) % 8 - 3) * (float)(kb + 1));
+        }
+        f32x4 d = mfma_16x16x32(a.v, b.v, f32x4{0.f, 0.f, 0.f, 0.f});
+        for (int r = 0; r < 4; ++r) bad_mfma += d[r] != want;
+    }
+    // [2] FP8 conversions over all 256 codes (4 per lane), both halves of the dword
+    for (int q = 0; q < 4; ++q) {
+        const int c0 = lane * 4 + q;
+        const uint32_t w = (uint32_t)c0 | ((uint32_t)(255 - c0) << 8) | ((uint32_t)c0 << 16) | ((uint32_t)(255 - c0) << 24);
+        const float e0 = e4m3fn_by_definition(c0), e1 = e4m3fn_by_definition(255 - c0);
+        const f32x2 lo = fp8x2_to_f32(w, false), hi = fp8x2_to_f32(w, true);
+        auto same = [](float a, float b) { return (a != a && b != b) || __float_as_uint(a) == __float_as_uint(b); };
+        bad_cvt += !same(lo[0], e0) + !same(lo[1], e1) + !same(hi[0], e0) + !same(hi[1], e1);
+        const uint32_t blo = fp8x2_to_bf16x2(w, false), bhi = fp8x2_to_bf16x2(w, true);
+        auto bf = [](uint32_t v, int h) { return __uint_as_float((h ? (v >> 16) : (v & 0xFFFFu)) << 16); };
+        bad_cvt_bf16 += !same(bf(blo, 0), e0) + !same(bf(blo, 1), e1) + !same(bf(bhi, 0), e0) + !same(bf(bhi, 1), e1);
+    }
+    // [3] float32 -> bf16 packing rounds to nearest even
+    {
+        const float v[4] = {1.00390625f, 1.01171875f, -3.0e-3f * (lane + 1), 65504.f + lane};
+        for (int i = 0; i < 4; ++i) {
+            uint32_t u = __float_as_uint(v[i]);
+            const uint32_t want = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+            bad_pack += (pack_bf16(v[i], 0.f) & 0xFFFFu) != want;
+            bad_pack += (pack_bf16(0.f, v[i]) >> 16) != want;
+        }
+    }
+    // [4] half-word interleave used for bf16 operands
+    {
+        const uint32_t a = 0x11002200u + lane, b = 0x33004400u + lane;
+        bad_perm += __builtin_amdgcn_perm(b, a, 0x05040100u) != ((b << 16) | (a & 0xFFFFu));
+        bad_perm += __builtin_amdgcn_perm(b, a, 0x07060302u) != ((b & 0xFFFF0000u) | (a >> 16));
+    }
+    // [5] the smallest FP8 subnormal (2^-9, exact in bf16) survives the matrix core unflushed
+    {
+        Pack8 a, b;
+        for (int i = 0; i < 4; ++i) a.u[i] = b.u[i] = 0u;
+        if (kb == 0) {
+            a.u[0] = fp8x2_to_bf16x2(0x01u, false);
+            b.u[0] = pack_bf16(1.f, 0.f);
+        }
+        f32x4 d = mfma_16x16x32(a.v, b.v, f32x4{0.f, 0.f, 0.f, 0.f});
+        for (int r = 0; r < 4; ++r) bad_denorm += d[r] != ldexpf(1.f, -9);
+    }
+
+    int vals[6] = {bad_mfma, bad_cvt, bad_cvt_bf16, bad_pack, bad_perm, bad_denorm};
+    for (int i = 0; i < 6; ++i) {
+        int v = vals[i];
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+        if (lane == 0) report[i] = v;
+    }
+    if (lane == 0) {
+        report[6] = 0;
+        report[7] = LYRA_ABI_VERSION;
+    }
+}
+
+}  // namespace lyra
+
+extern "C" int lyra_abi_version(void) { return LYRA_ABI_VERSION; }
+
+extern "C" const char* lyra_strerror(int code) {
+    switch (code) {
+        case LYRA_OK: return "ok";
+        case LYRA_E_BADARG: return "bad argument (null pointer, non-positive size, inconsistent dtype/scale)";
+        case LYRA_E_UNSUPPORTED: return "shape or dtype not supported by the gfx950 kernels";
+        case LYRA_E_WORKSPACE: return "workspace missing, misaligned or too small";
+        case LYRA_E_LAUNCH: return "HIP runtime refused the kernel launch";
+        default: return "unknown lyra error code";
+    }
+}
+
+extern "C" int lyra_selftest(int32_t* report, lyra_stream_t stream) {
+    if (!report) return LYRA_E_BADARG;
+    hipLaunchKernelGGL(lyra::selftest_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, report);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}

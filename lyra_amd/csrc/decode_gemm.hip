@@ -1,0 +1,432 @@
+// Decode grouped matmul for gfx950: out[r,:] = epilogue(lhs[r,:] @ rhs[expert(r)]) for a handful of
+// rows per expert, weights BF16 or block-scaled FP8 (e4m3fn), optional bias and fused SwiGLU.
+//
+// Maths (lyra/kernels/gemm.py:1575-1617 as called from lyra/kernels/decode_gemm.py:390-399):
+//   t = ragged_dot(lhs, W^, group_sizes) in float32;  t += bias[expert];  t = swiglu(t);  cast
+// with W^ = f32(Wq) * scale[k/bk, n/bn].  The kernel streams every weight byte of a touched expert
+// exactly once (experts with no rows are never read), multiplies raw FP8 values converted exactly
+// to BF16 on the matrix cores and applies the block scales to the float32 accumulators.
+//
+// Mapping: the weight matrix is row-major [K,N] (N contiguous).  A wavefront owns 128 output columns
+// (64 gate + 64 linear columns when SwiGLU is fused) and walks K in steps of 32 rows.  Lane
+// (x = lane & 15, kb = lane >> 4) reads 8 consecutive columns of the 8 rows 8*kb .. 8*kb+7; pairing two
+// rows in the bf16 pack step yields the K-major B operand, so the transposition costs nothing.
+//   D[16 rows, 16 cols] += X[16 rows x 32 k] . W[32 k x 16 cols]   for each of the 8 column phases.
+#include <algorithm>
+
+#include "lyra_device.h"
+
+namespace lyra {
+
+struct GemmParams {
+    const uint16_t* lhs;
+    const uint8_t* rhs;
+    const float* scale;
+    const int32_t* group_sizes;
+    const float* bias;
+    void* out;
+    float* part;  // [ksplit, M, N] float32 partial products when ksplit > 1
+    int M, G, K, N;
+    int bk, bn, KB, NB;
+    int scale_mode;  // 0 none, 1 one scale per lane and k-block (bn % 8 == 0), 2 per column (bk == K)
+    int out_f32, swiglu;
+    float beta, limit;
+    int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
+};
+
+__device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, float limit) {
+    glu = fminf(glu, limit);
+    lin = fminf(fmaxf(lin, -limit), limit);
+    const float sig = 1.0f / (1.0f + fast_exp2(-beta * kLog2e * glu));
+    return (lin + 1.0f) * (glu * sig);
+}
+
+template <bool FP8, int MT>
+struct RawStep {
+    static constexpr int WW = FP8 ? 2 : 4;  // dwords per lane per weight row (8 columns)
+    uint32_t w[8][WW];
+    u32x4 x[MT];
+};
+
+template <bool FP8, int MT>
+__device__ __forceinline__ void load_step(RawStep<FP8, MT>& s, const uint8_t* wlane, size_t row_bytes,
+                                          const uint16_t* xlane, size_t x_stride, int kk, int n_mt,
+                                          const bool (&row_ok)[MT]) {
+    constexpr int WW = RawStep<FP8, MT>::WW;
+    const uint8_t* wp = wlane + (size_t)kk * row_bytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if constexpr (WW == 2) {
+            u32x2 d = *(const u32x2*)(wp + (size_t)i * row_bytes);
+            s.w[i][0] = d[0];
+            s.w[i][1] = d[1];
+        } else {
+            u32x4 d = *(const u32x4*)(wp + (size_t)i * row_bytes);
+            s.w[i][0] = d[0];
+            s.w[i][1] = d[1];
+            s.w[i][2] = d[2];
+            s.w[i][3] = d[3];
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        u32x4 d = u32x4{0u, 0u, 0u, 0u};
+        if (mt < n_mt && row_ok[mt]) d = *(const u32x4*)(xlane + (size_t)mt * 16 * x_stride + kk);
+        s.x[mt] = d;
+    }
+}
+
+template <bool FP8, int MT>
+__device__ __forceinline__ void compute_step(const RawStep<FP8, MT>& s, int n_mt, f32x4 (&acc)[MT][8]) {
+#pragma unroll
+    for (int c = 0; c < 8; c += 2) {
+        Pack8 b0, b1;
+        if constexpr (FP8) {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                const f32x2 fa = fp8x2_to_f32(s.w[i][c >> 2], (c & 2) != 0);
+                const f32x2 fb = fp8x2_to_f32(s.w[i + 1][c >> 2], (c & 2) != 0);
+                b0.u[i >> 1] = pack_bf16(fa[0], fb[0]);
+                b1.u[i >> 1] = pack_bf16(fa[1], fb[1]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                const uint32_t a = s.w[i][c >> 1], b = s.w[i + 1][c >> 1];
+                b0.u[i >> 1] = __builtin_amdgcn_perm(b, a, 0x05040100u);
+                b1.u[i >> 1] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt < n_mt) {
+                const bf16x8 xa = __builtin_bit_cast(bf16x8, s.x[mt]);
+                acc[mt][c] = mfma_16x16x32(xa, b0.v, acc[mt][c]);
+                acc[mt][c + 1] = mfma_16x16x32(xa, b1.v, acc[mt][c + 1]);
+            }
+        }
+    }
+}
+
+// Writes 8 consecutive result columns of one row: fused epilogue (ksplit == 1) or float32 partials.
+// Must be called by all lanes of the wavefront (SwiGLU exchanges gate and linear halves by shuffle);
+// `store` says whether this lane's row exists.
+__device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], int g, int row, int ncol, int out_col,
+                                           int ks, bool store, bool is_lin_lane) {
+    if (p.ksplit > 1) {
+        if (store) {
+            float* dst = p.part + ((size_t)ks * p.M + row) * p.N + ncol;
+            *(f32x4*)dst = f32x4{t[0], t[1], t[2], t[3]};
+            *(f32x4*)(dst + 4) = f32x4{t[4], t[5], t[6], t[7]};
+        }
+        return;
+    }
+    if (p.bias) {
+        const float* bp = p.bias + (size_t)g * p.N + ncol;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) t[c] += bp[c];
+    }
+    int NO = p.N;
+    if (p.swiglu) {
+        NO = p.N / 2;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float other = __shfl_xor(t[c], 8, kWave);  // gate lanes x<8 pair with linear lanes x+8
+            t[c] = swiglu_one(t[c], other, p.beta, p.limit);
+        }
+        store = store && !is_lin_lane;
+    }
+    if (store) {
+        if (p.out_f32) {
+            float* dst = (float*)p.out + (size_t)row * NO + out_col;
+            *(f32x4*)dst = f32x4{t[0], t[1], t[2], t[3]};
+            *(f32x4*)(dst + 4) = f32x4{t[4], t[5], t[6], t[7]};
+        } else {
+            u32x4 d;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) d[c] = pack_bf16(t[2 * c], t[2 * c + 1]);
+            *(u32x4*)((uint16_t*)p.out + (size_t)row * NO + out_col) = d;
+        }
+    }
+}
+
+template <bool FP8, int MT>
+__global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
+    constexpr int ES = FP8 ? 1 : 2;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int x = lane & 15, kb = lane >> 4;
+    const int g = blockIdx.z, ks = blockIdx.y;
+    const int span = blockIdx.x * waves + wave;  // which 128-column span this wavefront owns
+
+    // rows of this group: [off, off + cnt)
+    int part_sum = 0;
+    for (int i = lane; i < g; i += 64) part_sum += p.group_sizes[i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) part_sum += __shfl_xor(part_sum, o, kWave);
+    const int off = min(part_sum, p.M);
+    const int cnt = min(p.group_sizes[g], p.M - off);
+    const int pad_from = (g == p.G - 1 && p.ksplit == 1 && ks == 0) ? off + cnt : p.M;  // rows past the last group
+    if (cnt <= 0 && pad_from >= p.M) return;
+
+    // columns of this lane
+    int ncol, out_col;
+    bool span_ok;
+    const bool is_lin_lane = p.swiglu && x >= 8;
+    if (p.swiglu) {
+        const int half = p.N >> 1;
+        span_ok = span * 64 < half;
+        out_col = span * 64 + 8 * (x & 7);
+        ncol = is_lin_lane ? half + out_col : out_col;
+    } else {
+        span_ok = span * 128 < p.N;
+        ncol = out_col = span * 128 + 8 * x;
+    }
+    if (!span_ok) return;
+
+    const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
+    const size_t row_bytes = (size_t)p.N * ES;
+    const uint8_t* wlane = p.rhs + ((size_t)g * p.K + 8 * kb) * row_bytes + (size_t)ncol * ES;
+    const float* sc_lane = nullptr;
+    if (FP8 && p.scale_mode == 1) sc_lane = p.scale + (size_t)g * p.KB * p.NB + ncol / p.bn;
+
+    for (int rb = 0; rb < cnt; rb += 16 * MT) {
+        const int rowbase = off + rb;
+        const int rows_here = min(16 * MT, cnt - rb);
+        const int n_mt = (rows_here + 15) >> 4;
+        bool row_ok[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) row_ok[mt] = mt * 16 + x < rows_here;
+        const uint16_t* xlane = p.lhs + (size_t)(rowbase + x) * p.K + 8 * kb;
+
+        f32x4 acc[MT][8];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // accumulators are kept in units of the current block scale; on a k-block boundary they are
+        // re-expressed in the next block's unit, and the last unit is applied at the end
+        float s_cur = 1.f, s_next = 1.f;
+        if (FP8 && p.scale_mode == 1) {
+            s_cur = sc_lane[(size_t)(k0 / p.bk) * p.NB];
+            s_next = s_cur;
+        }
+
+        RawStep<FP8, MT> cur, nxt;
+        if (k0 < k1) load_step<FP8, MT>(cur, wlane, row_bytes, xlane, p.K, k0, n_mt, row_ok);
+        for (int kk = k0; kk < k1; kk += 32) {
+            const bool more = kk + 32 < k1;
+            if (more) load_step<FP8, MT>(nxt, wlane, row_bytes, xlane, p.K, kk + 32, n_mt, row_ok);
+            if (FP8 && p.scale_mode == 1 && p.bk < p.K) {
+                if (kk % p.bk == 0) {
+                    if (kk != k0) {
+                        const float ratio = s_cur / s_next;
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            if (mt < n_mt)
+#pragma unroll
+                                for (int c = 0; c < 8; ++c) {
+                                    acc[mt][c][0] *= ratio;
+                                    acc[mt][c][1] *= ratio;
+                                    acc[mt][c][2] *= ratio;
+                                    acc[mt][c][3] *= ratio;
+                                }
+                        s_cur = s_next;
+                    }
+                    const int nb = kk / p.bk + 1;  // prefetch the following block's scale
+                    if (nb * p.bk < k1) s_next = sc_lane[(size_t)nb * p.NB];
+                }
+            }
+            compute_step<FP8, MT>(cur, n_mt, acc);
+            if (more) cur = nxt;
+        }
+
+        float colscale[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = s_cur;
+        if (FP8 && p.scale_mode == 2) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)g * p.NB + (ncol + c) / p.bn];
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt < n_mt) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int lr = mt * 16 + 4 * kb + r;
+                    float t[8];
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) t[c] = acc[mt][c][r] * colscale[c];
+                    finish_row(p, t, g, rowbase + lr, ncol, out_col, ks, lr < rows_here, is_lin_lane);
+                }
+            }
+        }
+    }
+
+    // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
+    for (int row0 = pad_from; row0 < p.M; row0 += 4) {
+        float t[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) t[c] = 0.f;
+        finish_row(p, t, g, row0 + kb, ncol, out_col, ks, row0 + kb < p.M, is_lin_lane);
+    }
+}
+
+// Second pass when K was split across workgroups: sum the partials, then bias / SwiGLU / cast.
+// One thread per 4 output columns.
+__global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
+    const int NO = p.swiglu ? p.N / 2 : p.N;
+    const int quads = NO / 4;
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)p.M * quads) return;
+    const int row = (int)(idx / quads), col = (int)(idx - (long)row * quads) * 4;
+    int total = 0, g = p.G - 1;
+    for (int i = 0; i < p.G; ++i) {
+        const int nt = total + p.group_sizes[i];
+        if (row >= total && row < nt) g = i;
+        total = nt;
+    }
+    const bool live = row < total;
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        for (int s = 0; s < p.ksplit; ++s) {
+            const float* src = p.part + ((size_t)s * p.M + row) * p.N;
+            const f32x4 va = *(const f32x4*)(src + col);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a[c] += va[c];
+            if (p.swiglu) {
+                const f32x4 vb = *(const f32x4*)(src + NO + col);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) b[c] += vb[c];
+            }
+        }
+    }
+    if (p.bias) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            a[c] += p.bias[(size_t)g * p.N + col + c];
+            if (p.swiglu) b[c] += p.bias[(size_t)g * p.N + NO + col + c];
+        }
+    }
+    if (p.swiglu) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] = swiglu_one(a[c], b[c], p.beta, p.limit);
+    }
+    if (p.out_f32) {
+        *(f32x4*)((float*)p.out + (size_t)row * NO + col) = f32x4{a[0], a[1], a[2], a[3]};
+    } else {
+        u32x2 d;
+        d[0] = pack_bf16(a[0], a[1]);
+        d[1] = pack_bf16(a[2], a[3]);
+        *(u32x2*)((uint16_t*)p.out + (size_t)row * NO + col) = d;
+    }
+}
+
+struct GemmPlan {
+    int mt;      // 16-row tiles held in registers per pass
+    int waves;   // wavefronts per workgroup
+    int spans;   // 128-column spans (64+64 with SwiGLU)
+    int ksplit, kpart;
+};
+
+// Shape-only plan (group sizes live on the device): enough workgroups to fill 256 compute units,
+// splitting K when the column spans of the touched experts alone are too few.
+static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) {
+    GemmPlan pl;
+    pl.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
+    const int touched = std::max(1, std::min(G, M));
+    const long waves_noksplit = (long)pl.spans * touched;
+    const long target_waves = 256L * 8;
+    int unit = 32;
+    if (bk > 0 && bk < K) unit = bk;  // splits start on a scale-block boundary
+    const int max_split = std::max(1, K / std::max(unit, 256));
+    int ksplit = (int)std::min((long)max_split, std::max(1L, target_waves / std::max(1L, waves_noksplit)));
+    int kpart = (K + ksplit - 1) / ksplit;
+    kpart = (kpart + unit - 1) / unit * unit;
+    ksplit = (K + kpart - 1) / kpart;
+    pl.ksplit = ksplit;
+    pl.kpart = kpart;
+    pl.waves = pl.spans % 4 == 0 ? 4 : (pl.spans % 2 == 0 ? 2 : 1);
+    if ((long)pl.spans / pl.waves * touched * ksplit < 256) pl.waves = 1;
+    return pl;
+}
+
+}  // namespace lyra
+
+extern "C" size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu) {
+    if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return 0;
+    // the split factor may depend on the scale block; size for the largest split the plan can choose
+    const lyra::GemmPlan pl = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu);
+    if (pl.ksplit == 1) return 256;
+    return ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+}
+
+extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
+                                const int32_t* group_sizes, const float* bias, void* out, void* workspace,
+                                size_t workspace_bytes, int M, int G, int K, int N, int rhs_dtype, int out_dtype,
+                                int fused_swiglu, float swiglu_beta, float swiglu_limit, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!lhs || !rhs || !group_sizes || !out) return LYRA_E_BADARG;
+    if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
+    const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
+    if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
+    if (K % 32 || N % 128 || (fused_swiglu && N % 256) || G > 65535) return LYRA_E_UNSUPPORTED;
+
+    GemmParams p;
+    p.scale_mode = 0;
+    p.bk = p.bn = 1;
+    p.KB = p.NB = 1;
+    if (fp8) {
+        if (bk <= 0 || bn <= 0 || K % bk || N % bn) return LYRA_E_BADARG;
+        p.bk = bk; p.bn = bn; p.KB = K / bk; p.NB = N / bn;
+        if (bn % 8 == 0 && (bk % 32 == 0 || bk == K)) p.scale_mode = 1;
+        else if (bk == K) p.scale_mode = 2;
+        else return LYRA_E_UNSUPPORTED;
+    }
+    const GemmPlan pl = plan_gemm(M, G, K, N, fp8 ? bk : 0, fused_swiglu);
+    p.lhs = (const uint16_t*)lhs;
+    p.rhs = (const uint8_t*)rhs;
+    p.scale = rhs_scale;
+    p.group_sizes = group_sizes;
+    p.bias = bias;
+    p.out = out;
+    p.part = nullptr;
+    p.M = M; p.G = G; p.K = K; p.N = N;
+    p.out_f32 = out_dtype == LYRA_DTYPE_F32;
+    p.swiglu = fused_swiglu != 0;
+    p.beta = swiglu_beta;
+    p.limit = swiglu_limit;
+    p.ksplit = pl.ksplit;
+    p.kpart = pl.kpart;
+    if (pl.ksplit > 1) {
+        const size_t need = ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+        if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
+        p.part = (float*)workspace;
+    }
+
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((pl.spans + pl.waves - 1) / pl.waves, pl.ksplit, G), block(pl.waves * 64);
+#define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, 0, st, p)
+    if (fp8) {
+        if (pl.mt == 1) LYRA_LAUNCH_GEMM(true, 1);
+        else if (pl.mt == 2) LYRA_LAUNCH_GEMM(true, 2);
+        else LYRA_LAUNCH_GEMM(true, 4);
+    } else {
+        if (pl.mt == 1) LYRA_LAUNCH_GEMM(false, 1);
+        else if (pl.mt == 2) LYRA_LAUNCH_GEMM(false, 2);
+        else LYRA_LAUNCH_GEMM(false, 4);
+    }
+#undef LYRA_LAUNCH_GEMM
+    if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
+    if (pl.ksplit > 1) {
+        const int NO = fused_swiglu ? N / 2 : N;
+        const long threads = (long)M * (NO / 4);
+        const dim3 fgrid((unsigned)((threads + 255) / 256)), fblock(256);
+        hipLaunchKernelGGL(decode_gemm_finish_kernel, fgrid, fblock, 0, st, p);
+        if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
+    }
+    return LYRA_OK;
+}

@@ -1,0 +1,98 @@
+// Device-side helpers shared by the gfx950 decode kernels: vector types, FP8/BF16 conversions,
+// the 16x16x32 BF16 matrix-core tile and wavefront (64-lane) reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lyra_hip.h"
+
+namespace lyra {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// D(16x16,f32) += A(16x32,bf16) * B(32x16,bf16).  Lane l supplies row (l & 15) of A and column
+// (l & 15) of B, each as the 8 consecutive k-slots of k-group (l >> 4); both operands use the same
+// slot -> k mapping, so only "same k in the same slot" matters.  Lane l receives D[4*(l>>4)+r][l&15]
+// in element r of the result.
+__device__ __forceinline__ f32x4 mfma_16x16x32(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+union Pack8 {
+    bf16x8 v;
+    uint32_t u[4];
+    bf16x2 h[4];
+};
+
+// two e4m3fn codes (low or high half of a dword) -> two float32, exact
+__device__ __forceinline__ f32x2 fp8x2_to_f32(uint32_t w, bool hi) {
+    return hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+}
+
+// two float32 -> packed bf16x2 (round to nearest even), one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    bf16x2 r;
+    r[0] = (__bf16)lo;
+    r[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// two e4m3fn codes -> packed bf16x2 in one instruction (the conversion is exact; scale 1)
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+    bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// 8 consecutive e4m3fn codes (two dwords) -> bf16x8 in the same order
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
+    Pack8 p;
+    p.u[0] = fp8x2_to_bf16x2(w0, false);
+    p.u[1] = fp8x2_to_bf16x2(w0, true);
+    p.u[2] = fp8x2_to_bf16x2(w1, false);
+    p.u[3] = fp8x2_to_bf16x2(w1, true);
+    return p.v;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    __bf16 h = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// butterfly over the four 16-lane groups of a wavefront (lanes l, l^16, l^32, l^48)
+__device__ __forceinline__ float group4_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16, kWave));
+    x = fmaxf(x, __shfl_xor(x, 32, kWave));
+    return x;
+}
+__device__ __forceinline__ float group4_sum(float x) {
+    x += __shfl_xor(x, 16, kWave);
+    x += __shfl_xor(x, 32, kWave);
+    return x;
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, kWave));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, kWave);
+    return x;
+}
+
+}  // namespace lyra

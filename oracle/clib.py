@@ -28,6 +28,8 @@ def load() -> ctypes.CDLL:
     lib.lyra_oracle_f32_to_bf16.argtypes = [c.c_float]
     lib.lyra_oracle_quantize_rows.restype = None
     lib.lyra_oracle_quantize_rows.argtypes = [c.c_void_p, c.c_int64, c.c_int, c.c_void_p, c.c_void_p]
+    lib.lyra_oracle_quantize_blocks.restype = c.c_int
+    lib.lyra_oracle_quantize_blocks.argtypes = [c.c_void_p] + [c.c_int] * 5 + [c.c_void_p] * 2
     for name in ("lyra_oracle_decode_window",):
         getattr(lib, name).restype = c.c_int
         getattr(lib, name).argtypes = [c.c_int]
@@ -48,6 +50,30 @@ def load() -> ctypes.CDLL:
 
 def _p(a):
     return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def quantize_rows(x: np.ndarray):
+    """Block (1,H) quantiser (KV cache); bit-identical to lyra_oracle.quantize(x, (1, H))."""
+    lib = load()
+    H = x.shape[-1]
+    flat = np.ascontiguousarray(x.reshape(-1, H), dtype=np.float32)
+    q = np.empty(flat.shape, dtype=np.uint8)
+    s = np.empty(flat.shape[0], dtype=np.float32)
+    lib.lyra_oracle_quantize_rows(_p(flat), flat.shape[0], H, _p(q), _p(s))
+    return q.reshape(x.shape), s.reshape(*x.shape[:-1], 1)
+
+
+def quantize_blocks(w: np.ndarray, block):
+    """Block (bk,bn) quantiser of [G,K,N] weights; bit-identical to lyra_oracle.quantize(w, block)."""
+    lib = load()
+    G, K, N = w.shape
+    bk, bn = block
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    q = np.empty(w.shape, dtype=np.uint8)
+    s = np.empty((G, K // bk, N // bn), dtype=np.float32)
+    if lib.lyra_oracle_quantize_blocks(_p(w), G, K, N, bk, bn, _p(q), _p(s)):
+        raise ValueError(f"block {block} does not divide {(K, N)}")
+    return q, s
 
 
 def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_scale, sliding_window, *, ref_rounding=False):

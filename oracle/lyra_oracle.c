@@ -94,6 +94,7 @@ uint16_t lyra_oracle_f32_to_bf16(float f) { return f32_to_bf16(f); }
 /* ---- quantise one block-row (KV cache block (1,H)): quant.py:68-72 ------------------ */
 void lyra_oracle_quantize_rows(const float* x, int64_t rows, int H, uint8_t* qval, float* scale) {
     fp8_init();
+#pragma omp parallel for schedule(static)
     for (int64_t r = 0; r < rows; ++r) {
         const float* xr = x + r * H;
         float amax = 0.0f;
@@ -107,6 +108,34 @@ void lyra_oracle_quantize_rows(const float* x, int64_t rows, int H, uint8_t* qva
             qval[r * H + h] = lyra_oracle_f32_to_fp8_e4m3fn(t);
         }
     }
+}
+
+/* ---- quantise [G,K,N] weights with block (bk,bn): quant.py:48-75; scale is [G,K/bk,N/bn] ------- */
+int lyra_oracle_quantize_blocks(const float* x, int G, int K, int N, int bk, int bn, uint8_t* qval, float* scale) {
+    if (G <= 0 || K <= 0 || N <= 0 || bk <= 0 || bn <= 0 || K % bk || N % bn) return -1;
+    fp8_init();
+    const int KB = K / bk, NB = N / bn;
+#pragma omp parallel for collapse(3) schedule(static)
+    for (int g = 0; g < G; ++g) {
+        for (int kb = 0; kb < KB; ++kb) {
+            for (int nb = 0; nb < NB; ++nb) {
+                const size_t base = ((size_t)g * K + (size_t)kb * bk) * N + (size_t)nb * bn;
+                float amax = 0.0f;
+                for (int i = 0; i < bk; ++i)
+                    for (int j = 0; j < bn; ++j) amax = fmaxf(amax, fabsf(x[base + (size_t)i * N + j]));
+                const float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+                const float inv = 1.0f / s;
+                scale[((size_t)g * KB + kb) * NB + nb] = s;
+                for (int i = 0; i < bk; ++i)
+                    for (int j = 0; j < bn; ++j) {
+                        float t = x[base + (size_t)i * N + j] * inv;
+                        t = fminf(fmaxf(t, -448.0f), 448.0f);
+                        qval[base + (size_t)i * N + j] = lyra_oracle_f32_to_fp8_e4m3fn(t);
+                    }
+            }
+        }
+    }
+    return 0;
 }
 
 /* ---- window arithmetic: decode_attention.py:63-69, :277-280 -------------------------- */

@@ -111,10 +111,16 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
     """Round float32 to the nearest bfloat16 (ties to even); result kept as float32."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     bits = x.view(np.uint32)
-    lsb = (bits >> 16) & 1
-    rounded = (bits + np.uint32(0x7FFF) + lsb) & np.uint32(0xFFFF0000)
-    out = rounded.view(np.float32)
-    return np.where(np.isnan(x), x, out).astype(np.float32)
+    r = bits >> np.uint32(16)
+    r &= np.uint32(1)
+    r += np.uint32(0x7FFF)
+    r += bits
+    r &= np.uint32(0xFFFF0000)
+    out = r.view(np.float32)
+    nan = np.isnan(x)
+    if nan.any():
+        out[nan] = x[nan]
+    return out
 
 
 def bf16_bits(x: np.ndarray) -> np.ndarray:

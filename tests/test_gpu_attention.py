@@ -1,0 +1,228 @@
+"""GPU parity of the HIP decode-attention kernel (through the C ABI) against the CPU oracle.
+
+Tolerance: |got - want| <= 2e-2 + 1e-2*|want| against the fp32 oracle (tests/gpu_util.py); float32
+outputs are additionally held to 4e-3.  Index/mask behaviour is checked through outputs that differ
+by O(1) if a single key is wrongly included or dropped.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import clib
+from oracle import lyra_oracle as O
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(case, sm_scale, sw, pos, *, dtype=torch.bfloat16, gate=None, implementation="pallas"):
+    from lyra_amd.kernels.decode_attention import decode_attention
+
+    q, k, v, sinks = U.attention_torch_inputs(case)
+    p = pos if np.ndim(pos) == 0 else torch.from_numpy(np.asarray(pos, dtype=np.int32)).to(U.dev())
+    g = None if gate is None else U.t_bf16(gate)
+    out = decode_attention(q, k, v, sinks, sm_scale, sw, p, dtype=dtype, implementation=implementation, gate=g)
+    torch.cuda.synchronize()
+    return U.to_np(out)
+
+
+def _note(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def test_selftest_layouts_and_conversions():
+    from lyra_amd import _lib
+
+    rep = torch.full((8,), -1, dtype=torch.int32, device=U.dev())
+    _lib.check(_lib.lib.lyra_selftest(rep.data_ptr(), None), "lyra_selftest")
+    torch.cuda.synchronize()
+    r = rep.cpu().tolist()
+    assert r[:6] == [0, 0, 0, 0, 0, 0], f"mfma/cvt/cvt_bf16/pack/perm/denorm mismatches: {r}"
+    assert r[7] == 1
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("H,N,K", [(128, 16, 4), (64, 32, 4), (64, 64, 8), (128, 4, 4), (64, 16, 1)])
+@pytest.mark.parametrize("sw", [0, 128])
+def test_small_shapes_match_oracle(fp8, H, N, K, sw):
+    S = 512
+    case = U.attention_case(100 + H + N + K, 2, N, K, S, H, fp8=fp8)
+    for pos in (511, 130, 5):
+        _note(f"attn small fp8={fp8} H={H} N={N} K={K} sw={sw} pos={pos}")
+        want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, sw, pos)
+        got = _run(case, H**-0.5, sw, pos)
+        U.assert_close(got, want, what=f"pos={pos}")
+        got32 = _run(case, H**-0.5, sw, pos, dtype=torch.float32)
+        U.assert_close(got32, want, atol=4e-3, rtol=4e-3, what=f"f32 pos={pos}")
+
+
+def test_config1_lyra_small_bf16_global_with_gate():
+    """BASELINE config 1 at the variants.py shape (16Q/4KV/H=128) and at its literal 32Q/4KV/H=64."""
+    for (N, K, H) in ((16, 4, 128), (32, 4, 64)):
+        case = U.attention_case(1001, 1, N, K, 512, H, fp8=False)
+        rng = np.random.default_rng(7)
+        gate = O.bf16_round((2.0 / (1.0 + np.exp(-rng.standard_normal((1, N))))).astype(np.float32))
+        _note(f"attn cfg1 N={N} K={K} H={H}")
+        want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, 511, gate=gate)
+        got = _run(case, H**-0.5, 0, 511, gate=gate)
+        U.assert_close(got, want, what="cfg1")
+        # the kernel rounds like the JAX code: bf16(bf16(attn) * gate)
+        ref = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, 511, gate=gate, mode="ref")
+        assert np.abs(got - ref).max() <= 2e-2
+
+
+@pytest.mark.parametrize("S", [1, 3, 31, 33, 100, 257, 1000])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_odd_cache_lengths_and_every_boundary(S, fp8):
+    case = U.attention_case(200 + S, 1, 8, 2, S, 64, fp8=fp8)
+    for sw in (0, 1, 7, 128):
+        for pos in sorted({0, S // 2, S - 1, min(S - 1, 31), min(S - 1, 32)}):
+            _note(f"attn odd S={S} fp8={fp8} sw={sw} pos={pos}")
+            want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], 0.125, sw, pos)
+            got = _run(case, 0.125, sw, pos)
+            U.assert_close(got, want, what=f"S={S} sw={sw} pos={pos}")
+
+
+def test_window_mask_is_exact_one_key_at_a_time():
+    """A single huge-logit key just outside / inside the window flips the output by O(1)."""
+    B, N, K, S, H = 1, 4, 1, 640, 64
+    rng = np.random.default_rng(3)
+    q = np.zeros((B, N, 1, H), np.float32)
+    q[..., 0] = 8.0
+    k = np.zeros((B, K, S, H), np.float32)
+    v = O.bf16_round(rng.standard_normal((B, K, S, H)).astype(np.float32))
+    sinks = np.full(N, -30.0, np.float32)
+    for sw in (0, 128, 200):
+        for pos in (127, 128, 300, 639):
+            lo, hi = O.visible_range(pos, sw, S)
+            for spike in {lo - 1, lo, hi, hi + 1}:
+                if not 0 <= spike < S:
+                    continue
+                kk = k.copy()
+                kk[0, 0, spike, 0] = 16.0  # logit 128*sm_scale: dominates iff visible
+                case = {"q": q, "k": kk, "v": v, "sinks": sinks, "fp8": False}
+                _note(f"attn mask sw={sw} pos={pos} spike={spike}")
+                want = O.decode_attention_reference(q, kk, v, sinks, 1.0, sw, pos)
+                got = _run(case, 1.0, sw, pos)
+                U.assert_close(got, want, what=f"sw={sw} pos={pos} spike={spike}")
+                if lo <= spike <= hi:
+                    np.testing.assert_allclose(got[0, 0, 0], v[0, 0, spike], atol=2e-2)
+
+
+def test_unwritten_cache_beyond_position_is_never_read_into_the_result():
+    """Bytes past `position` may be anything (NaN codes, NaN/inf scales)."""
+    B, N, K, S, H = 2, 8, 2, 256, 128
+    case = U.attention_case(5, B, N, K, S, H, fp8=True)
+    pos = np.array([70, 200])
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, pos)
+    (kq, ks), (vq, vs) = case["k"], case["v"]
+    kq, vq, ks, vs = kq.copy(), vq.copy(), ks.copy(), vs.copy()
+    for b in range(B):
+        kq[b, :, pos[b] + 1 :] = 0x7F
+        vq[b, :, pos[b] + 1 :] = 0xFF
+        ks[b, :, pos[b] + 1 :] = np.nan
+        vs[b, :, pos[b] + 1 :] = np.inf
+    dirty = dict(case, k=(kq, ks), v=(vq, vs))
+    got = _run(dirty, H**-0.5, 0, pos)
+    U.assert_close(got, want, what="dirty tail")
+    # the same for a bf16 cache and a sliding window (keys before the window are garbage too)
+    case = U.attention_case(6, B, N, K, S, H, fp8=False)
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 64, pos)
+    kd, vd = case["k"].copy(), case["v"].copy()
+    for b in range(B):
+        kd[b, :, pos[b] + 1 :] = np.nan
+        vd[b, :, pos[b] + 1 :] = np.nan
+        kd[b, :, : pos[b] - 63] = np.nan
+        vd[b, :, : pos[b] - 63] = np.inf
+    got = _run(dict(case, k=kd, v=vd), H**-0.5, 64, pos)
+    U.assert_close(got, want, what="dirty head and tail")
+
+
+def test_sink_extremes_and_no_visible_key():
+    B, N, K, S, H = 1, 8, 2, 256, 64
+    case = U.attention_case(8, B, N, K, S, H, fp8=True)
+    for sink in (-1e30, -float("inf"), 50.0, 1e4):
+        c = dict(case, sinks=np.full(N, sink, np.float32))
+        want = O.decode_attention_reference(c["q"], c["k"], c["v"], np.full(N, max(sink, -1e30), np.float32), 0.125, 0, 255)
+        got = _run(c, 0.125, 0, 255)
+        U.assert_close(got, want, what=f"sink={sink}")
+    got = _run(case, 0.125, 0, -1)  # nothing cached yet: only the sink, whose value is 0
+    assert np.abs(got).max() == 0.0
+
+
+def test_split_count_does_not_change_the_result():
+    """Partition invariance of the log-sum-exp merge: same keys, different chunking (B changes the plan)."""
+    N, K, S, H = 8, 2, 4096, 128
+    base = U.attention_case(9, 1, N, K, S, H, fp8=True)
+    want = O.decode_attention_reference(base["q"], base["k"], base["v"], base["sinks"], H**-0.5, 0, 4000)
+    got1 = _run(base, H**-0.5, 0, 4000)  # B*K = 2 pairs -> many chunks
+    rep = 96  # B*K = 192 pairs -> fewer, longer chunks
+    big = dict(base, q=np.repeat(base["q"], rep, 0), k=tuple(np.repeat(a, rep, 0) for a in base["k"]), v=tuple(np.repeat(a, rep, 0) for a in base["v"]))
+    got2 = _run(big, H**-0.5, 0, 4000)
+    U.assert_close(got1, want, what="many chunks")
+    for b in (0, 17, rep - 1):
+        U.assert_close(got2[b : b + 1], want, what="few chunks")
+    assert np.abs(got2[:1] - got1).max() <= 1e-2
+
+
+def test_config4_gpt_oss_shape_ragged_fp8_full_size():
+    """BASELINE config 4: B=64, 64Q/8KV, H=64, S=4096, L_b ~ U{256..4096}, FP8 cache; global and window 128."""
+    B, N, K, S, H = 64, 64, 8, 4096, 64
+    case = U.attention_case(1004, B, N, K, S, H, fp8=True)
+    rng = np.random.default_rng(1004)
+    pos = (rng.integers(256, 4097, B) - 1).astype(np.int32)
+    (kq, ks), (vq, vs) = case["k"], case["v"]
+    for sw in (0, 128):
+        _note(f"attn cfg4 sw={sw}")
+        want = clib.decode_attention(O.bf16_bits(case["q"]), kq, vq, ks[..., 0], vs[..., 0], case["sinks"], pos, None, H**-0.5, sw)
+        got = _run(case, H**-0.5, sw, pos)
+        U.assert_close(got, want, what=f"cfg4 sw={sw}")
+    # size-independent property: doubling every V scale doubles the output bit for bit (power-of-two scaling
+    # commutes with every rounding in the kernel)
+    got2 = _run(dict(case, v=(vq, vs * 2.0)), H**-0.5, 0, pos)
+    got1 = _run(case, H**-0.5, 0, pos)
+    np.testing.assert_array_equal(got2, got1 * 2.0)
+
+
+def test_headline_shape_b64_ctx4096_fp8():
+    """B=64, ctx 4096, FP8 cache at the lyra-small shape (16Q/4KV/H=128), all rows full."""
+    B, N, K, S, H = 64, 16, 4, 4096, 128
+    case = U.attention_case(1000, B, N, K, S, H, fp8=True)
+    (kq, ks), (vq, vs) = case["k"], case["v"]
+    pos = np.full(B, S - 1, np.int32)
+    want = clib.decode_attention(O.bf16_bits(case["q"]), kq, vq, ks[..., 0], vs[..., 0], case["sinks"], pos, None, H**-0.5, 0)
+    got = _run(case, H**-0.5, 0, S - 1)
+    U.assert_close(got, want, what="headline")
+    # permuting the cached keys (with their values and scales) cannot change attention
+    perm = np.random.default_rng(1).permutation(S)
+    shuf = dict(case, k=(kq[:, :, perm], ks[:, :, perm]), v=(vq[:, :, perm], vs[:, :, perm]))
+    got_p = _run(shuf, H**-0.5, 0, S - 1)
+    assert np.abs(got_p - got).max() <= 1e-2
+
+
+def test_xla_path_and_dispatch_contract():
+    from lyra_amd.kernels.decode_attention import decode_attention
+
+    case = U.attention_case(11, 2, 8, 2, 384, 64, fp8=True)
+    q, k, v, sinks = U.attention_torch_inputs(case)
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], 0.125, 128, 300)
+    for impl in ("auto", "pallas", "hip", "xla"):
+        out = decode_attention(q, k, v, sinks, 0.125, 128, torch.tensor(300, dtype=torch.int32, device=U.dev()), implementation=impl)
+        assert out.shape == q.shape and out.dtype == q.dtype
+        U.assert_close(U.to_np(out), want, what=impl)
+    # unsupported head_dim: "pallas" raises like common.py:147-151, "auto" falls back to the plain path
+    c2 = U.attention_case(12, 1, 4, 2, 64, 32, fp8=False)
+    q2, k2, v2, s2 = U.attention_torch_inputs(c2)
+    with pytest.raises(ValueError, match="no HIP kernel configuration"):
+        decode_attention(q2, k2, v2, s2, 0.2, 0, 63, implementation="pallas")
+    out = decode_attention(q2, k2, v2, s2, 0.2, 0, 63, implementation="auto")
+    U.assert_close(U.to_np(out), O.decode_attention_reference(c2["q"], c2["k"], c2["v"], c2["sinks"], 0.2, 0, 63), what="fallback")
+    # a QArray handed to a dense config (and vice versa) is an error: decode_attention.py:199-200,215-216
+    from lyra_amd.kernels.decode_attention import DecodeAttentionConfig, _decode_attention
+
+    with pytest.raises(ValueError, match="requires QArray"):
+        _decode_attention(q, k.qval.to(torch.bfloat16), v.qval.to(torch.bfloat16), sinks, 0.125, 0, 3, DecodeAttentionConfig(cache_dtype=torch.float8_e4m3fn), torch.bfloat16)
+    with pytest.raises(ValueError, match="received QArray"):
+        _decode_attention(q, k, v, sinks, 0.125, 0, 3, DecodeAttentionConfig(), torch.bfloat16)

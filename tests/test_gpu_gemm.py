@@ -1,0 +1,208 @@
+"""GPU parity of the HIP decode GEMM (through the C ABI) against the CPU oracle.
+
+Tolerance: |got - want| <= 2e-2 + 1e-2*|want| against the fp32 oracle on the same dequantised
+weights; float32 outputs are held to 2e-3 + 2e-3*|want|.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import clib
+from oracle import lyra_oracle as O
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _note(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _weights(rng, G, K, N, w_std):
+    """N(0, w_std) weights.  Big shapes draw one expert-sized pool and give expert g a shifted window of it
+    (i.i.d. within an expert, which is all a parity test needs) to keep generation in seconds."""
+    if G * K * N <= (1 << 24):
+        return (rng.standard_normal((G, K, N), dtype=np.float32) * np.float32(w_std)).astype(np.float32)
+    pool = rng.standard_normal(K * N + 1009 * G, dtype=np.float32) * np.float32(w_std)
+    return np.stack([pool[1009 * g : 1009 * g + K * N].reshape(K, N) for g in range(G)])
+
+
+def _case(seed, M, G, K, N, sizes, *, kind, block=(256, 256), bias=False, w_std=0.02):
+    rng = np.random.default_rng(seed)
+    lhs = O.bf16_round(rng.standard_normal((M, K), dtype=np.float32))
+    w = _weights(rng, G, K, N, w_std)
+    c = {"lhs": lhs, "sizes": np.asarray(sizes, np.int32), "kind": kind, "block": block}
+    c["bias"] = rng.standard_normal((G, N)).astype(np.float32) if bias else None
+    if kind == "fp8":
+        c["w"] = clib.quantize_blocks(w, block)  # bit-identical to O.quantize (tests/test_oracle_formats.py)
+    else:
+        c["w"] = O.bf16_round(w)
+    return c
+
+
+def _want(c, swiglu, big=False):
+    if big:  # the C restatement (same arithmetic, threaded) for shapes numpy would take minutes on
+        if c["kind"] == "fp8":
+            q, s = c["w"]
+            return clib.decode_gemm(O.bf16_bits(c["lhs"]), q, s, c["block"], c["sizes"], c["bias"], fused_swiglu=swiglu)
+        return clib.decode_gemm(O.bf16_bits(c["lhs"]), O.bf16_bits(c["w"]), None, None, c["sizes"], c["bias"], fused_swiglu=swiglu)
+    if c["kind"] == "fp8":
+        return O.decode_gemm_reference(c["lhs"], c["w"], c["sizes"], block=c["block"], bias=c["bias"], fused_swiglu=swiglu)
+    return O.decode_gemm_reference(c["lhs"], c["w"], c["sizes"], bias=c["bias"], fused_swiglu=swiglu)
+
+
+def _run(c, swiglu, *, out_f32=False, implementation="pallas"):
+    from lyra_amd.kernels.decode_gemm import decode_gemm
+    from lyra_amd.nn.quant import QArray
+
+    lhs = U.t_bf16(c["lhs"])
+    if out_f32:
+        lhs = lhs.to(torch.float32)
+    if c["kind"] == "fp8":
+        q, s = c["w"]
+        rhs = QArray(U.t_fp8(q), U.t_f32(s), tuple(c["block"]))
+        qd = torch.float8_e4m3fn
+    else:
+        rhs = U.t_bf16(c["w"])
+        qd = None
+    gs = torch.from_numpy(c["sizes"]).to(U.dev())
+    bias = None if c["bias"] is None else U.t_f32(c["bias"])
+    out = decode_gemm(lhs, rhs, gs, bias=bias, fused_swiglu=swiglu, quant_dtype=qd, implementation=implementation)
+    torch.cuda.synchronize()
+    return U.to_np(out)
+
+
+@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", (512, 1)), ("fp8", (512, 128)), ("fp8", (64, 64))])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_small_grouped_shapes(kind, block, swiglu):
+    M, G, K, N = 11, 4, 512, 512
+    sizes = [3, 0, 7, 1]
+    c = _case(1, M, G, K, N, sizes, kind=kind, block=block, bias=True, w_std=0.05)
+    _note(f"gemm small kind={kind} block={block} swiglu={swiglu}")
+    want = _want(c, swiglu)
+    U.assert_close(_run(c, swiglu), want, what="bf16 out")
+    U.assert_close(_run(c, swiglu, out_f32=True), want, atol=2e-3, rtol=2e-3, what="f32 out")
+
+
+@pytest.mark.parametrize("sizes,M", [([0, 0, 0, 5], 5), ([5, 0, 0, 0], 5), ([1, 1, 1, 1], 4), ([2, 0, 1, 0], 6), ([0, 0, 0, 0], 3),
+                                     ([17, 0, 33, 2], 52), ([70, 1, 0, 9], 80)])
+def test_group_layouts_empty_groups_padding_rows_and_many_rows(sizes, M):
+    for K in (256, 1024):  # 1024 rows of K are split across workgroups, 256 are not
+        for kind, block in (("bf16", None), ("fp8", (256, 256))):
+            for swiglu in (False, True):
+                c = _case(2, M, 4, K, 256, sizes, kind=kind, block=(256, 256) if block else None, bias=True, w_std=0.05)
+                _note(f"gemm groups sizes={sizes} M={M} K={K} kind={kind} swiglu={swiglu}")
+                U.assert_close(_run(c, swiglu), _want(c, swiglu), what=f"sizes={sizes} K={K}")
+
+
+def test_untouched_experts_are_never_read():
+    """Weights of experts with no rows may be anything (here NaN codes / NaN scales)."""
+    M, G, K, N = 6, 8, 512, 256
+    sizes = [0, 4, 0, 0, 2, 0, 0, 0]
+    c = _case(3, M, G, K, N, sizes, kind="fp8", block=(256, 256))
+    want = _want(c, True)
+    q, s = c["w"]
+    q, s = q.copy(), s.copy()
+    for g, n in enumerate(sizes):
+        if n == 0:
+            q[g] = 0x7F
+            s[g] = np.nan
+    got = _run(dict(c, w=(q, s)), True)
+    U.assert_close(got, want, what="poisoned idle experts")
+
+
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (2048, 6144), (3072, 2048), (2880, 2816)])
+def test_dense_projection_is_the_one_group_case(K, N):
+    """quant.dot on [B,1,C] x [C,N] = decode_gemm with G == 1 (lyra-small widths, gpt-oss width 2880)."""
+    for M in (1, 8, 64):
+        for kind, block in (("fp8", (K, 1)), ("bf16", None)):
+            c = _case(4, M, 1, K, N, [M], kind=kind, block=block)
+            _note(f"gemm dense K={K} N={N} M={M} kind={kind}")
+            swiglu = N % 256 == 0 and N == 6144
+            U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what=f"dense M={M}")
+
+
+def _zipf_routing(rng, T, n_routed, k, n_shared):
+    p = 1.0 / np.arange(1, n_routed + 1) ** 1.1
+    p /= p.sum()
+    ids = np.stack([rng.choice(n_routed, size=k, replace=False, p=p) for _ in range(T)])
+    if n_shared:
+        ids = np.concatenate([ids, np.broadcast_to(np.arange(n_routed, n_routed + n_shared), (T, n_shared))], axis=1)
+    return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
+
+
+@pytest.mark.parametrize("T", [1, 16, 64])
+def test_config3_moe_medium_shape_zipf_routing(T):
+    """BASELINE config 3: width 4096, 31 routed + 1 shared expert, FP8 per-channel scales, top-(3+1) Zipf(1.1)."""
+    C, Hd, E = 4096, 4096, 32
+    rng = np.random.default_rng(1003 + T)
+    sizes = _zipf_routing(rng, T, 31, 3, 1)
+    M = int(sizes.sum())
+    up = _case(5, M, E, C, 2 * Hd, sizes, kind="fp8", block=(C, 1))
+    _note(f"gemm cfg3 up T={T} M={M} touched={(sizes > 0).sum()}")
+    want_up = _want(up, True, big=True)
+    got_up = _run(up, True)
+    U.assert_close(got_up, want_up, what="up+swiglu")
+    down = _case(6, M, E, Hd, C, sizes, kind="fp8", block=(Hd, 1))
+    down["lhs"] = O.bf16_round(want_up)
+    _note(f"gemm cfg3 down T={T}")
+    U.assert_close(_run(down, False), _want(down, False, big=True), what="down")
+
+
+def test_reference_default_blocks_256_at_small_moe_shape():
+    """lyra-small MoE: 15+1 experts, K=2048, up N=4096 with SwiGLU; QArray block (256,256) (model.py:154-156)."""
+    rng = np.random.default_rng(8)
+    sizes = _zipf_routing(rng, 8, 15, 3, 1)
+    M = int(sizes.sum())
+    c = _case(9, M, 16, 2048, 4096, sizes, kind="fp8", block=(256, 256), bias=True)
+    U.assert_close(_run(c, True), _want(c, True, big=True), what="small up")
+
+
+def test_linearity_and_row_independence_at_full_size():
+    """Size-independent properties at the medium expert shape: out(2x) == 2 out(x) bit for bit (no SwiGLU,
+    power-of-two scaling commutes with every rounding), and a row's result does not depend on its neighbours."""
+    C, N, E = 4096, 4096, 32
+    sizes = np.zeros(E, np.int32)
+    sizes[[0, 5, 31]] = [3, 1, 64]
+    M = int(sizes.sum())
+    c = _case(10, M, E, C, N, sizes, kind="fp8", block=(C, 1))
+    a = _run(c, False)
+    b = _run(dict(c, lhs=c["lhs"] * 2.0), False)
+    np.testing.assert_array_equal(b, a * 2.0)
+    solo = np.zeros(E, np.int32)
+    solo[31] = 1
+    one = _run(dict(c, lhs=c["lhs"][10:11], sizes=solo), False)
+    np.testing.assert_allclose(one[0], a[10], atol=1e-2, rtol=1e-2)
+
+
+def test_quantize_on_the_fly_and_dispatch_contract():
+    from lyra_amd.kernels.decode_gemm import decode_gemm
+    from lyra_amd.nn.quant import QArray
+
+    rng = np.random.default_rng(11)
+    M, G, K, N = 4, 2, 512, 512
+    lhs = O.bf16_round(rng.standard_normal((M, K), dtype=np.float32))
+    w = (rng.standard_normal((G, K, N)) * 0.05).astype(np.float32)
+    sizes = np.array([1, 3], np.int32)
+    gs = torch.from_numpy(sizes).to(U.dev())
+    # float weights + quant_dtype=fp8: quantised with block (gcd(K,256), gcd(N,256)) first (decode_gemm.py:427-428)
+    q, s = O.quantize(O.bf16_round(w), (256, 256))
+    want = O.decode_gemm_reference(lhs, (q, s), sizes, block=(256, 256))
+    for impl in ("auto", "pallas", "xla"):
+        out = decode_gemm(U.t_bf16(lhs), U.t_bf16(w), gs, quant_dtype=torch.float8_e4m3fn, implementation=impl)
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16
+        U.assert_close(U.to_np(out), want, what=f"on-the-fly {impl}")
+    # a QArray without quant_dtype is dequantised to lhs.dtype and multiplied as bf16 (decode_gemm.py:432-434)
+    rhs = QArray(U.t_fp8(q), U.t_f32(s), (256, 256))
+    out = decode_gemm(U.t_bf16(lhs), rhs, gs, implementation="pallas")
+    U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, (q, s), sizes, block=(256, 256), mode="ref"), what="dequantised")
+    # unsupported N: "pallas" raises, "auto" takes the plain path
+    w2 = U.t_bf16(w[:, :, :200])
+    with pytest.raises(ValueError, match="no HIP kernel configuration"):
+        decode_gemm(U.t_bf16(lhs), w2, gs, implementation="pallas")
+    out = decode_gemm(U.t_bf16(lhs), w2, gs, implementation="auto")
+    U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, O.bf16_round(w[:, :, :200]), sizes), what="fallback")
+    with pytest.raises(ValueError, match="Unsupported bias shape"):
+        decode_gemm(U.t_bf16(lhs), U.t_bf16(w), gs, bias=torch.zeros(3, N, device=U.dev()))

@@ -132,6 +132,19 @@ def test_quantize_matches_torch_elementwise():
     np.testing.assert_array_equal(sc, s.reshape(-1))
 
 
+def test_c_block_quantiser_matches_numpy():
+    rng = np.random.default_rng(6)
+    w = (rng.standard_normal((3, 512, 256)) * 0.02).astype(np.float32)
+    w[1, :256, :128] = 0.0
+    for block in ((256, 256), (512, 1), (64, 64), (512, 128)):
+        q, s = O.quantize(w, block)
+        qc, sc = clib.quantize_blocks(w, block)
+        np.testing.assert_array_equal(qc, q)
+        np.testing.assert_array_equal(sc, s)
+    with pytest.raises(ValueError):
+        clib.quantize_blocks(w, (300, 256))
+
+
 def test_qupdate_writes_one_token():
     rng = np.random.default_rng(5)
     cache = rng.standard_normal((2, 3, 16, 64)).astype(np.float32)
