@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 1
+#define LYRA_ABI_VERSION 2
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -54,8 +54,11 @@ const char* lyra_strerror(int code);
  *   out      [B,N,H] out_dtype (bf16 or float32)
  *   sliding_window  0 = global layer; w > 0 = only keys j with position-w < j <= position
  *   sm_scale        multiplies q.k (the reference passes H**-0.5)
- *   workspace       at least lyra_decode_attention_workspace(...) bytes, 256-byte aligned; holds
- *                   split partials for the duration of the call only
+ *   workspace       at least lyra_decode_attention_workspace(...) bytes, 256-byte aligned.  It holds split
+ *                   partials and arrival counters.  The counters must read zero when a call starts and are
+ *                   zero again when it ends: zero the buffer once after allocating it (lyra_workspace_init
+ *                   or any memset) and it can be reused by every later call, of any shape, on the same stream,
+ *                   as long as nothing else writes to it in between.
  * Supported: H in {64,128}; 1 <= N/K <= 16; any B, S >= 1.
  */
 int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
@@ -64,6 +67,12 @@ int lyra_decode_attention(const void* q, const void* k, const void* v, const flo
                           float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream);
 
 size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sliding_window);
+
+/*
+ * Zero `workspace_bytes` (a multiple of 4) of a workspace with a fill kernel on `stream` (safe to record
+ * into a HIP graph).  No counterpart in the reference; needed once per workspace allocation.
+ */
+int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t stream);
 
 /*
  * Decode grouped matmul: out[r,:] = epilogue(lhs[r,:] @ rhs[e(r)]) with rows sorted by group.

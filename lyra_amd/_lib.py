@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _c = ctypes
 SIGNATURES = {
@@ -19,6 +19,7 @@ SIGNATURES = {
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_workspace": (_c.c_size_t, [_c.c_int] * 6),
+    "lyra_workspace_init": (_c.c_int, [_c.c_void_p, _c.c_size_t, _c.c_void_p]),
     "lyra_decode_gemm": (
         _c.c_int,
         [_c.c_void_p] * 3 + [_c.c_int] * 2 + [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 7 + [_c.c_float] * 2 + [_c.c_void_p],
@@ -56,16 +57,20 @@ def check(code: int, what: str) -> None:
         raise LyraHipError(f"{what}: {lib.lyra_strerror(code).decode()} ({code})")
 
 
-_WORKSPACES: dict[tuple[int, int], "object"] = {}
+_WORKSPACES: dict[tuple[str, int, int], "object"] = {}
 
 
-def workspace(device, stream_ptr: int, nbytes: int):
-    """A reusable device scratch buffer per (device, stream); grows, never shrinks."""
+def workspace(kind: str, device, stream_ptr: int, nbytes: int):
+    """A reusable, zero-initialised device scratch buffer per (operator, device, stream); grows, never shrinks.
+
+    The attention kernel keeps arrival counters in it and returns them to zero, so it is zeroed only when
+    allocated and never shared with another operator.
+    """
     import torch
 
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    key = (kind, device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     buf = _WORKSPACES.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _WORKSPACES[key] = buf
     return buf

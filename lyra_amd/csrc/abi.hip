@@ -83,16 +83,27 @@ __global__ __launch_bounds__(64) void selftest_kernel(int32_t* report) {
         for (int r = 0; r < 4; ++r) bad_denorm += d[r] != ldexpf(1.f, -9);
     }
 
-    int vals[6] = {bad_mfma, bad_cvt, bad_cvt_bf16, bad_pack, bad_perm, bad_denorm};
-    for (int i = 0; i < 6; ++i) {
+    // [6] row exchanges: reductions over lanes {l, l^16, l^32, l^48}
+    int bad_rows = 0;
+    {
+        const float v = (float)((lane * 37) % 101);
+        float wmax = -1.f, wsum = 0.f;
+        for (int g = 0; g < 4; ++g) {
+            const float o = (float)(((16 * g + x) * 37) % 101);
+            wmax = fmaxf(wmax, o);
+            wsum += o;
+        }
+        bad_rows += group4_max(v) != wmax;
+        bad_rows += group4_sum(v) != wsum;
+    }
+
+    int vals[7] = {bad_mfma, bad_cvt, bad_cvt_bf16, bad_pack, bad_perm, bad_denorm, bad_rows};
+    for (int i = 0; i < 7; ++i) {
         int v = vals[i];
         for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
         if (lane == 0) report[i] = v;
     }
-    if (lane == 0) {
-        report[6] = 0;
-        report[7] = LYRA_ABI_VERSION;
-    }
+    if (lane == 0) report[7] = LYRA_ABI_VERSION;
 }
 
 }  // namespace lyra

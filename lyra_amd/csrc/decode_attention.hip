@@ -10,7 +10,8 @@
 //
 // Work decomposition (flash-decoding): workgroup = (chunk of the visible range, kv head, batch row);
 // its 4 wavefronts walk 32-token tiles round-robin, each keeping its own running (max, sum, out);
-// they are merged through LDS, and chunks are merged by a second kernel with wavefront shuffles.
+// they are merged through LDS.  Chunks are merged by whichever workgroup of the (batch row, kv head)
+// finishes last (an arrival counter in the workspace), so one launch does everything.
 //
 // Matrix-core mapping, per 32-token tile and wavefront (lane = 16*kb + x):
 //   S^T[token, head]  = K[16 tokens x H] . Q^T[H x 16 heads]   (A = K tile, B = Q^T, heads padded to 16)
@@ -18,6 +19,7 @@
 // The accumulator layout of the first product (lane x holds head x, tokens 4*kb+r) is exactly the B
 // operand layout of the second, so probabilities never leave their lane.
 #include <algorithm>
+#include <cstdlib>
 
 #include "lyra_device.h"
 
@@ -36,6 +38,7 @@ struct AttnParams {
     void* out;
     float* part_o;   // [B,K,n_chunks,G,H]
     float* part_ml;  // [B,K,n_chunks,G,2]
+    int* arrivals;   // [B,K] zero on entry, zero again on exit
     int B, N, K, S, G;
     float scale_log2;  // sm_scale * log2(e)
     int sw;
@@ -45,8 +48,8 @@ struct AttnParams {
     int scale_vec4;  // S % 4 == 0 -> scales are fetched as float4
 };
 
-constexpr int kAttnWaves = 4;
 constexpr int kTile = 32;
+constexpr int kMergeStageFloats = 3 * 1024 + 16;  // LDS floats used when the last workgroup merges chunks
 
 // Visible key range of one batch row; bit-exact restatement of the mask
 // (key <= pos) & (key > pos - sw)   (decode_attention.py:285-286, :338-340).
@@ -72,93 +75,118 @@ __device__ __forceinline__ void store_out(const AttnParams& p, size_t idx, float
     }
 }
 
+// Raw (still quantised) operands of one 32-token tile as this lane holds them.
 template <int H, bool FP8>
-struct RawTile {
+struct RawK {
     static constexpr int ES = FP8 ? 1 : 2;
     static constexpr int KW = ES * H / 16;  // dwords of one K row held by a lane (a quarter row)
-    static constexpr int VW = ES * H / 64;  // dwords of one V row held by a lane (H/16 columns)
     uint32_t k[2][KW];
-    uint32_t v[8][VW];
+};
+struct RawS {  // per-token scales of the 8 tokens whose logits this lane holds
     float ks[8];
     float vs[8];
 };
+template <int H, bool FP8>
+struct RawV {
+    static constexpr int ES = FP8 ? 1 : 2;
+    static constexpr int VW = ES * H / 64;  // dwords of one V row held by a lane (H/16 columns)
+    uint32_t v[8][VW];
+};
+
+// Buffer descriptors of one (batch row, kv head) slab.  Loads past the end of the slab return 0, and the
+// per-lane byte offsets are computed once: inside the loop only the tile offset (a scalar) changes.
+struct Slab {
+    __amdgpu_buffer_rsrc_t k, v, ks, vs;
+    int voff_k, voff_v, voff_s;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
 
 template <int H, bool FP8>
-__device__ __forceinline__ void load_tile(RawTile<H, FP8>& t, const AttnParams& p, const uint8_t* kbase,
-                                          const uint8_t* vbase, const float* ksbase, const float* vsbase, int base,
-                                          int lane) {
-    constexpr int ES = RawTile<H, FP8>::ES;
-    constexpr int KW = RawTile<H, FP8>::KW;
-    constexpr int VW = RawTile<H, FP8>::VW;
-    const int x = lane & 15, kb = lane >> 4;
-    const int last = p.S - 1;
+__device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base) {
+    constexpr int ES = RawK<H, FP8>::ES;
+    constexpr int KW = RawK<H, FP8>::KW;
+    constexpr int RB = H * ES;  // bytes per cached row
+    const int soff = __builtin_amdgcn_readfirstlane(base * RB);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int tok = min(base + 16 * j + x, last);
-        const uint8_t* row = kbase + (size_t)tok * (H * ES) + kb * (KW * 4);
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int w = 0; w < KW; w += 4) {
-            u32x4 d = *(const u32x4*)(row + w * 4);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, sl.voff_k + j * 16 * RB + w * 4, soff, 0);
             t.k[j][w] = d[0];
             t.k[j][w + 1] = d[1];
             t.k[j][w + 2] = d[2];
             t.k[j][w + 3] = d[3];
         }
-    }
+}
+
+template <bool VEC4>
+__device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base) {
+    const int ssoff = __builtin_amdgcn_readfirstlane(base * 4);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int tok0 = base + 16 * j + 4 * kb;
+        if constexpr (VEC4) {
+            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(sl.ks, sl.voff_s + j * 64, ssoff, 0);
+            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(sl.vs, sl.voff_s + j * 64, ssoff, 0);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int tok = min(tok0 + r, last);
-            const uint8_t* row = vbase + (size_t)tok * (H * ES) + x * (VW * 4);
-            if constexpr (VW == 1) {
-                t.v[4 * j + r][0] = *(const uint32_t*)row;
-            } else if constexpr (VW == 2) {
-                u32x2 d = *(const u32x2*)row;
-                t.v[4 * j + r][0] = d[0];
-                t.v[4 * j + r][1] = d[1];
-            } else {
-                u32x4 d = *(const u32x4*)row;
-                t.v[4 * j + r][0] = d[0];
-                t.v[4 * j + r][1] = d[1];
-                t.v[4 * j + r][2] = d[2];
-                t.v[4 * j + r][3] = d[3];
+            for (int r = 0; r < 4; ++r) {
+                t.ks[4 * j + r] = __uint_as_float(a[r]);
+                t.vs[4 * j + r] = __uint_as_float(b[r]);
             }
-        }
-        if constexpr (FP8) {
-            if (p.scale_vec4) {
-                const int g0 = min(tok0, p.S - 4);  // S % 4 == 0: the group of 4 is inside or wholly outside
-                f32x4 a = *(const f32x4*)(ksbase + g0);
-                f32x4 b = *(const f32x4*)(vsbase + g0);
+        } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    t.ks[4 * j + r] = a[r];
-                    t.vs[4 * j + r] = b[r];
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int tok = min(tok0 + r, last);
-                    t.ks[4 * j + r] = ksbase[tok];
-                    t.vs[4 * j + r] = vsbase[tok];
-                }
+            for (int r = 0; r < 4; ++r) {
+                t.ks[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.ks, sl.voff_s + j * 64 + r * 4, ssoff, 0));
+                t.vs[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.vs, sl.voff_s + j * 64 + r * 4, ssoff, 0));
             }
         }
     }
 }
 
-// One tile of online softmax.  MASKED tiles straddle the ends of the visible range: logits of
-// invisible keys become -inf and their V rows / scales are zeroed so that unwritten cache memory
-// (which may decode to NaN) cannot reach the accumulators.
-template <int H, bool FP8, bool MASKED>
-__device__ __forceinline__ void process_tile(RawTile<H, FP8>& t, const bf16x8 (&qop)[H / 32], int base, int lo, int hi,
-                                             float scale_log2, int lane, float& m, float& lsum, f32x4 (&o)[H / 16]) {
-    constexpr int NC = H / 32;  // k-steps of the S^T product
-    constexpr int CB = H / 16;  // 16-column blocks of O^T
-    const int kb = lane >> 4;
+template <int H, bool FP8>
+__device__ __forceinline__ void load_v(RawV<H, FP8>& t, const Slab& sl, int base) {
+    constexpr int ES = RawV<H, FP8>::ES;
+    constexpr int VW = RawV<H, FP8>::VW;
+    constexpr int RB = H * ES;
+    const int soff = __builtin_amdgcn_readfirstlane(base * RB);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int off = sl.voff_v + (16 * (i >> 2) + (i & 3)) * RB;
+        if constexpr (VW == 1) {
+            t.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(sl.v, off, soff, 0);
+        } else if constexpr (VW == 2) {
+            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(sl.v, off, soff, 0);
+            t.v[i][0] = d[0];
+            t.v[i][1] = d[1];
+        } else {
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.v, off, soff, 0);
+            t.v[i][0] = d[0];
+            t.v[i][1] = d[1];
+            t.v[i][2] = d[2];
+            t.v[i][3] = d[3];
+        }
+    }
+}
 
-    f32x4 s[2];
+// Running state of one wavefront: per lane the max and partial sum of head (lane & 15), and the
+// transposed output tile O^T[col, head] in matrix-core accumulator layout.
+template <int H>
+struct Acc {
+    float m, lsum;
+    f32x4 o[H / 16];
+};
+
+// First third of a tile: S^T = K Q^T on the matrix cores (raw FP8 values, scales applied later).
+template <int H, bool FP8>
+__device__ __forceinline__ void tile_logits(const RawK<H, FP8>& t, const uint16_t* sm_q, int lane, f32x4 (&s)[2]) {
+    constexpr int NC = H / 32;
+    constexpr int QP = H + 8;  // LDS pitch of a q row in bf16 elements
+    const int x = lane & 15, kb = lane >> 4;
+    bf16x8 qop[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) qop[c] = *(const bf16x8*)(sm_q + x * QP + kb * (H / 4) + 8 * c);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -178,57 +206,78 @@ __device__ __forceinline__ void process_tile(RawTile<H, FP8>& t, const bf16x8 (&
             s[j] = mfma_16x16x32(a, qop[c], s[j]);
         }
     }
+}
 
-    bool vis[8];
+// Second third: the online-softmax update, producing the probability operand (already multiplied by the
+// V scales).  MASKED tiles straddle the ends of the visible range: logits of invisible keys become -inf
+// and their probabilities exactly 0.
+template <int H, bool FP8, bool MASKED>
+__device__ __forceinline__ bf16x8 tile_softmax(const f32x4 (&s)[2], const RawS& t, int base, int lo, int hi, float scale_log2,
+                                               int lane, Acc<H>& acc, uint32_t& vis_bits) {
+    constexpr int CB = H / 16;
+    const int kb = lane >> 4;
     float sv[8];
     float tmax = -INFINITY;
+    vis_bits = 0xFFu;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int tok = base + 16 * (i >> 2) + 4 * kb + (i & 3);
-        vis[i] = !MASKED || (tok >= lo && tok <= hi);
-        float x = s[i >> 2][i & 3] * scale_log2;
-        if constexpr (FP8) x *= t.ks[i];
-        sv[i] = vis[i] ? x : -INFINITY;
-        tmax = fmaxf(tmax, sv[i]);
+        float v = s[i >> 2][i & 3];
+        if constexpr (FP8) v *= t.ks[i] * scale_log2;
+        else v *= scale_log2;
+        if constexpr (MASKED) {
+            const int tok = base + 16 * (i >> 2) + 4 * kb + (i & 3);
+            const bool ok = tok >= lo && tok <= hi;
+            if (!ok) {
+                v = -INFINITY;
+                vis_bits &= ~(1u << i);
+            }
+        }
+        sv[i] = v;
+        tmax = fmaxf(tmax, v);
     }
     tmax = group4_max(tmax);
-    const float m_new = fmaxf(m, tmax);
-    if (__ballot(m_new > m) != 0ull) {
-        const float alpha = fast_exp2(m - m_new);
-        lsum *= alpha;
+    const float m_new = fmaxf(acc.m, tmax);
+    if (__ballot(m_new > acc.m) != 0ull) {
+        const float alpha = fast_exp2(acc.m - m_new);
+        acc.lsum *= alpha;
 #pragma unroll
         for (int c = 0; c < CB; ++c) {
-            o[c][0] *= alpha;
-            o[c][1] *= alpha;
-            o[c][2] *= alpha;
-            o[c][3] *= alpha;
+            acc.o[c][0] *= alpha;
+            acc.o[c][1] *= alpha;
+            acc.o[c][2] *= alpha;
+            acc.o[c][3] *= alpha;
         }
-        m = m_new;
+        acc.m = m_new;
     }
-
     float pv[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const float pr = fast_exp2(sv[i] - m);
-        lsum += pr;
+        const float pr = fast_exp2(sv[i] - acc.m);
+        acc.lsum += pr;
         float w = pr;
         if constexpr (FP8) w *= t.vs[i];
-        pv[i] = vis[i] ? w : 0.f;
+        if constexpr (MASKED) w = (vis_bits >> i) & 1u ? w : 0.f;  // a garbage scale times 0 must stay 0
+        pv[i] = w;
     }
     Pack8 pop;
 #pragma unroll
     for (int i = 0; i < 4; ++i) pop.u[i] = pack_bf16(pv[2 * i], pv[2 * i + 1]);
+    return pop.v;
+}
 
+// Last third of a tile: O^T += V^T P^T.  Element i of column c of the V^T operand is V[token i, c]; the
+// bf16 pack step pairs two tokens, which transposes the row-major cache for free.  In MASKED tiles the
+// rows of invisible keys are zeroed first so unwritten cache memory (possibly NaN) cannot reach O.
+template <int H, bool FP8, bool MASKED>
+__device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_t vis_bits, Acc<H>& acc) {
+    constexpr int CB = H / 16;
     if constexpr (MASKED) {
-        constexpr int VW = RawTile<H, FP8>::VW;
+        constexpr int VW = RawV<H, FP8>::VW;
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int w = 0; w < VW; ++w) t.v[i][w] = vis[i] ? t.v[i][w] : 0u;
+            for (int w = 0; w < VW; ++w) t.v[i][w] = (vis_bits >> i) & 1u ? t.v[i][w] : 0u;
     }
-
-    // V^T operand: element i of column c is V[token i, c]; the bf16 pack step pairs two tokens, which
-    // transposes the row-major cache for free.
     if constexpr (FP8) {
 #pragma unroll
         for (int c = 0; c < CB; c += 2) {
@@ -240,8 +289,8 @@ __device__ __forceinline__ void process_tile(RawTile<H, FP8>& t, const bf16x8 (&
                 v0.u[i >> 1] = pack_bf16(fa[0], fb[0]);
                 v1.u[i >> 1] = pack_bf16(fa[1], fb[1]);
             }
-            o[c] = mfma_16x16x32(v0.v, pop.v, o[c]);
-            o[c + 1] = mfma_16x16x32(v1.v, pop.v, o[c + 1]);
+            acc.o[c] = mfma_16x16x32(v0.v, pop, acc.o[c]);
+            acc.o[c + 1] = mfma_16x16x32(v1.v, pop, acc.o[c + 1]);
         }
     } else {
 #pragma unroll
@@ -252,17 +301,18 @@ __device__ __forceinline__ void process_tile(RawTile<H, FP8>& t, const bf16x8 (&
                 const uint32_t a = t.v[i][c >> 1], b = t.v[i + 1][c >> 1];
                 vv.u[i >> 1] = (c & 1) ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
             }
-            o[c] = mfma_16x16x32(vv.v, pop.v, o[c]);
+            acc.o[c] = mfma_16x16x32(vv.v, pop, acc.o[c]);
         }
     }
 }
 
-template <int H, bool FP8>
-__global__ __launch_bounds__(kAttnWaves * 64) void decode_attention_kernel(AttnParams p) {
+template <int H, bool FP8, bool VEC4, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES >= 8 ? 4 : 3)))
+void decode_attention_kernel(AttnParams p) {
     constexpr int ES = FP8 ? 1 : 2;
-    constexpr int NC = H / 32;
     constexpr int CB = H / 16;
-    constexpr int HP = H + 4;  // LDS row pitch in floats
+    constexpr int HP = H + 4;  // LDS row pitch of the merge buffer in floats
+    constexpr int QP = H + 8;  // LDS row pitch of q in bf16 elements
     extern __shared__ float smem[];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -275,80 +325,114 @@ __global__ __launch_bounds__(kAttnWaves * 64) void decode_attention_kernel(AttnP
     const int c_lo = rg.start + c_idx * p.chunk;
     if (c_lo > rg.hi) {  // chunk holds no visible key (whole workgroup leaves together)
         if (p.n_chunks == 1)  // position < 0: only the sink is attended and its value is 0
-            for (int idx = threadIdx.x; idx < G * H; idx += kAttnWaves * 64)
+            for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64)
                 store_out(p, ((size_t)b * p.N + kh * G) * H + idx, 0.f, 1.f);
         return;
     }
     const int c_hi = min(c_lo + p.chunk, rg.hi + 1);
     const int n_tiles = (c_hi - c_lo + kTile - 1) / kTile;
 
-    // Q^T operand: lane (head x, k-group kb) holds q[head][kb*H/4 + 8c + i]; K lanes hold the same columns.
-    bf16x8 qop[NC];
-    {
-        const uint16_t* qrow = p.q + ((size_t)b * p.N + kh * G + min(x, G - 1)) * H + kb * (H / 4);
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            u32x4 d = *(const u32x4*)(qrow + 8 * c);
-            if (x >= G) d = u32x4{0u, 0u, 0u, 0u};
-            qop[c] = __builtin_bit_cast(bf16x8, d);
-        }
-    }
-    const float sink2 = x < G ? p.sinks[kh * G + x] * kLog2e : 0.f;
-    float m = fmaxf(sink2, -1e30f);  // finite start: fully masked tiles cannot produce inf - inf
-    float lsum = 0.f;
-    f32x4 o[CB];
-#pragma unroll
-    for (int c = 0; c < CB; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-
     const size_t head_row = ((size_t)b * p.K + kh) * p.S;
-    const uint8_t* kbase = p.k + head_row * (H * ES);
-    const uint8_t* vbase = p.v + head_row * (H * ES);
-    const float* ksbase = FP8 ? p.ks + head_row : nullptr;
-    const float* vsbase = FP8 ? p.vs + head_row : nullptr;
+    Slab sl;
+    sl.k = make_rsrc(p.k + head_row * (H * ES), (uint32_t)p.S * (H * ES));
+    sl.v = make_rsrc(p.v + head_row * (H * ES), (uint32_t)p.S * (H * ES));
+    sl.ks = make_rsrc(FP8 ? p.ks + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
+    sl.vs = make_rsrc(FP8 ? p.vs + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
+    sl.voff_k = x * (H * ES) + kb * (H * ES / 4);
+    sl.voff_v = 4 * kb * (H * ES) + x * (H * ES / 16);
+    sl.voff_s = 16 * kb;
 
-    RawTile<H, FP8> cur, nxt;
+    // first tile of this wavefront: request it before anything else so it overlaps the q staging
+    RawK<H, FP8> rk;
+    RawS rs;
+    RawV<H, FP8> rv;
     int tile = wave;
-    if (tile < n_tiles) load_tile<H, FP8>(cur, p, kbase, vbase, ksbase, vsbase, c_lo + tile * kTile, lane);
-    for (; tile < n_tiles; tile += kAttnWaves) {
-        const int base = c_lo + tile * kTile;
-        const bool more = tile + kAttnWaves < n_tiles;
-        if (more) load_tile<H, FP8>(nxt, p, kbase, vbase, ksbase, vsbase, base + kAttnWaves * kTile, lane);
-        if (base >= rg.lo && base + kTile - 1 <= rg.hi)
-            process_tile<H, FP8, false>(cur, qop, base, rg.lo, rg.hi, p.scale_log2, lane, m, lsum, o);
-        else
-            process_tile<H, FP8, true>(cur, qop, base, rg.lo, rg.hi, p.scale_log2, lane, m, lsum, o);
-        if (more) cur = nxt;
+    if (tile < n_tiles) {
+        load_k<H, FP8>(rk, sl, c_lo + tile * kTile);
+        if constexpr (FP8) load_s<VEC4>(rs, sl, c_lo + tile * kTile);
+        load_v<H, FP8>(rv, sl, c_lo + tile * kTile);
     }
-    lsum = group4_sum(lsum);
 
-    // ---- merge the 4 wavefronts through LDS -------------------------------------------------
-    float* sm_o = smem;                                  // [waves][G][HP]
-    float* sm_m = smem + kAttnWaves * G * HP;            // [waves][16]
-    float* sm_l = sm_m + kAttnWaves * 16;                // [waves][16]
+    // q of this kv head's G query heads, padded to 16 rows of zeros, in LDS: the Q^T operand of lane
+    // (head x, k-group kb) is q[x][kb*H/4 + 8c .. +8], the same columns the K lanes hold.
+    uint16_t* sm_q = (uint16_t*)smem;
+    for (int idx = threadIdx.x; idx < 16 * (H / 8); idx += WAVES * 64) {
+        const int row = idx / (H / 8), piece = idx - row * (H / 8);
+        u32x4 d = u32x4{0u, 0u, 0u, 0u};
+        if (row < G) d = *(const u32x4*)(p.q + ((size_t)b * p.N + kh * G + row) * H + piece * 8);
+        *(u32x4*)(sm_q + row * QP + piece * 8) = d;
+    }
+
+    Acc<H> acc;
+    const float sink2 = x < G ? p.sinks[kh * G + x] * kLog2e : 0.f;
+    acc.m = fmaxf(sink2, -1e30f);  // finite start: fully masked tiles cannot produce inf - inf
+    acc.lsum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CB; ++c) acc.o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+
+    // Software pipeline over this wavefront's tiles (wave, wave + WAVES, ...: a fixed assignment, so results are
+    // bit-reproducible from run to run) with a single register set: each operand of the
+    // next tile is requested right after the last use of the current one, so the loads fly during the rest
+    // of the iteration and no registers are spent on a second buffer.
+    while (tile < n_tiles) {
+        const int next_tile = tile + WAVES;
+        const int base = c_lo + tile * kTile;
+        const int next = c_lo + next_tile * kTile;
+        const bool more = next_tile < n_tiles;
+        const bool full = base >= rg.lo && base + kTile - 1 <= rg.hi;
+        f32x4 s[2];
+        tile_logits<H, FP8>(rk, sm_q, lane, s);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) load_k<H, FP8>(rk, sl, next);
+        __builtin_amdgcn_sched_barrier(0);
+        uint32_t vis;
+        bf16x8 pop;
+        if (full) pop = tile_softmax<H, FP8, false>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
+        else pop = tile_softmax<H, FP8, true>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (FP8) {
+            if (more) load_s<VEC4>(rs, sl, next);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (full) tile_values<H, FP8, false>(rv, pop, vis, acc);
+        else tile_values<H, FP8, true>(rv, pop, vis, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) load_v<H, FP8>(rv, sl, next);
+        __builtin_amdgcn_sched_barrier(0);
+        tile = next_tile;
+    }
+    acc.lsum = group4_sum(acc.lsum);
+
+    // ---- merge the wavefronts through LDS ---------------------------------------------------
+    __syncthreads();  // everyone is done reading q
+    float* sm_o = smem;                             // [waves][G][HP]
+    float* sm_m = smem + WAVES * G * HP;            // [waves][16]
+    float* sm_l = sm_m + WAVES * 16;                // [waves][16]
     if (x < G) {
         float* dst = sm_o + ((size_t)wave * G + x) * HP;
 #pragma unroll
         for (int c = 0; c < CB; ++c)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dst[(4 * kb + r) * CB + c] = o[c][r];
+            for (int r = 0; r < 4; ++r) dst[(4 * kb + r) * CB + c] = acc.o[c][r];
         if (kb == 0) {
-            sm_m[wave * 16 + x] = m;
-            sm_l[wave * 16 + x] = lsum;
+            sm_m[wave * 16 + x] = acc.m;
+            sm_l[wave * 16 + x] = acc.lsum;
         }
     }
     __syncthreads();
 
     const bool final_out = p.n_chunks == 1;
-    for (int idx = threadIdx.x; idx < G * H; idx += kAttnWaves * 64) {
+    for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64) {
         const int g = idx / H, col = idx - g * H;
         float mm = sm_m[g];
 #pragma unroll
-        for (int w = 1; w < kAttnWaves; ++w) mm = fmaxf(mm, sm_m[w * 16 + g]);
-        float acc = 0.f, l = 0.f;
+        for (int w = 1; w < WAVES; ++w) mm = fmaxf(mm, sm_m[w * 16 + g]);
+        float o = 0.f, l = 0.f;
 #pragma unroll
-        for (int w = 0; w < kAttnWaves; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float f = fast_exp2(sm_m[w * 16 + g] - mm);
-            acc += sm_o[((size_t)w * G + g) * HP + col] * f;
+            o += sm_o[((size_t)w * G + g) * HP + col] * f;
             l += sm_l[w * 16 + g] * f;
         }
         const int n = kh * G + g;
@@ -356,97 +440,170 @@ __global__ __launch_bounds__(kAttnWaves * 64) void decode_attention_kernel(AttnP
             const float sk = p.sinks[n] * kLog2e;
             const float den = l + fast_exp2(sk - mm);  // mm >= sink by construction
             const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
-            store_out(p, ((size_t)b * p.N + n) * H + col, acc / den, gate);
+            store_out(p, ((size_t)b * p.N + n) * H + col, o / den, gate);
         } else {
             const size_t item = ((size_t)b * p.K + kh) * p.n_chunks + c_idx;
-            p.part_o[(item * G + g) * H + col] = acc;
+            store_agent(p.part_o + (item * G + g) * H + col, o);
             if (col == 0) {
-                p.part_ml[(item * G + g) * 2] = mm;
-                p.part_ml[(item * G + g) * 2 + 1] = l;
+                store_agent(p.part_ml + (item * G + g) * 2, mm);
+                store_agent(p.part_ml + (item * G + g) * 2 + 1, l);
             }
         }
     }
-}
+    if (final_out) return;
 
-// Merge of the per-chunk partials: one wavefront per (batch row, query head).  Lanes first span the
-// chunks (log-sum-exp weights by wavefront shuffles), then the H output columns.
-template <int H>
-__global__ __launch_bounds__(64) void decode_attention_merge_kernel(AttnParams p) {
-    const int lane = threadIdx.x;
-    const int b = blockIdx.x / p.N, n = blockIdx.x - b * p.N;
-    const int G = p.G, kh = n / G, g = n - kh * G;
-    const int pos = p.position[(size_t)b * p.pos_stride];
-    const Range rg = visible_range(pos, p.sw, p.S);
-    int nvalid = rg.hi >= rg.lo ? (rg.hi + 1 - rg.start + p.chunk - 1) / p.chunk : 0;
-    nvalid = min(nvalid, p.n_chunks);
-
+    // ---- merge the chunks: the workgroup that arrives last reads every partial of this kv head ----
+    const int n_valid = min((rg.hi + 1 - rg.start + p.chunk - 1) / p.chunk, p.n_chunks);
+    __shared__ int sm_last;
+    wait_all_memory();  // this lane's partials have reached device-wide visibility
+    __syncthreads();    // ... and so have everybody else's in this workgroup, before the arrival is counted
+    if (threadIdx.x == 0) {
+        const int seen = add_agent(&p.arrivals[b * p.K + kh], 1);
+        sm_last = seen == n_valid - 1;
+        if (sm_last) store_agent(&p.arrivals[b * p.K + kh], 0);  // leave the counter ready for the next launch
+    }
+    __syncthreads();
+    if (!sm_last) return;
+    // weights of the chunks: every thread fetches one (max, sum) pair, then LDS holds exp2(m_c - m*) and the
+    // denominator per head; the output columns are then gathered with all loads of a thread in flight at once
     const size_t item0 = ((size_t)b * p.K + kh) * p.n_chunks;
-    const float sk = p.sinks[n] * kLog2e;
-    float mm = fmaxf(sk, -1e30f);
-    for (int c = lane; c < nvalid; c += 64) mm = fmaxf(mm, p.part_ml[((item0 + c) * G + g) * 2]);
-    mm = wave_max(mm);
-    float den = 0.f;
-    for (int c = lane; c < nvalid; c += 64) {
-        const float* ml = p.part_ml + ((item0 + c) * G + g) * 2;
-        den += ml[1] * fast_exp2(ml[0] - mm);
-    }
-    den = wave_sum(den) + fast_exp2(sk - mm);
-    const float inv = 1.f / den;
-
-    float acc[H / 64];
-#pragma unroll
-    for (int i = 0; i < H / 64; ++i) acc[i] = 0.f;
-    for (int c0 = 0; c0 < nvalid; c0 += 64) {
-        const int c = c0 + lane;
-        const float wl = c < nvalid ? fast_exp2(p.part_ml[((item0 + c) * G + g) * 2] - mm) : 0.f;
-        const int cnt = min(64, nvalid - c0);
-        for (int cc = 0; cc < cnt; ++cc) {
-            const float w = __shfl(wl, cc, 64);
-            const float* po = p.part_o + ((item0 + c0 + cc) * G + g) * H;
-#pragma unroll
-            for (int i = 0; i < H / 64; ++i) acc[i] += w * po[lane + 64 * i];
+    float* sm_w = smem;                 // [n_valid][G] weight of chunk c for head g
+    float* sm_den = smem + 1024;        // [G]
+    float* sm_cm = smem + 1024 + 16;    // [n_valid][G] chunk maxima
+    float* sm_cl = sm_cm + 1024;        // [n_valid][G] chunk sums
+    const bool staged = n_valid * G <= 1024;
+    if (staged) {
+        for (int i = threadIdx.x; i < n_valid * G; i += WAVES * 64) {
+            const float* ml = p.part_ml + (item0 * G + i) * 2;
+            sm_cm[i] = load_agent(ml);
+            sm_cl[i] = load_agent(ml + 1);
         }
-    }
-    const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
+        __syncthreads();
+        if (threadIdx.x < G) {
+            const int g = threadIdx.x;
+            const float sk = p.sinks[kh * G + g] * kLog2e;
+            float mm = fmaxf(sk, -1e30f);
+            for (int c = 0; c < n_valid; ++c) mm = fmaxf(mm, sm_cm[c * G + g]);
+            float den = fast_exp2(sk - mm);
+            for (int c = 0; c < n_valid; ++c) {
+                const float f = fast_exp2(sm_cm[c * G + g] - mm);
+                sm_w[c * G + g] = f;
+                den += sm_cl[c * G + g] * f;
+            }
+            sm_den[g] = den;
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64) {
+            const int g = idx / H, col = idx - g * H;
+            const int n = kh * G + g;
+            float o = 0.f;
+            for (int c0 = 0; c0 < n_valid; c0 += 8) {
+                float v[8];
 #pragma unroll
-    for (int i = 0; i < H / 64; ++i) {
-        store_out(p, ((size_t)b * p.N + n) * H + lane + 64 * i, acc[i] * inv, gate);
+                for (int u = 0; u < 8; ++u)
+                    v[u] = c0 + u < n_valid ? load_agent(p.part_o + ((item0 + c0 + u) * G + g) * H + col) : 0.f;
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (c0 + u < n_valid) o += v[u] * sm_w[(c0 + u) * G + g];
+            }
+            const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
+            store_out(p, ((size_t)b * p.N + n) * H + col, o / sm_den[g], gate);
+        }
+        return;
+    }
+    // more chunks than the staging area holds: plain per-thread loops (long contexts at tiny batch)
+    for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64) {
+        const int g = idx / H, col = idx - g * H;
+        const int n = kh * G + g;
+        const float sk = p.sinks[n] * kLog2e;
+        float mm = fmaxf(sk, -1e30f);
+        for (int c = 0; c < n_valid; ++c) mm = fmaxf(mm, load_agent(p.part_ml + ((item0 + c) * G + g) * 2));
+        float o = 0.f, den = fast_exp2(sk - mm);
+        for (int c = 0; c < n_valid; ++c) {
+            const float* ml = p.part_ml + ((item0 + c) * G + g) * 2;
+            const float f = fast_exp2(load_agent(ml) - mm);
+            den += load_agent(ml + 1) * f;
+            o += load_agent(p.part_o + ((item0 + c) * G + g) * H + col) * f;
+        }
+        const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
+        store_out(p, ((size_t)b * p.N + n) * H + col, o / den, gate);
     }
 }
 
 // ---- host side ---------------------------------------------------------------------------------
 struct AttnPlan {
-    int chunk, n_chunks;
+    int chunk, n_chunks, waves;
 };
+constexpr long kMaxSplitPairs = 16384;  // (batch row, kv head) pairs beyond which a launch is never chunked
 
-// Split so that the launch has a few workgroups per compute unit even at small batch, never below
-// one 128-token pass per workgroup.  Depends only on shapes, so plan and workspace size agree.
+static long env_long(const char* name) {
+    const char* e = getenv(name);
+    return e ? atol(e) : 0L;
+}
+
+// Split so that the launch fills the 256 compute units even at small batch, never below one pass of the
+// workgroup's wavefronts.  Depends only on shapes, so plan and workspace size agree.
 static AttnPlan plan_attention(int B, int K, int S, int sliding_window) {
+    static const long target_env = env_long("LYRA_ATTN_TARGET_WGS");  // tuning overrides, read once
+    static const long waves_env = env_long("LYRA_ATTN_WAVES");
     int span = S;  // longest visible range, measured from its tile-aligned start
     if (sliding_window > 0) span = std::min(S, sliding_window + kTile - 1);
-    const int unit = kAttnWaves * kTile;
-    const int max_chunks = (span + unit - 1) / unit;
     const long pairs = (long)B * K;
-    const long target = 256L * 8;  // workgroups
+    AttnPlan pl;
+    pl.waves = 4;
+    if (pairs >= 192 && span >= 2048) pl.waves = 8;  // one big workgroup per pair instead of chunks
+    if (waves_env == 4 || waves_env == 8 || waves_env == 16) pl.waves = (int)waves_env;
+    const int unit = pl.waves * kTile;
+    const int max_chunks = (span + unit - 1) / unit;
+    const long target = target_env > 0 ? target_env : 512;  // workgroups
     long want = (target + pairs - 1) / pairs;
+    if (span <= 2 * 128) want = 1;  // a window of a few tiles: one workgroup, no merge
+    if (pairs > kMaxSplitPairs) want = 1;
     int n_chunks = (int)std::max(1L, std::min((long)max_chunks, want));
     int chunk = (span + n_chunks - 1) / n_chunks;
     chunk = (chunk + unit - 1) / unit * unit;
-    n_chunks = (span + chunk - 1) / chunk;
-    return AttnPlan{chunk, n_chunks};
+    pl.n_chunks = (span + chunk - 1) / chunk;
+    pl.chunk = chunk;
+    return pl;
 }
 
+}  // namespace lyra
+
+namespace lyra {
+struct AttnWorkspace {
+    size_t arrivals_bytes, o_bytes, ml_bytes;
+    size_t total() const { return arrivals_bytes + o_bytes + ml_bytes; }
+};
+static AttnWorkspace attention_workspace(int B, int N, int K, int H, const AttnPlan& pl) {
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    AttnWorkspace w;
+    // fixed size whatever the shape, so calls of different shapes sharing one workspace never leave
+    // partial results where another call's counters live (chunking only happens below kMaxSplitPairs pairs)
+    w.arrivals_bytes = kMaxSplitPairs * sizeof(int);
+    const size_t items = (size_t)B * K * pl.n_chunks * (N / K);
+    w.o_bytes = up(items * H * sizeof(float));
+    w.ml_bytes = up(items * 2 * sizeof(float));
+    return w;
+}
+__global__ void zero_fill_kernel(uint32_t* p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
 }  // namespace lyra
 
 extern "C" size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sliding_window) {
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || H <= 0 || N % K) return 0;
     const lyra::AttnPlan pl = lyra::plan_attention(B, K, S, sliding_window);
     if (pl.n_chunks == 1) return 256;
-    const size_t items = (size_t)B * K * pl.n_chunks * (N / K);
-    size_t bytes = items * H * sizeof(float);
-    bytes = (bytes + 255) / 256 * 256;
-    bytes += items * 2 * sizeof(float);
-    return (bytes + 255) / 256 * 256;
+    return lyra::attention_workspace(B, N, K, H, pl).total();
+}
+
+extern "C" int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t stream) {
+    if (!workspace || workspace_bytes % 4 || ((uintptr_t)workspace % 4)) return LYRA_E_BADARG;
+    if (workspace_bytes == 0) return LYRA_OK;
+    const size_t n = workspace_bytes / 4;
+    const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
+    hipLaunchKernelGGL(lyra::zero_fill_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t*)workspace, n);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 
 extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale,
@@ -486,32 +643,42 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     p.chunk = pl.chunk;
     p.n_chunks = pl.n_chunks;
     p.out_f32 = out_dtype == LYRA_DTYPE_F32;
-    p.scale_vec4 = (S % 4 == 0) && (((uintptr_t)k_scale | (uintptr_t)v_scale) % 16 == 0);
+    const bool vec4 = (S % 4 == 0) && (((uintptr_t)k_scale | (uintptr_t)v_scale) % 16 == 0);
+    p.scale_vec4 = vec4;
+    p.arrivals = nullptr;
     if (pl.n_chunks > 1) {
-        const size_t need = lyra_decode_attention_workspace(B, N, K, S, H, sliding_window);
-        if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
-        const size_t items = (size_t)B * K * pl.n_chunks * G;
-        size_t obytes = (items * H * sizeof(float) + 255) / 256 * 256;
-        p.part_o = (float*)workspace;
-        p.part_ml = (float*)((char*)workspace + obytes);
+        const AttnWorkspace w = attention_workspace(B, N, K, H, pl);
+        if (!workspace || workspace_bytes < w.total() || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
+        p.arrivals = (int*)workspace;
+        p.part_o = (float*)((char*)workspace + w.arrivals_bytes);
+        p.part_ml = (float*)((char*)workspace + w.arrivals_bytes + w.o_bytes);
     }
 
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(pl.n_chunks, K, B), block(kAttnWaves * 64);
-    const size_t lds = ((size_t)kAttnWaves * G * (H + 4) + 2 * kAttnWaves * 16) * sizeof(float);
+    const dim3 grid(pl.n_chunks, K, B), block(pl.waves * 64);
+    const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16) * sizeof(float);
+    const size_t lds_q = (size_t)16 * (H + 8) * sizeof(uint16_t);
+    const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
+    const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
+#define LYRA_LAUNCH_ATTN_W(HH, F, V, W) \
+    hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W>), grid, block, lds, st, p)
+#define LYRA_LAUNCH_ATTN(HH, F, V)                              \
+    do {                                                        \
+        if (pl.waves == 4) LYRA_LAUNCH_ATTN_W(HH, F, V, 4);     \
+        else if (pl.waves == 8) LYRA_LAUNCH_ATTN_W(HH, F, V, 8); \
+        else LYRA_LAUNCH_ATTN_W(HH, F, V, 16);                  \
+    } while (0)
     if (H == 128) {
-        if (fp8) hipLaunchKernelGGL((decode_attention_kernel<128, true>), grid, block, lds, st, p);
-        else hipLaunchKernelGGL((decode_attention_kernel<128, false>), grid, block, lds, st, p);
+        if (!fp8) LYRA_LAUNCH_ATTN(128, false, false);
+        else if (vec4) LYRA_LAUNCH_ATTN(128, true, true);
+        else LYRA_LAUNCH_ATTN(128, true, false);
     } else {
-        if (fp8) hipLaunchKernelGGL((decode_attention_kernel<64, true>), grid, block, lds, st, p);
-        else hipLaunchKernelGGL((decode_attention_kernel<64, false>), grid, block, lds, st, p);
+        if (!fp8) LYRA_LAUNCH_ATTN(64, false, false);
+        else if (vec4) LYRA_LAUNCH_ATTN(64, true, true);
+        else LYRA_LAUNCH_ATTN(64, true, false);
     }
+#undef LYRA_LAUNCH_ATTN
+#undef LYRA_LAUNCH_ATTN_W
     if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
-    if (pl.n_chunks > 1) {
-        const dim3 mgrid(B * N), mblock(64);
-        if (H == 128) hipLaunchKernelGGL((decode_attention_merge_kernel<128>), mgrid, mblock, 0, st, p);
-        else hipLaunchKernelGGL((decode_attention_merge_kernel<64>), mgrid, mblock, 0, st, p);
-        if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
-    }
     return LYRA_OK;
 }

@@ -72,17 +72,54 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// butterfly over the four 16-lane groups of a wavefront (lanes l, l^16, l^32, l^48)
+// Exchange between the four 16-lane rows of a wavefront without going through LDS.
+// v_permlane32_swap swaps the upper 32 lanes of its first operand with the lower 32 of its second;
+// fed the same value twice it returns {x[l & 31], x[l | 32]}: both halves' values in every lane.
+// v_permlane16_swap does the same for odd/even rows of 16: {x[l & ~16], x[l | 16]}.
+__device__ __forceinline__ void both_halves32(float x, float& a, float& b) {
+    const uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void both_rows16(float x, float& a, float& b) {
+    const uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+}
+// reductions over lanes l, l^16, l^32, l^48 (the four rows that share l & 15)
 __device__ __forceinline__ float group4_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16, kWave));
-    x = fmaxf(x, __shfl_xor(x, 32, kWave));
-    return x;
+    float a, b;
+    both_halves32(x, a, b);
+    x = fmaxf(a, b);
+    both_rows16(x, a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float group4_sum(float x) {
-    x += __shfl_xor(x, 16, kWave);
-    x += __shfl_xor(x, 32, kWave);
-    return x;
+    float a, b;
+    both_halves32(x, a, b);
+    x = a + b;
+    both_rows16(x, a, b);
+    return a + b;
 }
+
+// Device-wide visible stores and loads (write-through / cache-bypassing at agent scope).  Producers publish
+// with store_agent + wait_all_memory, then bump an arrival counter with add_agent; a consumer that saw the
+// final count reads with load_agent.  No cache-wide write-back or invalidate is involved.
+__device__ __forceinline__ void store_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int add_agent(int* p, int v) {
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(int* p, int v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void wait_all_memory() { __builtin_amdgcn_s_waitcnt(0); }
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll

@@ -115,7 +115,7 @@ def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config
     out = torch.empty((B, N, 1, H), dtype=out_dtype, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     need = _lib.lib.lyra_decode_attention_workspace(B, N, K, S, H, int(sliding_window))
-    ws = _lib.workspace(dev, stream, need)
+    ws = _lib.workspace("attention", dev, stream, need)
     with torch.cuda.device(dev):
         rc = _lib.lib.lyra_decode_attention(
             q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(),

@@ -104,7 +104,7 @@ def _decode_gemm(lhs, rhs, group_sizes, config: DecodeGEMMConfig, *, bias, fused
     out = torch.empty((M, NO), dtype=k_out, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     need = _lib.lib.lyra_decode_gemm_workspace(M, G, K, N, int(fused_swiglu))
-    ws = _lib.workspace(dev, stream, need)
+    ws = _lib.workspace("gemm", dev, stream, need)
     with torch.cuda.device(dev):
         rc = _lib.lib.lyra_decode_gemm(
             lhs_c.data_ptr(), rhs_val.data_ptr(), rhs_scale.data_ptr() if rhs_scale is not None else None, bk, bn,

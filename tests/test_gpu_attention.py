@@ -39,8 +39,8 @@ def test_selftest_layouts_and_conversions():
     _lib.check(_lib.lib.lyra_selftest(rep.data_ptr(), None), "lyra_selftest")
     torch.cuda.synchronize()
     r = rep.cpu().tolist()
-    assert r[:6] == [0, 0, 0, 0, 0, 0], f"mfma/cvt/cvt_bf16/pack/perm/denorm mismatches: {r}"
-    assert r[7] == 1
+    assert r[:7] == [0] * 7, f"mfma/cvt/cvt_bf16/pack/perm/denorm/rows mismatches: {r}"
+    assert r[7] == _lib.ABI_VERSION
 
 
 @pytest.mark.parametrize("fp8", [False, True])
