@@ -92,8 +92,8 @@ int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t s
  *               g = min(t[:, j], limit)  (lyra/kernels/common.py:98-114); out is then [M,N/2]
  *   out         [M,N] or [M,N/2], out_dtype (bf16 or float32)
  *   workspace   at least lyra_decode_gemm_workspace(...) bytes, 256-byte aligned
- * Supported: K % 32 == 0, N % 128 == 0 (N % 256 == 0 with fused_swiglu), fp8 blocks with
- * bk % 32 == 0 or bk == K, and bn % 128 == 0 or bn == 1.
+ * Supported: K % 32 == 0, N % 128 == 0 (N % 256 == 0 with fused_swiglu), G <= 8191; fp8 blocks with bn a
+ * power of two, and either (bn % 8 == 0 and (bk % 32 == 0 or bk == K)) or bk == K.
  */
 int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
                      const int32_t* group_sizes, const float* bias, void* out, void* workspace,

@@ -8,11 +8,13 @@
 // to BF16 on the matrix cores and applies the block scales to the float32 accumulators.
 //
 // Mapping: the weight matrix is row-major [K,N] (N contiguous).  A wavefront owns 128 output columns
-// (64 gate + 64 linear columns when SwiGLU is fused) and walks K in steps of 32 rows.  Lane
+// (64 gate + 64 linear columns when SwiGLU is fused) and walks K in steps of 32 rows; the 4 wavefronts of a
+// workgroup share the activations, staged in LDS 512 rows of K at a time.  Lane
 // (x = lane & 15, kb = lane >> 4) reads 8 consecutive columns of the 8 rows 8*kb .. 8*kb+7; pairing two
 // rows in the bf16 pack step yields the K-major B operand, so the transposition costs nothing.
 //   D[16 rows, 16 cols] += X[16 rows x 32 k] . W[32 k x 16 cols]   for each of the 8 column phases.
 #include <algorithm>
+#include <cstdlib>
 
 #include "lyra_device.h"
 
@@ -28,10 +30,12 @@ struct GemmParams {
     float* part;  // [ksplit, M, N] float32 partial products when ksplit > 1
     int M, G, K, N;
     int bk, bn, KB, NB;
+    int bn_shift;  // log2(bn): scale columns are power-of-two wide
     int scale_mode;  // 0 none, 1 one scale per lane and k-block (bn % 8 == 0), 2 per column (bk == K)
     int out_f32, swiglu;
     float beta, limit;
     int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
+    int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
 };
 
 __device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, float limit) {
@@ -41,69 +45,52 @@ __device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, fl
     return (lin + 1.0f) * (glu * sig);
 }
 
-template <bool FP8, int MT>
-struct RawStep {
+constexpr int kGemmWaves = 4;  // wavefronts per workgroup, each on its own 128-column span
+
+template <bool FP8>
+struct RawW {
     static constexpr int WW = FP8 ? 2 : 4;  // dwords per lane per weight row (8 columns)
     uint32_t w[8][WW];
-    u32x4 x[MT];
 };
 
-template <bool FP8, int MT>
-__device__ __forceinline__ void load_step(RawStep<FP8, MT>& s, const uint8_t* wlane, size_t row_bytes,
-                                          const uint16_t* xlane, size_t x_stride, int kk, int n_mt,
-                                          const bool (&row_ok)[MT]) {
-    constexpr int WW = RawStep<FP8, MT>::WW;
-    const uint8_t* wp = wlane + (size_t)kk * row_bytes;
+// Two of the 8 weight rows of this lane (rows kk + 8*kb + 2*pair, +1), 8 columns each.  The lane part of the
+// address is fixed (voff); the row part is uniform and travels in a scalar register.
+template <bool FP8>
+__device__ __forceinline__ void load_w_pair(RawW<FP8>& t, int pair, __amdgpu_buffer_rsrc_t rsrc, int voff, int kk, int row_bytes) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        if constexpr (WW == 2) {
-            u32x2 d = *(const u32x2*)(wp + (size_t)i * row_bytes);
-            s.w[i][0] = d[0];
-            s.w[i][1] = d[1];
+    for (int h = 0; h < 2; ++h) {
+        const int i = 2 * pair + h;
+        const int soff = __builtin_amdgcn_readfirstlane((kk + i) * row_bytes);
+        if constexpr (FP8) {
+            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 0);
+            t.w[i][0] = d[0];
+            t.w[i][1] = d[1];
         } else {
-            u32x4 d = *(const u32x4*)(wp + (size_t)i * row_bytes);
-            s.w[i][0] = d[0];
-            s.w[i][1] = d[1];
-            s.w[i][2] = d[2];
-            s.w[i][3] = d[3];
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+            t.w[i][0] = d[0];
+            t.w[i][1] = d[1];
+            t.w[i][2] = d[2];
+            t.w[i][3] = d[3];
         }
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        u32x4 d = u32x4{0u, 0u, 0u, 0u};
-        if (mt < n_mt && row_ok[mt]) d = *(const u32x4*)(xlane + (size_t)mt * 16 * x_stride + kk);
-        s.x[mt] = d;
     }
 }
 
-template <bool FP8, int MT>
-__device__ __forceinline__ void compute_step(const RawStep<FP8, MT>& s, int n_mt, f32x4 (&acc)[MT][8]) {
+// Element `pair` of the K-major B operands of all 8 column phases: pairing two weight rows in the bf16 pack
+// step transposes the row-major weights for free.
+template <bool FP8>
+__device__ __forceinline__ void convert_pair(const RawW<FP8>& t, int pair, Pack8 (&bop)[8]) {
+    const int i = 2 * pair;
 #pragma unroll
     for (int c = 0; c < 8; c += 2) {
-        Pack8 b0, b1;
         if constexpr (FP8) {
-#pragma unroll
-            for (int i = 0; i < 8; i += 2) {
-                const f32x2 fa = fp8x2_to_f32(s.w[i][c >> 2], (c & 2) != 0);
-                const f32x2 fb = fp8x2_to_f32(s.w[i + 1][c >> 2], (c & 2) != 0);
-                b0.u[i >> 1] = pack_bf16(fa[0], fb[0]);
-                b1.u[i >> 1] = pack_bf16(fa[1], fb[1]);
-            }
+            const f32x2 fa = fp8x2_to_f32(t.w[i][c >> 2], (c & 2) != 0);
+            const f32x2 fb = fp8x2_to_f32(t.w[i + 1][c >> 2], (c & 2) != 0);
+            bop[c].u[pair] = pack_bf16(fa[0], fb[0]);
+            bop[c + 1].u[pair] = pack_bf16(fa[1], fb[1]);
         } else {
-#pragma unroll
-            for (int i = 0; i < 8; i += 2) {
-                const uint32_t a = s.w[i][c >> 1], b = s.w[i + 1][c >> 1];
-                b0.u[i >> 1] = __builtin_amdgcn_perm(b, a, 0x05040100u);
-                b1.u[i >> 1] = __builtin_amdgcn_perm(b, a, 0x07060302u);
-            }
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            if (mt < n_mt) {
-                const bf16x8 xa = __builtin_bit_cast(bf16x8, s.x[mt]);
-                acc[mt][c] = mfma_16x16x32(xa, b0.v, acc[mt][c]);
-                acc[mt][c + 1] = mfma_16x16x32(xa, b1.v, acc[mt][c + 1]);
-            }
+            const uint32_t a = t.w[i][c >> 1], b = t.w[i + 1][c >> 1];
+            bop[c].u[pair] = __builtin_amdgcn_perm(b, a, 0x05040100u);
+            bop[c + 1].u[pair] = __builtin_amdgcn_perm(b, a, 0x07060302u);
         }
     }
 }
@@ -151,12 +138,16 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
 }
 
 template <bool FP8, int MT>
-__global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 3 : 2)))
+void decode_gemm_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    constexpr int KC = 512;          // rows of K whose activations are staged in LDS at a time
+    constexpr int XPITCH = KC + 8;   // LDS pitch of a staged row in bf16 elements (keeps 16-lane reads conflict free)
+    extern __shared__ uint16_t sm_x[];  // [16*MT rows][XPITCH] activations of the current K chunk, zero padded
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
-    const int g = blockIdx.z, ks = blockIdx.y;
-    const int span = blockIdx.x * waves + wave;  // which 128-column span this wavefront owns
+    const int g = blockIdx.z / p.row_par, rpar = blockIdx.z - g * p.row_par, ks = blockIdx.y;
+    const int span = blockIdx.x * kGemmWaves + wave;  // which 128-column span this wavefront owns
 
     // rows of this group: [off, off + cnt)
     int part_sum = 0;
@@ -165,8 +156,8 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
     for (int o = 32; o > 0; o >>= 1) part_sum += __shfl_xor(part_sum, o, kWave);
     const int off = min(part_sum, p.M);
     const int cnt = min(p.group_sizes[g], p.M - off);
-    const int pad_from = (g == p.G - 1 && p.ksplit == 1 && ks == 0) ? off + cnt : p.M;  // rows past the last group
-    if (cnt <= 0 && pad_from >= p.M) return;
+    const int pad_from = (g == p.G - 1 && rpar == 0 && p.ksplit == 1 && ks == 0) ? off + cnt : p.M;  // rows past the last group
+    if (cnt <= rpar * 16 * MT && pad_from >= p.M) return;  // no rows for this workgroup: its weights are never touched
 
     // columns of this lane
     int ncol, out_col;
@@ -181,22 +172,20 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
         span_ok = span * 128 < p.N;
         ncol = out_col = span * 128 + 8 * x;
     }
-    if (!span_ok) return;
+    if (!span_ok) ncol = out_col = 0;  // idle wavefront of the last workgroup: keeps pace, stores nothing
 
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
-    const size_t row_bytes = (size_t)p.N * ES;
-    const uint8_t* wlane = p.rhs + ((size_t)g * p.K + 8 * kb) * row_bytes + (size_t)ncol * ES;
+    const int row_bytes = p.N * ES;
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+    const int wvoff = 8 * kb * row_bytes + ncol * ES;
     const float* sc_lane = nullptr;
-    if (FP8 && p.scale_mode == 1) sc_lane = p.scale + (size_t)g * p.KB * p.NB + ncol / p.bn;
+    if (FP8 && p.scale_mode == 1) sc_lane = p.scale + (size_t)g * p.KB * p.NB + (ncol >> p.bn_shift);
 
-    for (int rb = 0; rb < cnt; rb += 16 * MT) {
+    for (int rb = rpar * 16 * MT; rb < cnt; rb += p.row_par * 16 * MT) {
         const int rowbase = off + rb;
         const int rows_here = min(16 * MT, cnt - rb);
         const int n_mt = (rows_here + 15) >> 4;
-        bool row_ok[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) row_ok[mt] = mt * 16 + x < rows_here;
-        const uint16_t* xlane = p.lhs + (size_t)(rowbase + x) * p.K + 8 * kb;
 
         f32x4 acc[MT][8];
 #pragma unroll
@@ -207,18 +196,40 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
         // accumulators are kept in units of the current block scale; on a k-block boundary they are
         // re-expressed in the next block's unit, and the last unit is applied at the end
         float s_cur = 1.f, s_next = 1.f;
+        const float* sc_ptr = sc_lane;  // scale of the k-block that starts at blk_kk
+        int blk_kk = k0;
         if (FP8 && p.scale_mode == 1) {
-            s_cur = sc_lane[(size_t)(k0 / p.bk) * p.NB];
+            sc_ptr += (size_t)(k0 / p.bk) * p.NB;
+            s_cur = *sc_ptr;
             s_next = s_cur;
         }
 
-        RawStep<FP8, MT> cur, nxt;
-        if (k0 < k1) load_step<FP8, MT>(cur, wlane, row_bytes, xlane, p.K, k0, n_mt, row_ok);
-        for (int kk = k0; kk < k1; kk += 32) {
-            const bool more = kk + 32 < k1;
-            if (more) load_step<FP8, MT>(nxt, wlane, row_bytes, xlane, p.K, kk + 32, n_mt, row_ok);
-            if (FP8 && p.scale_mode == 1 && p.bk < p.K) {
-                if (kk % p.bk == 0) {
+        // One register set of raw weights: a pair of rows is requested again (for the next step) as soon as it
+        // has been converted, so weight loads are in flight during the whole step.
+        RawW<FP8> w;
+        if (k0 < k1) {
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) load_w_pair<FP8>(w, pr, wrsrc, wvoff, k0, row_bytes);
+        }
+
+        for (int kc = k0; kc < k1; kc += KC) {
+            const int kc_end = min(kc + KC, k1);
+            // The 4 wavefronts share the activations of this K chunk through LDS: lane = 16-byte piece of a row,
+            // wavefront = row phase.  (The first weights of the chunk are already in flight.)
+            __syncthreads();  // the previous chunk has been consumed by every wavefront
+            const int pieces = (kc_end - kc) >> 3;  // <= 64
+            if (lane < pieces) {
+                for (int r = wave; r < 16 * n_mt; r += kGemmWaves) {
+                    u32x4 d = u32x4{0u, 0u, 0u, 0u};
+                    if (r < rows_here) d = *(const u32x4*)(p.lhs + (size_t)(rowbase + r) * p.K + kc + lane * 8);
+                    *(u32x4*)(sm_x + r * XPITCH + lane * 8) = d;
+                }
+            }
+            __syncthreads();
+
+            for (int kk = kc; kk < kc_end; kk += 32) {
+                const bool more = kk + 32 < k1;
+                if (FP8 && p.scale_mode == 1 && p.bk < p.K && kk == blk_kk) {
                     if (kk != k0) {
                         const float ratio = s_cur / s_next;
 #pragma unroll
@@ -233,12 +244,28 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
                                 }
                         s_cur = s_next;
                     }
-                    const int nb = kk / p.bk + 1;  // prefetch the following block's scale
-                    if (nb * p.bk < k1) s_next = sc_lane[(size_t)nb * p.NB];
+                    blk_kk += p.bk;  // prefetch the following block's scale
+                    sc_ptr += p.NB;
+                    if (blk_kk < k1) s_next = *sc_ptr;
                 }
+                Pack8 bop[8];
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    convert_pair<FP8>(w, pr, bop);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (more) load_w_pair<FP8>(w, pr, wrsrc, wvoff, kk + 32, row_bytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    if (mt < n_mt) {
+                        const bf16x8 a = *(const bf16x8*)(sm_x + (mt * 16 + x) * XPITCH + (kk - kc) + 8 * kb);
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(a, bop[c].v, acc[mt][c]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            compute_step<FP8, MT>(cur, n_mt, acc);
-            if (more) cur = nxt;
         }
 
         float colscale[8];
@@ -246,7 +273,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
         for (int c = 0; c < 8; ++c) colscale[c] = s_cur;
         if (FP8 && p.scale_mode == 2) {
 #pragma unroll
-            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)g * p.NB + (ncol + c) / p.bn];
+            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)g * p.NB + ((ncol + c) >> p.bn_shift)];
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -257,7 +284,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
                     float t[8];
 #pragma unroll
                     for (int c = 0; c < 8; ++c) t[c] = acc[mt][c][r] * colscale[c];
-                    finish_row(p, t, g, rowbase + lr, ncol, out_col, ks, lr < rows_here, is_lin_lane);
+                    finish_row(p, t, g, rowbase + lr, ncol, out_col, ks, span_ok && lr < rows_here, is_lin_lane);
                 }
             }
         }
@@ -268,7 +295,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(GemmParams p) {
         float t[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) t[c] = 0.f;
-        finish_row(p, t, g, row0 + kb, ncol, out_col, ks, row0 + kb < p.M, is_lin_lane);
+        finish_row(p, t, g, row0 + kb, ncol, out_col, ks, span_ok && row0 + kb < p.M, is_lin_lane);
     }
 }
 
@@ -323,32 +350,39 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
 }
 
 struct GemmPlan {
-    int mt;      // 16-row tiles held in registers per pass
-    int waves;   // wavefronts per workgroup
-    int spans;   // 128-column spans (64+64 with SwiGLU)
+    int mt;       // 16-row tiles held in registers per pass
+    int row_par;  // row blocks of one group spread over this many workgroups
+    int spans;    // 128-column spans (64+64 with SwiGLU)
     int ksplit, kpart;
 };
 
-// Shape-only plan (group sizes live on the device): enough workgroups to fill 256 compute units,
-// splitting K when the column spans of the touched experts alone are too few.
+// Shape-only plan (group sizes live on the device).  Large weight sets are streamed once: wide row blocks, K
+// split only as far as needed to fill 256 compute units.  Small ones (a few MB: the dense projections) are
+// latency bound, so they are cut into as many independent 16-row x 128-column x K-slice pieces as the
+// float32 partials allow, even though row tiles of one group then read the same weights through L2.
 static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) {
+    static const long target_env = [] {
+        const char* e = getenv("LYRA_GEMM_TARGET_WGS");  // tuning override, read once
+        return e ? atol(e) : 0L;
+    }();
     GemmPlan pl;
-    pl.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
     const int touched = std::max(1, std::min(G, M));
-    const long waves_noksplit = (long)pl.spans * touched;
-    const long target_waves = 256L * 8;
+    const double weight_bytes = (double)touched * K * N;
+    const bool small = weight_bytes <= 48e6 && M > 16;
+    pl.mt = M <= 16 ? 1 : (small ? 1 : (M <= 32 ? 2 : 4));
+    pl.row_par = small ? std::min(8, (M / std::max(1, touched) + 15) / 16) : 1;
+    pl.row_par = std::max(1, pl.row_par);
+    pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
+    const long wgs_noksplit = (long)((pl.spans + kGemmWaves - 1) / kGemmWaves) * touched * pl.row_par;
+    const long target = target_env > 0 ? target_env : 512;
     int unit = 32;
-    if (bk > 0 && bk < K) unit = bk;  // splits start on a scale-block boundary
+    if (bk > 0 && bk < K) unit = std::max(unit, bk);  // splits start on a scale-block boundary
     const int max_split = std::max(1, K / std::max(unit, 256));
-    int ksplit = (int)std::min((long)max_split, std::max(1L, target_waves / std::max(1L, waves_noksplit)));
+    int ksplit = (int)std::min((long)max_split, std::max(1L, target / std::max(1L, wgs_noksplit)));
     int kpart = (K + ksplit - 1) / ksplit;
     kpart = (kpart + unit - 1) / unit * unit;
-    ksplit = (K + kpart - 1) / kpart;
-    pl.ksplit = ksplit;
+    pl.ksplit = (K + kpart - 1) / kpart;
     pl.kpart = kpart;
-    pl.waves = pl.spans % 4 == 0 ? 4 : (pl.spans % 2 == 0 ? 2 : 1);
-    if ((long)pl.spans / pl.waves * touched * ksplit < 256) pl.waves = 1;
     return pl;
 }
 
@@ -373,15 +407,18 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
     if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
-    if (K % 32 || N % 128 || (fused_swiglu && N % 256) || G > 65535) return LYRA_E_UNSUPPORTED;
+    if (K % 32 || N % 128 || (fused_swiglu && N % 256) || G > 8191) return LYRA_E_UNSUPPORTED;
 
     GemmParams p;
     p.scale_mode = 0;
     p.bk = p.bn = 1;
     p.KB = p.NB = 1;
+    p.bn_shift = 0;
     if (fp8) {
         if (bk <= 0 || bn <= 0 || K % bk || N % bn) return LYRA_E_BADARG;
+        if (bn & (bn - 1)) return LYRA_E_UNSUPPORTED;  // scale columns must be a power of two wide
         p.bk = bk; p.bn = bn; p.KB = K / bk; p.NB = N / bn;
+        p.bn_shift = __builtin_ctz((unsigned)bn);
         if (bn % 8 == 0 && (bk % 32 == 0 || bk == K)) p.scale_mode = 1;
         else if (bk == K) p.scale_mode = 2;
         else return LYRA_E_UNSUPPORTED;
@@ -400,6 +437,7 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
     p.beta = swiglu_beta;
     p.limit = swiglu_limit;
     p.ksplit = pl.ksplit;
+    p.row_par = pl.row_par;
     p.kpart = pl.kpart;
     if (pl.ksplit > 1) {
         const size_t need = ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
@@ -408,8 +446,9 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
     }
 
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid((pl.spans + pl.waves - 1) / pl.waves, pl.ksplit, G), block(pl.waves * 64);
-#define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, 0, st, p)
+    const dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
+    const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t);
+#define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p)
     if (fp8) {
         if (pl.mt == 1) LYRA_LAUNCH_GEMM(true, 1);
         else if (pl.mt == 2) LYRA_LAUNCH_GEMM(true, 2);

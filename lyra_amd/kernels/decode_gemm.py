@@ -27,7 +27,7 @@ class DecodeGEMMConfig:
 
 def _scale_layout_supported(k: int, n: int, block: tuple[int, int]) -> bool:
     bk, bn = block
-    if bk <= 0 or bn <= 0 or k % bk or n % bn:
+    if bk <= 0 or bn <= 0 or k % bk or n % bn or bn & (bn - 1):
         return False
     if bn % 8 == 0 and (bk % 32 == 0 or bk == k):
         return True
