@@ -1,0 +1,63 @@
+"""Generation driver for decode mode (lyra/generate.py of the reference, minus tokenizer and REPL)."""
+from __future__ import annotations
+
+import torch
+
+from lyra_amd.model import ModelCache, ModelConfig, ModelWeights, model_apply
+
+
+def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Generator | None = None) -> torch.Tensor:
+    """lyra/generate.py:46-53 applied to each row of ``logits`` [B, V]: greedy when temperature <= 0, else
+    temperature scaling, top-k masking (lowest index wins ties, like lax.top_k) and a categorical draw."""
+    if cfg.sample_temperature <= 0:
+        return torch.argmax(logits, dim=-1).to(torch.int32)
+    logits = logits.to(torch.float32) / cfg.sample_temperature
+    if 0 < cfg.sample_topk < logits.shape[-1]:
+        top = torch.topk(logits, cfg.sample_topk, dim=-1)
+        masked = torch.full_like(logits, torch.finfo(torch.float32).min)
+        logits = masked.scatter(-1, top.indices, top.values)
+    probs = torch.softmax(logits, dim=-1)
+    return torch.multinomial(probs, 1, generator=generator)[:, 0].to(torch.int32)
+
+
+def generate(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig,
+             generator: torch.Generator | None = None) -> tuple[torch.Tensor, ModelCache]:
+    """lyra/generate.py:56-61 for a batch of sequences, one new token each: tokens [B] -> next tokens [B]."""
+    logits, cache = model_apply(tokens, model, cache, cfg)
+    return sample_token(logits, cfg, generator), cache
+
+
+class GraphedDecoder:
+    """One decode step captured in a HIP graph: the per-token host work collapses to one graph launch.
+
+    The reference jits the step (lyra/generate.py:119-125); here every kernel of the step is recorded once and
+    replayed.  Token ids are read from / written to fixed device buffers.
+    """
+
+    def __init__(self, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, batch: int, warmup: int = 2):
+        self.cfg, self.model, self.cache = cfg, model, cache
+        dev = model.emb.device
+        self.tokens = torch.zeros(batch, dtype=torch.int64, device=dev)
+        self.next_tokens = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.graph = torch.cuda.CUDAGraph()
+        stream = torch.cuda.Stream(device=dev)
+        stream.wait_stream(torch.cuda.current_stream(dev))
+        start_pos = cache.pos.clone()
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):  # allocates workspaces and warms caches outside the capture
+                self._step()
+            cache.pos.copy_(start_pos)
+            with torch.cuda.graph(self.graph, stream=stream):
+                self._step()
+            cache.pos.copy_(start_pos)
+        torch.cuda.current_stream(dev).wait_stream(stream)
+
+    def _step(self):
+        logits, _ = model_apply(self.tokens, self.model, self.cache, self.cfg)
+        self.logits = logits
+        self.next_tokens.copy_(torch.argmax(logits, dim=-1))
+
+    def step(self) -> torch.Tensor:
+        """Run one decode step on ``self.tokens``; returns the greedy next tokens (device, int32)."""
+        self.graph.replay()
+        return self.next_tokens

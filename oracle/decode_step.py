@@ -1,0 +1,148 @@
+"""CPU restatement of one decode step of the reference model (lyra/model.py:734-793 in Mode.DECODE).
+
+TEST INFRASTRUCTURE ONLY (parity checker for lyra_amd.model and the timed CPU baseline of bench.py).
+It chains the oracle pieces exactly in the order the reference calls them:
+embedding -> per layer [attention_apply (model.py:284-374), mlp_apply (:498-567 / :608-636)] -> final norm ->
+LM head.  bf16 arrays are float32 arrays holding bf16-representable values; every point where the JAX code
+holds a bf16 array is rounded with ``bf16_round``.  The heavy contractions (attention, grouped matmul) run in
+the threaded C restatement when ``use_c`` is set (bench baseline, large parity cases), else in NumPy.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from oracle import clib
+from oracle import lyra_oracle as O
+
+R = O.bf16_round
+
+
+def _gemm(lhs, w, sizes, *, swiglu=False, beta=1.702, limit=7.0, use_c=False, out_bf16=True):
+    """decode_gemm / quant.dot: w is float32 [G,K,N] (bf16 weights) or (qval, scale, block)."""
+    if isinstance(w, tuple):
+        q, s, block = w
+        if use_c:
+            y = clib.decode_gemm(O.bf16_bits(lhs), q, s, block, sizes, None, fused_swiglu=swiglu, beta=beta, limit=limit, ref_rounding=True)
+        else:
+            y = O.decode_gemm_reference(lhs, (q, s), sizes, block=block, fused_swiglu=swiglu, swiglu_beta=beta, swiglu_limit=limit, mode="ref")
+    else:
+        if use_c:
+            y = clib.decode_gemm(O.bf16_bits(lhs), O.bf16_bits(w), None, None, sizes, None, fused_swiglu=swiglu, beta=beta, limit=limit, ref_rounding=out_bf16)
+        else:
+            y = O.decode_gemm_reference(lhs, w, sizes, fused_swiglu=swiglu, swiglu_beta=beta, swiglu_limit=limit, mode="ref" if out_bf16 else "fp32")
+    return y
+
+
+def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False):
+    """tokens [B] int; weights/cache: dicts of NumPy arrays mirroring lyra_amd.model; pos: int.
+
+    cache["k"][l], cache["v"][l]: float32 [B,K,S,H] (bf16 cache) or (qval uint8, scale f32 [B,K,S,1]); updated in
+    place.  Returns float32 logits [B, padded_vocab] with -inf beyond vocab_size.
+    """
+    B = tokens.shape[0]
+    C, H, N, K = cfg.n_embd, cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
+    cos_t, sin_t = O.rope_tables(cfg.seq_len, H, cfg.rope_base, cfg.rope_scale, cfg.ntk_alpha, cfg.ntk_beta)
+    cos, sin = cos_t[pos], sin_t[pos]
+    one = np.array([B], np.int32)
+    h = R(weights["emb"][tokens])
+    for idx, lw in enumerate(weights["layers"]):
+        # ---- attention_apply ----
+        a = lw["attn"]
+        hn = R(O.rms_norm(h, a["norm_scale"], cfg.norm_eps))
+        qkv = _gemm(hn, a["qkv"], one, use_c=use_c)
+        q, k, v = np.split(qkv, [N * H, (N + K) * H], axis=-1)
+        q, k, v = q.reshape(B, N, H), k.reshape(B, K, H), v.reshape(B, K, H)
+        if a["qnorm_scale"] is not None:
+            q = R(O.rms_norm(q, a["qnorm_scale"], cfg.norm_eps))
+            k = R(O.rms_norm(k, a["knorm_scale"], cfg.norm_eps))
+        q, k = R(O.rotate(q, cos, sin)), R(O.rotate(k, cos, sin))
+        ck, cv = cache["k"][idx], cache["v"][idx]
+        if isinstance(ck, tuple):  # qupdate: quantise the new token with block (1, H) and write it at pos
+            for (cq, cs), new in ((ck, k), (cv, v)):
+                nq, ns = O.quantize(new[:, :, None, :], (1, H))
+                cq[:, :, pos : pos + 1] = nq
+                cs[:, :, pos : pos + 1] = ns
+        else:
+            ck[:, :, pos] = k
+            cv[:, :, pos] = v
+        sw = cfg.sliding_window if idx % 2 == 0 else 0
+        gate = None
+        if a["sdpa_gate"] is not None:
+            gate = R((2.0 / (1.0 + np.exp(-(hn.astype(np.float32) @ a["sdpa_gate"])))).astype(np.float32))
+        if use_c:
+            if isinstance(ck, tuple):
+                t = clib.decode_attention(O.bf16_bits(q[:, :, None, :]), ck[0], cv[0], ck[1][..., 0], cv[1][..., 0], a["sinks"],
+                                          pos, gate, H**-0.5, sw, ref_rounding=True)
+            else:
+                t = clib.decode_attention(O.bf16_bits(q[:, :, None, :]), O.bf16_bits(ck), O.bf16_bits(cv), None, None, a["sinks"],
+                                          pos, gate, H**-0.5, sw, ref_rounding=True)
+        else:
+            t = O.decode_attention_reference(q[:, :, None, :], ck, cv, a["sinks"], H**-0.5, sw, pos, mode="ref", gate=gate)
+        t = _gemm(R(t.reshape(B, N * H)), a["out"], one, use_c=use_c)
+        t = R(t * np.float32(cfg.residual_scale))
+        h = R(h + t)
+        # ---- mlp_apply ----
+        m = lw["mlp"]
+        xn = R(O.rms_norm(h, m["norm_scale"], cfg.norm_eps))
+        if "router" in m:
+            logits = xn.astype(np.float32) @ m["router"]
+            if m["router_bias"] is not None:
+                logits = logits + m["router_bias"]
+            scores, active_map, groups = O.route_tokens(logits, cfg.n_active_routed_experts, cfg.n_routed_experts, cfg.n_shared_experts)
+            topk = cfg.n_active_experts
+            perm, dest = O.bpermute(active_map, groups, cfg.n_experts)
+            t = xn[perm // topk]
+            t = _gemm(t, m["mlp_up"], groups, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c)
+            t = _gemm(R(t), m["mlp_down"], groups, use_c=use_c)
+            t = R(O.combine(R(t), scores, dest))
+            t = R(t * np.float32(cfg.residual_scale))
+            h = R(h + t)
+        else:
+            t = _gemm(xn, m["mlp_up"], one, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c)
+            t = _gemm(R(t), m["mlp_down"], one, use_c=use_c)
+            t = R(t * np.float32(cfg.dense_residual_scale))
+            h = R(h + t)
+    h = R(O.rms_norm(h, weights["norm_scale"], cfg.norm_eps))
+    logits = _gemm(h, weights["unemb_t"], one, use_c=use_c, out_bf16=False)
+    logits[:, cfg.vocab_size :] = -np.inf
+    return logits
+
+
+def weights_to_numpy(model, cfg):
+    """lyra_amd.model.ModelWeights (torch) -> the dict layout decode_step takes."""
+    import torch
+
+    from lyra_amd.nn.quant import QArray
+
+    def conv(w):
+        if isinstance(w, QArray):
+            return (w.qval.view(torch.uint8).cpu().numpy(), w.scale.float().cpu().numpy(), tuple(w.block))
+        return w.float().cpu().numpy()
+
+    f = lambda t: None if t is None else t.float().cpu().numpy()
+    layers = []
+    for lw in model.layers:
+        a = lw.attn
+        attn = dict(qkv=conv(a.qkv), out=conv(a.out), sinks=f(a.sinks), norm_scale=f(a.norm_scale), qnorm_scale=f(a.qnorm_scale),
+                    knorm_scale=f(a.knorm_scale), sdpa_gate=f(a.sdpa_gate))
+        m = lw.mlp
+        mlp = dict(mlp_up=conv(m.mlp_up), mlp_down=conv(m.mlp_down), norm_scale=f(m.norm_scale))
+        if hasattr(m, "router"):
+            mlp.update(router=f(m.router), router_bias=f(m.router_bias))
+        layers.append(dict(attn=attn, mlp=mlp))
+    return dict(emb=f(model.emb), unemb_t=f(model.unemb_t), norm_scale=f(model.norm_scale), layers=layers)
+
+
+def cache_to_numpy(cache):
+    import torch
+
+    from lyra_amd.nn.quant import QArray
+
+    def conv(c):
+        if isinstance(c, QArray):
+            return (c.qval.view(torch.uint8).cpu().numpy().copy(), c.scale.float().cpu().numpy().copy())
+        return c.float().cpu().numpy().copy()
+
+    return dict(k=[conv(l.k) for l in cache.layers], v=[conv(l.v) for l in cache.layers])
