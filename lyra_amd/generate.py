@@ -45,6 +45,7 @@ class GraphedDecoder:
         start_pos = cache.pos.clone()
         with torch.cuda.stream(stream):
             for _ in range(warmup):  # allocates workspaces and warms caches outside the capture
+                cache.pos.copy_(start_pos)  # (always at the caller's position: it may be the last cache row)
                 self._step()
             cache.pos.copy_(start_pos)
             with torch.cuda.graph(self.graph, stream=stream):
