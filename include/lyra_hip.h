@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 2
+#define LYRA_ABI_VERSION 3
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -101,6 +101,64 @@ int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, i
                      int fused_swiglu, float swiglu_beta, float swiglu_limit, lyra_stream_t stream);
 
 size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu);
+
+/*
+ * lyra_decode_gemm with the two neighbouring model steps fused in (no counterpart kernel in the reference; the
+ * model code around its two matmul call sites, lyra/model.py:371-374, 536-567, 631-636):
+ *   lhs_row_map [M] int32 or NULL: sorted row r reads lhs[lhs_row_map[r], :] - the token gather that feeds the
+ *               expert up-projection (x[permute_map // topk], model.py:536-540); lhs then has as many rows as
+ *               the map addresses.
+ *   post_scale  != 0: out = bf16(residual + bf16(bf16(t) * out_scale)), t the plain result - a projection's
+ *               output scaled in bf16 and added to the residual stream; residual [M,N] bf16 or NULL (scale only).
+ *               residual requires post_scale and a bf16 output.
+ */
+int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
+                        int bn, const int32_t* group_sizes, const float* bias, const void* residual, float out_scale,
+                        int post_scale, void* out, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
+                        int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
+                        lyra_stream_t stream);
+
+/*
+ * The elementwise steps of a decode layer between the two kernels above, one launch each.  They follow the
+ * reference's dtype flow exactly: float32 arithmetic inside an op, a bf16 rounding wherever its JAX code holds a
+ * bf16 array.
+ *
+ * lyra_rmsnorm_proj: h = bf16(x * rsqrt(mean(x^2) + eps) * scale) (lyra/model.py:189-191), optionally followed by a
+ *   narrow float32 projection of f32(h): y = h @ proj (+ bias), proj [C,n] float32.
+ *   mode 1: y -> bf16(2 * sigmoid(y)), the per-head output gate (model.py:343-347), y is bf16 [B,n];
+ *   mode 2: y float32 [B,n], the router logits (model.py:455-457).  proj NULL: norm only.
+ */
+int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj, const float* bias, void* y, int B, int C,
+                      int n, int mode, float eps, lyra_stream_t stream);
+
+/*
+ * lyra_qkv_post: everything between the fused q/k/v projection and the attention kernel (model.py:309-336):
+ *   qkv [B,(N+2K)*H] bf16 -> per head rms_norm (qnorm/knorm [H] float32, both NULL = no QK norm) -> half-split
+ *   rotary embedding with row position[b] of cos_t/sin_t [rope_rows, H/2] float32 (model.py:183-186) -> q_out
+ *   [B,N,H] bf16; k and v rows are appended to the caches [B,K,S,H] at index position[b]: copied (bf16) or
+ *   quantised with one scale per row, scale = amax/448 (1 for a zero row), code = e4m3fn_rne(clip(x/scale))
+ *   (lyra/nn/quant.py:68-72, 213-231), scales into k_scale/v_scale [B,K,S].  Rows with position outside [0,S)
+ *   are not appended.  H in {64,128}.
+ */
+int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,
+                  const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache, float* k_scale,
+                  float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype, float eps,
+                  lyra_stream_t stream);
+
+/*
+ * lyra_moe_route: router top-k, softmax over the chosen logits, shared experts appended with score 1, and the stable
+ * sort of assignments by expert (model.py:459-491, 393-417).  logits [tokens,n_routed] float32 ->
+ *   scores [tokens,topk] float32, groups [E] int32 (rows per expert), row_map [tokens*topk] int32 (token of each
+ *   sorted row = permute_map // topk), dest [tokens*topk] int32 (sorted row of each assignment = unpermute_map);
+ *   topk = k_routed + n_shared, E = n_routed + n_shared.  k_routed <= 8, n_routed <= 128.
+ *
+ * lyra_moe_combine: out[f] = bf16(x[f] + bf16(bf16(sum_k scores[f,k] * rows[dest[f*topk+k]]) * residual_scale))
+ *   (model.py:557-567); rows [tokens*topk,C] bf16 in sorted order, x/out [tokens,C] bf16.
+ */
+int lyra_moe_route(const float* logits, float* scores, int32_t* groups, int32_t* row_map, int32_t* dest, int tokens,
+                   int n_routed, int n_shared, int k_routed, lyra_stream_t stream);
+int lyra_moe_combine(const void* rows, const float* scores, const int32_t* dest, const void* x, void* out, int tokens, int topk,
+                     int C, float residual_scale, lyra_stream_t stream);
 
 /*
  * Self-check of the matrix-core register layouts and FP8 conversions the kernels rely on.

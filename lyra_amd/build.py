@@ -8,7 +8,7 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
-SOURCES = ("abi.hip", "decode_attention.hip", "decode_gemm.hip")
+SOURCES = ("abi.hip", "decode_attention.hip", "decode_gemm.hip", "decode_fused.hip")
 HIPCC_FLAGS = (
     "--offload-arch=gfx950",
     "-O3",

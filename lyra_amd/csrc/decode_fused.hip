@@ -1,0 +1,319 @@
+// Small fused kernels around the two decode hot kernels: everything the reference's model code does between
+// them for one new token per sequence (lyra/model.py:284-374, 451-567), so that a decode step is a few launches
+// per layer instead of hundreds of elementwise ones.  All arithmetic follows the reference's dtype flow: bf16
+// activations, float32 maths inside an op, a bf16 rounding wherever the JAX code holds a bf16 array.
+#include <algorithm>
+
+#include "lyra_device.h"
+
+namespace lyra {
+
+__device__ __forceinline__ float bf16r(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ float block_sum(float v, float* sm) {  // blockDim.x <= 1024, multiple of 64
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) sm[wave] = v;
+    __syncthreads();
+    float t = lane < nw ? sm[lane] : 0.f;
+    return wave_sum(t);
+}
+
+// ---- RMS norm (+ a narrow float32 projection of the normalised row) ---------------------------------------
+// h = bf16(x * rsqrt(mean(x^2) + eps) * scale)                      lyra/model.py:189-191
+// y[j] = sum_c f32(h[c]) * P[c, j] (+ bias[j]), j < n                router logits (model.py:455-457) or the
+// gate = bf16(2 * sigmoid(y))                                        output gate (model.py:343-347)
+struct NormProjParams {
+    const uint16_t* x;
+    const float* scale;
+    uint16_t* h;
+    const float* proj;  // [C, n] or null
+    const float* bias;  // [n] or null
+    void* y;            // mode 1: bf16 [B, n] gate; mode 2: float32 [B, n]
+    int C, n, mode;
+    float eps;
+};
+
+__global__ __launch_bounds__(256) void rmsnorm_proj_kernel(NormProjParams p) {
+    __shared__ float sm[64];
+    const int b = blockIdx.x;
+    const uint16_t* xr = p.x + (size_t)b * p.C;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
+        const float v = bf16_bits_to_f32(xr[c]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, sm);
+    const float inv = rsqrtf(ss / (float)p.C + p.eps);
+    for (int c = threadIdx.x; c < p.C; c += blockDim.x)
+        p.h[(size_t)b * p.C + c] = f32_to_bf16_bits(bf16_bits_to_f32(xr[c]) * inv * p.scale[c]);
+    if (!p.proj) return;
+    for (int j0 = 0; j0 < p.n; j0 += 16) {  // 16 output columns per sweep over the row
+        float acc[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+        for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
+            const float hv = bf16r(bf16_bits_to_f32(xr[c]) * inv * p.scale[c]);
+            const float* pr = p.proj + (size_t)c * p.n + j0;
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                if (j0 + j < p.n) acc[j] += hv * pr[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if (j0 + j >= p.n) break;
+            float v = block_sum(acc[j], sm);
+            if (threadIdx.x == 0) {
+                if (p.bias) v += p.bias[j0 + j];
+                const size_t o = (size_t)b * p.n + j0 + j;
+                if (p.mode == 1) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(2.f / (1.f + __expf(-v)));
+                else ((float*)p.y)[o] = v;
+            }
+        }
+    }
+}
+
+// ---- after the q/k/v projection: QK norm, RoPE, KV-cache append (quantised) ---------------------------------
+// One wavefront per (batch row, head).  Lane i holds elements i and i + H/2 of the head: exactly the pair the
+// half-split rotary embedding mixes (lyra/model.py:183-186).
+//   q, k: rms_norm over the head (model.py:315-320) -> bf16 -> rotate -> bf16
+//   k, v: written at `position` into the cache; FP8 caches quantise the row with block (1, H):
+//         scale = amax / 448 (1 if the row is zero), code = fp8_rne(clip(x / scale))   (lyra/nn/quant.py:68-72)
+struct QkvPostParams {
+    const uint16_t* qkv;  // [B, (N + 2K) * H]
+    const float* qnorm;   // [H] or null
+    const float* knorm;
+    const float* cos_t;   // [seq, H/2]
+    const float* sin_t;
+    const int32_t* position;
+    int pos_stride;
+    uint16_t* q_out;      // [B, N, H]
+    void* k_cache;        // [B, K, S, H]
+    void* v_cache;
+    float* k_scale;       // [B, K, S] or null (bf16 cache)
+    float* v_scale;
+    int B, N, K, S, H, seq;
+    float eps;
+};
+
+__device__ __forceinline__ uint8_t f32_to_e4m3fn(float v) {  // round to nearest even; |v| <= 448 by construction
+    const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false);
+    return (uint8_t)(packed & 0xFF);
+}
+
+__global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, head) over N + 2K heads
+    const int heads = p.N + 2 * p.K;
+    if (item >= p.B * heads) return;
+    const int b = item / heads, hd = item - b * heads;
+    const int half = p.H >> 1;
+    const bool active = lane < half;
+    const uint16_t* src = p.qkv + ((size_t)b * heads + hd) * p.H;
+    float a = active ? bf16_bits_to_f32(src[lane]) : 0.f;
+    float c = active ? bf16_bits_to_f32(src[lane + half]) : 0.f;
+    const int pos = p.position[(size_t)b * p.pos_stride];
+    const bool is_q = hd < p.N, is_k = !is_q && hd < p.N + p.K;
+    if (is_q || is_k) {
+        const float* ns = is_q ? p.qnorm : p.knorm;
+        if (ns) {
+            const float ss = wave_sum(a * a + c * c);
+            const float inv = rsqrtf(ss / (float)p.H + p.eps);
+            a = bf16r(a * inv * (active ? ns[lane] : 0.f));
+            c = bf16r(c * inv * (active ? ns[lane + half] : 0.f));
+        }
+        const int rp = min(max(pos, 0), p.seq - 1);
+        const float cs = active ? p.cos_t[(size_t)rp * half + lane] : 0.f;
+        const float sn = active ? p.sin_t[(size_t)rp * half + lane] : 0.f;
+        const float ra = bf16r(a * cs - c * sn), rc = bf16r(c * cs + a * sn);
+        a = ra;
+        c = rc;
+    }
+    if (is_q) {
+        if (active) {
+            uint16_t* dst = p.q_out + ((size_t)b * p.N + hd) * p.H;
+            dst[lane] = f32_to_bf16_bits(a);
+            dst[lane + half] = f32_to_bf16_bits(c);
+        }
+        return;
+    }
+    if (pos < 0 || pos >= p.S) return;  // nothing to append outside the cache
+    const int kh = is_k ? hd - p.N : hd - p.N - p.K;
+    const size_t row = ((size_t)b * p.K + kh) * p.S + pos;
+    void* cache = is_k ? p.k_cache : p.v_cache;
+    float* scales = is_k ? p.k_scale : p.v_scale;
+    if (scales) {
+        const float amax = wave_max(fmaxf(fabsf(a), fabsf(c)));
+        const float scale = amax > 0.f ? amax / 448.f : 1.f;
+        const float inv = 1.0f / scale;
+        if (active) {
+            uint8_t* dst = (uint8_t*)cache + row * p.H;
+            dst[lane] = f32_to_e4m3fn(fminf(fmaxf(a * inv, -448.f), 448.f));
+            dst[lane + half] = f32_to_e4m3fn(fminf(fmaxf(c * inv, -448.f), 448.f));
+        }
+        if (lane == 0) scales[row] = scale;
+    } else if (active) {
+        uint16_t* dst = (uint16_t*)cache + row * p.H;
+        dst[lane] = f32_to_bf16_bits(a);
+        dst[lane + half] = f32_to_bf16_bits(c);
+    }
+}
+
+// ---- MoE routing: top-k, softmax, shared experts, stable counting sort ------------------------------------
+// lyra/model.py:459-491.  One workgroup; thread t < tokens routes token t, then every assignment finds its
+// destination row: start of its expert's rows + number of earlier assignments to the same expert.
+struct RouteParams {
+    const float* logits;  // [tokens, n_routed] (bias already added)
+    float* scores;        // [tokens, topk]
+    int32_t* groups;      // [E]
+    int32_t* row_map;     // [tokens * topk]: token of each sorted row   (permute_map // topk)
+    int32_t* dest;        // [tokens * topk]: sorted row of each assignment (unpermute_map)
+    int tokens, n_routed, n_shared, k_routed;
+};
+
+__global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
+    extern __shared__ int sm_i[];
+    const int topk = p.k_routed + p.n_shared, E = p.n_routed + p.n_shared, M = p.tokens * topk;
+    int* sm_expert = sm_i;        // [M]
+    int* sm_count = sm_i + M;     // [E]
+    int* sm_start = sm_count + E; // [E]
+    for (int e = threadIdx.x; e < E; e += blockDim.x) sm_count[e] = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < p.tokens; t += blockDim.x) {
+        const float* lg = p.logits + (size_t)t * p.n_routed;
+        float top[8];
+        int idx[8];
+        unsigned long long taken_lo = 0ull, taken_hi = 0ull;  // up to 128 routed experts
+        for (int j = 0; j < p.k_routed; ++j) {
+            float best = -INFINITY;
+            int bi = -1;
+            for (int e = 0; e < p.n_routed; ++e) {
+                const bool used = e < 64 ? (taken_lo >> e) & 1ull : (taken_hi >> (e - 64)) & 1ull;
+                const float v = lg[e];
+                if (!used && (bi < 0 || v > best)) {  // strict >: ties go to the lower index (lax.top_k)
+                    best = v;
+                    bi = e;
+                }
+            }
+            if (bi < 64) taken_lo |= 1ull << bi; else taken_hi |= 1ull << (bi - 64);
+            top[j] = best;
+            idx[j] = bi;
+        }
+        float den = 0.f;
+        const float top_max = top[0];
+        for (int j = 0; j < p.k_routed; ++j) {
+            top[j] = __expf(top[j] - top_max);
+            den += top[j];
+        }
+        for (int j = 0; j < p.k_routed; ++j) {
+            p.scores[(size_t)t * topk + j] = top[j] / den;
+            sm_expert[t * topk + j] = idx[j];
+            atomicAdd(&sm_count[idx[j]], 1);
+        }
+        for (int s = 0; s < p.n_shared; ++s) {
+            p.scores[(size_t)t * topk + p.k_routed + s] = 1.f;  // model.py:476
+            sm_expert[t * topk + p.k_routed + s] = p.n_routed + s;
+            atomicAdd(&sm_count[p.n_routed + s], 1);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            sm_start[e] = run;
+            run += sm_count[e];
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) p.groups[e] = sm_count[e];
+    for (int i = threadIdx.x; i < M; i += blockDim.x) {
+        const int e = sm_expert[i];
+        int rank = 0;
+        for (int j = 0; j < i; ++j) rank += sm_expert[j] == e;
+        const int d = sm_start[e] + rank;
+        p.dest[i] = d;
+        p.row_map[d] = i / topk;
+    }
+}
+
+// ---- MoE combine + residual --------------------------------------------------------------------------------
+// out[f] = bf16(x[f] + bf16(bf16(sum_k scores[f,k] * rows[dest[f*topk + k]]) * residual_scale))   model.py:557-567
+struct CombineParams {
+    const uint16_t* rows;   // [M, C] expert outputs in sorted order
+    const float* scores;    // [tokens, topk]
+    const int32_t* dest;    // [tokens * topk]
+    const uint16_t* x;      // [tokens, C] residual stream
+    uint16_t* out;          // [tokens, C]
+    int tokens, topk, C;
+    float residual_scale;
+};
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
+    const int f = blockIdx.x;
+    for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < p.topk; ++k) {
+            const int r = p.dest[f * p.topk + k];
+            acc += bf16_bits_to_f32(p.rows[(size_t)r * p.C + c]) * p.scores[f * p.topk + k];
+        }
+        const float t = bf16r(bf16r(acc) * p.residual_scale);
+        p.out[(size_t)f * p.C + c] = f32_to_bf16_bits(bf16_bits_to_f32(p.x[(size_t)f * p.C + c]) + t);
+    }
+}
+
+}  // namespace lyra
+
+extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj, const float* bias, void* y,
+                                 int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!x || !scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
+    if (proj && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj, bias, y, C, proj ? n : 0, mode, eps};
+    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,
+                             const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache,
+                             float* k_scale, float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype,
+                             float eps, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!qkv || !cos_t || !sin_t || !position || !q_out || !k_cache || !v_cache) return LYRA_E_BADARG;
+    if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || rope_rows <= 0) return LYRA_E_BADARG;
+    if (H != 64 && H != 128) return LYRA_E_UNSUPPORTED;
+    if ((qnorm == nullptr) != (knorm == nullptr)) return LYRA_E_BADARG;
+    const bool fp8 = kv_dtype == LYRA_DTYPE_E4M3FN;
+    if (!fp8 && kv_dtype != LYRA_DTYPE_BF16) return LYRA_E_UNSUPPORTED;
+    if (fp8 != (k_scale != nullptr) || fp8 != (v_scale != nullptr)) return LYRA_E_BADARG;
+    if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
+    QkvPostParams p{(const uint16_t*)qkv, qnorm, knorm, cos_t, sin_t, position, position_stride, (uint16_t*)q_out,
+                    k_cache, v_cache, k_scale, v_scale, B, N, K, S, H, rope_rows, eps};
+    const int items = B * (N + 2 * K);
+    hipLaunchKernelGGL(qkv_post_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" int lyra_moe_route(const float* logits, float* scores, int32_t* groups, int32_t* row_map, int32_t* dest, int tokens,
+                              int n_routed, int n_shared, int k_routed, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!logits || !scores || !groups || !row_map || !dest) return LYRA_E_BADARG;
+    if (tokens <= 0 || n_routed <= 0 || n_shared < 0 || k_routed <= 0) return LYRA_E_BADARG;
+    if (k_routed > 8 || k_routed > n_routed || n_routed > 128) return LYRA_E_UNSUPPORTED;
+    const int topk = k_routed + n_shared, E = n_routed + n_shared;
+    const size_t lds = ((size_t)tokens * topk + 2 * E) * sizeof(int);
+    if (lds > 60000) return LYRA_E_UNSUPPORTED;
+    RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed};
+    const int threads = std::min(1024, std::max(64, (tokens * topk + 63) / 64 * 64));
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" int lyra_moe_combine(const void* rows, const float* scores, const int32_t* dest, const void* x, void* out, int tokens,
+                                int topk, int C, float residual_scale, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!rows || !scores || !dest || !x || !out || tokens <= 0 || topk <= 0 || C <= 0) return LYRA_E_BADARG;
+    CombineParams p{(const uint16_t*)rows, scores, dest, (const uint16_t*)x, (uint16_t*)out, tokens, topk, C, residual_scale};
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}

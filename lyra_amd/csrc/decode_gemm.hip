@@ -36,7 +36,21 @@ struct GemmParams {
     float beta, limit;
     int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
+    const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
+    const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
+    float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
+    int post_scale;
 };
+
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// Residual epilogue of a projection (lyra/model.py:371-374, 631-636): the product is a bf16 array, it is scaled in
+// bf16, then added to the bf16 residual stream.
+__device__ __forceinline__ float residual_epilogue(const GemmParams& p, float t, size_t idx) {
+    t = round_bf16(round_bf16(t) * p.out_scale);
+    if (p.residual) t += bf16_bits_to_f32(p.residual[idx]);
+    return t;
+}
 
 __device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, float limit) {
     glu = fminf(glu, limit);
@@ -124,6 +138,10 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
         store = store && !is_lin_lane;
     }
     if (store) {
+        if (p.post_scale) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) t[c] = residual_epilogue(p, t[c], (size_t)row * NO + out_col + c);
+        }
         if (p.out_f32) {
             float* dst = (float*)p.out + (size_t)row * NO + out_col;
             *(f32x4*)dst = f32x4{t[0], t[1], t[2], t[3]};
@@ -221,7 +239,10 @@ void decode_gemm_kernel(GemmParams p) {
             if (lane < pieces) {
                 for (int r = wave; r < 16 * n_mt; r += kGemmWaves) {
                     u32x4 d = u32x4{0u, 0u, 0u, 0u};
-                    if (r < rows_here) d = *(const u32x4*)(p.lhs + (size_t)(rowbase + r) * p.K + kc + lane * 8);
+                    if (r < rows_here) {
+                        const int src = p.row_map ? p.row_map[rowbase + r] : rowbase + r;
+                        d = *(const u32x4*)(p.lhs + (size_t)src * p.K + kc + lane * 8);
+                    }
                     *(u32x4*)(sm_x + r * XPITCH + lane * 8) = d;
                 }
             }
@@ -339,6 +360,10 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) a[c] = swiglu_one(a[c], b[c], p.beta, p.limit);
     }
+    if (p.post_scale) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] = residual_epilogue(p, a[c], (size_t)row * NO + col + c);
+    }
     if (p.out_f32) {
         *(f32x4*)((float*)p.out + (size_t)row * NO + col) = f32x4{a[0], a[1], a[2], a[3]};
     } else {
@@ -400,7 +425,17 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
                                 const int32_t* group_sizes, const float* bias, void* out, void* workspace,
                                 size_t workspace_bytes, int M, int G, int K, int N, int rhs_dtype, int out_dtype,
                                 int fused_swiglu, float swiglu_beta, float swiglu_limit, lyra_stream_t stream) {
+    return lyra_decode_gemm_ex(lhs, nullptr, rhs, rhs_scale, bk, bn, group_sizes, bias, nullptr, 1.0f, 0, out, workspace,
+                               workspace_bytes, M, G, K, N, rhs_dtype, out_dtype, fused_swiglu, swiglu_beta, swiglu_limit, stream);
+}
+
+extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
+                                   int bn, const int32_t* group_sizes, const float* bias, const void* residual, float out_scale,
+                                   int post_scale, void* out, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
+                                   int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
+                                   lyra_stream_t stream) {
     using namespace lyra;
+    if (residual && (!post_scale || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
     if (!lhs || !rhs || !group_sizes || !out) return LYRA_E_BADARG;
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
     if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
@@ -439,6 +474,10 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
     p.ksplit = pl.ksplit;
     p.row_par = pl.row_par;
     p.kpart = pl.kpart;
+    p.row_map = lhs_row_map;
+    p.residual = (const uint16_t*)residual;
+    p.out_scale = out_scale;
+    p.post_scale = post_scale != 0;
     if (pl.ksplit > 1) {
         const size_t need = ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
         if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;

@@ -1,0 +1,140 @@
+"""Host wrappers of the fused decode-step kernels (include/lyra_hip.h: lyra_rmsnorm_proj, lyra_qkv_post,
+lyra_decode_gemm_ex, lyra_moe_route, lyra_moe_combine).
+
+The reference leaves these steps to XLA fusion inside its jitted decode step (lyra/model.py:284-374, 451-567,
+608-636); here each is one HIP launch.  Every function takes and returns torch device tensors and launches on the
+current stream, so a whole decode step can be captured in a HIP graph.
+"""
+from __future__ import annotations
+
+import torch
+
+from lyra_amd import _lib
+from lyra_amd.nn.quant import QArray
+
+_L = _lib.lib
+
+
+def _stream(dev) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _f32(t):
+    assert t.dtype == torch.float32 and t.is_contiguous()
+    return t
+
+
+def rmsnorm_proj(x: torch.Tensor, scale: torch.Tensor, eps: float, proj: torch.Tensor | None = None,
+                 bias: torch.Tensor | None = None, gate: bool = False):
+    """rms_norm (lyra/model.py:189-191) of x [B,C] bf16; with ``proj`` [C,n] f32 also f32(h) @ proj (+ bias) as
+    float32 logits, or bf16 ``2*sigmoid`` gates when ``gate`` is set (model.py:343-347).  Returns (h, y | None)."""
+    B, C = x.shape
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    h = torch.empty_like(x)
+    y, n = None, 0
+    if proj is not None:
+        n = proj.shape[1]
+        y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=x.device)
+        _f32(proj)
+    rc = _L.lyra_rmsnorm_proj(x.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
+                              1 if gate else 2, float(eps), _stream(x.device))
+    _lib.check(rc, "lyra_rmsnorm_proj")
+    return h, y
+
+
+def qkv_post(qkv: torch.Tensor, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
+             n_heads: int, n_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
+    """QK norm + rotary embedding + KV-cache append (quantising for an FP8 cache) for one new token per sequence
+    (lyra/model.py:309-336); ``pos`` is an int32 device scalar or a [B] tensor.  Returns q [B,N,H] bf16; the caches
+    are updated in place."""
+    B = qkv.shape[0]
+    N, K, H = n_heads, n_kv_heads, head_dim
+    assert qkv.dtype == torch.bfloat16 and qkv.is_contiguous() and qkv.shape[1] == (N + 2 * K) * H
+    assert pos.dtype == torch.int32
+    q = torch.empty((B, N, H), dtype=torch.bfloat16, device=qkv.device)
+    fp8 = isinstance(cache_k, QArray)
+    if fp8:
+        assert tuple(cache_k.block) == (1, H) and cache_k.scale.dtype == torch.float32
+        kq, vq, ks, vs = cache_k.qval, cache_v.qval, cache_k.scale, cache_v.scale
+        S = kq.shape[2]
+    else:
+        kq, vq, ks, vs = cache_k, cache_v, None, None
+        S = kq.shape[2]
+        assert kq.dtype == torch.bfloat16
+    assert kq.is_contiguous() and vq.is_contiguous() and tuple(kq.shape) == (B, K, S, H)
+    rc = _L.lyra_qkv_post(qkv.data_ptr(), _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(), _f32(sin_t).data_ptr(), pos.data_ptr(),
+                          0 if pos.numel() == 1 else 1, q.data_ptr(), kq.data_ptr(), vq.data_ptr(), _ptr(ks), _ptr(vs),
+                          B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
+                          _stream(qkv.device))
+    _lib.check(rc, "lyra_qkv_post")
+    return q
+
+
+def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,
+         residual: torch.Tensor | None = None, out_scale: float | None = None, fused_swiglu: bool = False,
+         swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False) -> torch.Tensor:
+    """lyra_decode_gemm_ex: the decode grouped matmul with an optional row gather on the input and an optional
+    ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray."""
+    dev = lhs.device
+    G, K, N = rhs.shape
+    M = rows if rows is not None else lhs.shape[0]
+    assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
+    assert group_sizes.dtype == torch.int32 and group_sizes.numel() == G
+    if isinstance(rhs, QArray):
+        bk, bn = rhs.block
+        rv, rs, rd = rhs.qval, _f32(rhs.scale), _lib.DTYPE_E4M3FN
+    else:
+        assert rhs.dtype == torch.bfloat16
+        bk = bn = 0
+        rv, rs, rd = rhs, None, _lib.DTYPE_BF16
+    assert rv.is_contiguous()
+    NO = N // 2 if fused_swiglu else N
+    out = torch.empty((M, NO), dtype=torch.float32 if out_f32 else torch.bfloat16, device=dev)
+    if residual is not None:
+        assert residual.dtype == torch.bfloat16 and residual.is_contiguous() and tuple(residual.shape) == (M, NO)
+    if row_map is not None:
+        assert row_map.dtype == torch.int32 and row_map.numel() >= M
+    stream = _stream(dev)
+    need = _L.lyra_decode_gemm_workspace(M, G, K, N, int(fused_swiglu))
+    ws = _lib.workspace("gemm", dev, stream, need)
+    rc = _L.lyra_decode_gemm_ex(lhs.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), None,
+                                _ptr(residual), 1.0 if out_scale is None else float(out_scale), int(out_scale is not None),
+                                out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
+                                _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
+                                float(swiglu_limit), stream)
+    _lib.check(rc, "lyra_decode_gemm_ex")
+    return out
+
+
+def moe_route(logits: torch.Tensor, n_routed: int, n_shared: int, k_routed: int):
+    """Router top-k + softmax + shared experts + stable sort by expert (lyra/model.py:459-491).
+    Returns (scores [T,topk] f32, groups [E] i32, row_map [T*topk] i32, dest [T*topk] i32)."""
+    T = logits.shape[0]
+    assert logits.dtype == torch.float32 and logits.is_contiguous() and logits.shape[1] == n_routed
+    topk, E = k_routed + n_shared, n_routed + n_shared
+    dev = logits.device
+    scores = torch.empty((T, topk), dtype=torch.float32, device=dev)
+    groups = torch.empty(E, dtype=torch.int32, device=dev)
+    row_map = torch.empty(T * topk, dtype=torch.int32, device=dev)
+    dest = torch.empty(T * topk, dtype=torch.int32, device=dev)
+    rc = _L.lyra_moe_route(logits.data_ptr(), scores.data_ptr(), groups.data_ptr(), row_map.data_ptr(), dest.data_ptr(), T,
+                           n_routed, n_shared, k_routed, _stream(dev))
+    _lib.check(rc, "lyra_moe_route")
+    return scores, groups, row_map, dest
+
+
+def moe_combine(rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, x: torch.Tensor, residual_scale: float) -> torch.Tensor:
+    """x + bf16(bf16(sum_k scores[f,k] * rows[dest[f,k]]) * residual_scale)  (lyra/model.py:557-567)."""
+    T, C = x.shape
+    topk = scores.shape[1]
+    assert rows.dtype == torch.bfloat16 and rows.is_contiguous() and tuple(rows.shape) == (T * topk, C)
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    out = torch.empty_like(x)
+    rc = _L.lyra_moe_combine(rows.data_ptr(), _f32(scores).data_ptr(), dest.data_ptr(), x.data_ptr(), out.data_ptr(), T, topk, C,
+                             float(residual_scale), _stream(x.device))
+    _lib.check(rc, "lyra_moe_combine")
+    return out

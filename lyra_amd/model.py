@@ -72,6 +72,7 @@ class ModelConfig:
     per_channel_scales: bool = False  # FP8 weights with one scale per output channel (block (K, 1)) instead of quant_block
     mode: Mode = Mode.DECODE
     implementation: Implementation = "auto"
+    fused_glue: bool = True  # run norms, RoPE, cache append, routing and residual adds as fused HIP launches
     sample_topk: int = 4
     sample_temperature: float = 0.8
     norm_eps: float = 1e-5
@@ -384,8 +385,88 @@ def dense_mlp_apply(x, w: DenseMLPWeights, cfg: ModelConfig):
     return (x + t).to(x.dtype)
 
 
+# ---- the same layers with every step between the two hot kernels as one fused HIP launch --------------------
+def _one_group(rows: int, device) -> torch.Tensor:
+    key = (rows, str(device))
+    if key not in _ONE_GROUP:
+        _ONE_GROUP[key] = torch.full((1,), rows, dtype=torch.int32, device=device)
+    return _ONE_GROUP[key]
+
+
+_ONE_GROUP: dict = {}
+
+
+def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
+    """attention_apply as 5-7 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append | attention |
+    output matmul with the scaled residual add in its epilogue."""
+    from lyra_amd.kernels import decode_fused as F
+
+    B = x.shape[0]
+    H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
+    one = _one_group(B, x.device)
+    h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+    qkv = F.gemm(h, w.qkv, one)
+    q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps)
+    sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
+    attn = attn_op(cfg.mode, cfg.implementation)
+    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate)
+    return F.gemm(t.reshape(B, N * H), w.out, one, residual=x, out_scale=cfg.residual_scale), cache
+
+
+def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
+    """moe_apply as norm+router | routing | up matmul (token gather fused) | down matmul | combine+residual."""
+    from lyra_amd.kernels import decode_fused as F
+
+    B = x.shape[0]
+    topk = cfg.n_active_experts
+    xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+    scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
+    t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
+               swiglu_limit=cfg.swiglu_limit)
+    t = F.gemm(t, w.mlp_down, groups)
+    return F.moe_combine(t, scores, dest, x, cfg.residual_scale)
+
+
+def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
+    from lyra_amd.kernels import decode_fused as F
+
+    one = _one_group(x.shape[0], x.device)
+    t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
+    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit)
+    return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)
+
+
+def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
+    """Shapes the fused launches cover (the matmul kernel's: K % 32, N % 128, N % 256 with SwiGLU)."""
+    if not (cfg.fused_glue and cfg.implementation != "xla" and model.emb.is_cuda):
+        return False
+    C, H = cfg.n_embd, cfg.head_dim
+    widths_ok = C % 128 == 0 and ((cfg.n_attn_heads + 2 * cfg.n_kv_heads) * H) % 128 == 0 and (cfg.n_attn_heads * H) % 32 == 0
+    hidden = [cfg.dense_hidden] + ([cfg.expert_hidden] if "moe" in cfg.mlp_map else [])
+    return (widths_ok and H in (64, 128) and all(h % 128 == 0 for h in hidden) and cfg.n_routed_experts <= 128
+            and cfg.n_active_routed_experts <= 8 and cfg.padded_vocab_size % 128 == 0)
+
+
+def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig):
+    from lyra_amd.kernels import decode_fused as F
+
+    h = model.emb[tokens]
+    cos_t, sin_t = _rope_tables(cfg, h.device)
+    pos = cache.pos
+    for idx, layer in enumerate(model.layers):
+        h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
+        h = moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
+    h, _ = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)
+    logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True)
+    logits[:, cfg.vocab_size :] = float("-inf")
+    cache.pos += 1
+    return logits, cache
+
+
 def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig):
     """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one)."""
+    if _fused_supported(model, cfg):
+        return model_apply_fused(tokens, model, cache, cfg)
     h = model.emb[tokens].to(torch.bfloat16)
     cos_t, sin_t = _rope_tables(cfg, h.device)
     pos = cache.pos

@@ -1,0 +1,249 @@
+"""GPU parity of the fused decode-step launches (norm+projection, QK norm + RoPE + cache append, routing, combine,
+matmul with row gather / residual epilogue) against the oracle's restatement of the reference's model code.
+
+Integer results (top-k choice, group sizes, permutations, FP8 codes of unchanged inputs) are bit-exact; bf16 results
+may differ from the float32 oracle by one bf16 rounding (|d| <= 2^-7 relative), float32 ones by accumulation order.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lyra_oracle as O
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def _bf16_close(got, want, what):
+    """Equal up to one bf16 step of a float32 oracle value rounded to bf16."""
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    err = np.abs(got - O.bf16_round(want.copy()))
+    bound = np.abs(want) * 2.0**-7 + 1e-30
+    assert (err <= bound).all(), f"{what}: {int((err > bound).sum())} values off by more than one bf16 step, max {err.max()}"
+    assert (err == 0).mean() > 0.97, f"{what}: only {(err == 0).mean():.3f} bit-identical"
+
+
+@pytest.mark.parametrize("B,C,n,mode", [(64, 2048, 16, "gate"), (5, 256, 7, "logits"), (64, 2048, 15, "logits"), (3, 4096, 63, "logits"),
+                                        (7, 2048, 0, "none"), (2, 4096, 32, "gate")])
+def test_rmsnorm_proj(B, C, n, mode):
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"rmsnorm_proj B{B} C{C} n{n} {mode}")
+    rng = np.random.default_rng(B * 131 + C + n)
+    x = O.bf16_round(rng.standard_normal((B, C), dtype=np.float32) * 3)
+    scale = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    proj = (rng.standard_normal((C, n)) / np.sqrt(C)).astype(np.float32) if n else None
+    bias = rng.standard_normal(n).astype(np.float32) if mode == "logits" else None
+    h, y = F.rmsnorm_proj(U.t_bf16(x), U.t_f32(scale), 1e-5, None if proj is None else U.t_f32(proj),
+                          None if bias is None else U.t_f32(bias), gate=mode == "gate")
+    want_h = O.rms_norm(x, scale, 1e-5)
+    _bf16_close(U.to_np(h), want_h, "h")
+    if n:
+        hn = U.to_np(h)  # the projection must consume the bf16-rounded row
+        logits = hn.astype(np.float64) @ proj.astype(np.float64) + (0 if bias is None else bias)
+        if mode == "gate":
+            _bf16_close(U.to_np(y), (2.0 / (1.0 + np.exp(-logits))).astype(np.float32), "gate")
+        else:
+            np.testing.assert_allclose(U.to_np(y), logits, atol=2e-5, rtol=1e-5)
+    else:
+        assert y is None
+
+
+@pytest.mark.parametrize("B,N,K,S,H,fp8,qknorm,per_row", [
+    (64, 16, 4, 512, 128, True, True, False),
+    (3, 2, 1, 256, 64, True, True, True),
+    (5, 8, 8, 128, 64, False, False, True),
+    (4, 16, 4, 300, 128, False, True, False),
+    (2, 4, 2, 64, 128, True, False, False),
+])
+def test_qkv_post(B, N, K, S, H, fp8, qknorm, per_row):
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray
+
+    _say(f"qkv_post B{B} N{N} K{K} S{S} H{H} fp8={fp8} qknorm={qknorm} per_row={per_row}")
+    rng = np.random.default_rng(B + N * 7 + S)
+    qkv = O.bf16_round(rng.standard_normal((B, (N + 2 * K) * H), dtype=np.float32) * 2)
+    qkv[0, N * H : N * H + H] = 0  # an all-zero key row: scale 1, codes 0
+    qn = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32) if qknorm else None
+    kn = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32) if qknorm else None
+    cos_t, sin_t = O.rope_tables(S, H)
+    pos = rng.integers(0, S, B).astype(np.int32) if per_row else np.full(B, S - 1, np.int32)
+    pos_t = torch.from_numpy(pos).to(U.dev()) if per_row else torch.tensor(S - 1, dtype=torch.int32, device=U.dev())
+    dev = U.dev()
+    sentinel = 0x55
+    if fp8:
+        mk = lambda: QArray(torch.full((B, K, S, H), sentinel, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn),
+                            torch.full((B, K, S, 1), 7.0, dtype=torch.float32, device=dev), (1, H))
+    else:
+        mk = lambda: torch.full((B, K, S, H), 7.0, dtype=torch.bfloat16, device=dev)
+    ck, cv = mk(), mk()
+    q = F.qkv_post(U.t_bf16(qkv), None if qn is None else U.t_f32(qn), None if kn is None else U.t_f32(kn), U.t_f32(cos_t),
+                   U.t_f32(sin_t), pos_t, ck, cv, N, K, H, 1e-5)
+    torch.cuda.synchronize()
+
+    qw, kw, vw = np.split(qkv, [N * H, (N + K) * H], axis=-1)
+    qw, kw, vw = qw.reshape(B, N, H), kw.reshape(B, K, H), vw.reshape(B, K, H)
+    if qknorm:
+        qw, kw = O.bf16_round(O.rms_norm(qw, qn, 1e-5)), O.bf16_round(O.rms_norm(kw, kn, 1e-5))
+    cos, sin = cos_t[pos][:, None, :], sin_t[pos][:, None, :]
+    qw, kw = O.rotate(qw, cos, sin), O.rotate(kw, cos, sin)
+    got_q = U.to_np(q)
+    # norm and rotation each round to bf16 once: allow two bf16 steps on q against the float32 chain
+    assert np.abs(got_q - qw).max() <= np.abs(qw).max() * 2.0**-6
+    assert (got_q == O.bf16_round(qw.copy())).mean() > 0.9
+
+    rows = np.arange(B)
+    for name, cache, want in (("k", ck, O.bf16_round(kw.copy())), ("v", cv, vw)):
+        if fp8:
+            codes = cache.qval.view(torch.uint8).cpu().numpy()
+            scales = cache.scale.cpu().numpy()[..., 0]
+            got_codes, got_scale = codes[rows, :, pos], scales[rows, :, pos]  # [B,K,H], [B,K]
+            if name == "v":  # V is appended untouched: codes and scales are those of the reference quantiser, bit for bit
+                wq, ws = O.quantize(want[:, :, None, :], (1, H))
+                assert np.array_equal(got_codes, wq[:, :, 0]) and np.array_equal(got_scale, ws[:, :, 0, 0])
+            else:  # K went through norm + RoPE (one bf16 step of slack): self-consistent quantisation of the GPU's own row
+                deq = O.fp8_e4m3fn_decode(got_codes) * got_scale[..., None]
+                np.testing.assert_allclose(deq, want, atol=np.abs(want).max() * 0.07, rtol=0.07)
+                amax = np.abs(deq).max(-1)
+                np.testing.assert_allclose(got_scale, np.where(amax > 0, amax / 448, 1.0), rtol=2e-2)
+            # nothing but the appended row was written
+            codes[rows, :, pos] = sentinel
+            scales[rows, :, pos] = 7.0
+            assert (codes == sentinel).all() and (scales == 7.0).all()
+        else:
+            arr = cache.float().cpu().numpy()
+            got = arr[rows, :, pos]
+            if name == "v":
+                assert np.array_equal(got, want)
+            else:
+                assert np.abs(got - want).max() <= np.abs(want).max() * 2.0**-6
+            arr[rows, :, pos] = 7.0
+            assert (arr == 7.0).all()
+
+
+def test_qkv_post_key_codes_bit_exact_at_position_zero():
+    """At position 0 the rotation is the identity (cos 1, sin 0) and without QK norm the key row reaches the
+    quantiser unchanged: its codes and scale must equal the reference quantiser's bit for bit."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray
+
+    B, N, K, S, H = 9, 4, 2, 32, 128
+    rng = np.random.default_rng(11)
+    qkv = O.bf16_round(rng.standard_normal((B, (N + 2 * K) * H), dtype=np.float32) * np.exp(rng.standard_normal((B, 1)) * 3).astype(np.float32))
+    cos_t, sin_t = O.rope_tables(S, H)
+    dev = U.dev()
+    mk = lambda: QArray(torch.zeros((B, K, S, H), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn),
+                        torch.ones((B, K, S, 1), dtype=torch.float32, device=dev), (1, H))
+    ck, cv = mk(), mk()
+    q = F.qkv_post(U.t_bf16(qkv), None, None, U.t_f32(cos_t), U.t_f32(sin_t), torch.tensor(0, dtype=torch.int32, device=dev), ck, cv,
+                   N, K, H, 1e-5)
+    assert np.array_equal(U.to_np(q).reshape(B, -1), qkv[:, : N * H])
+    k = qkv[:, N * H : (N + K) * H].reshape(B, K, 1, H)
+    wq, ws = O.quantize(k, (1, H))
+    assert np.array_equal(ck.qval.view(torch.uint8)[:, :, 0].cpu().numpy(), wq[:, :, 0])
+    assert np.array_equal(ck.scale[:, :, 0, 0].cpu().numpy(), ws[:, :, 0, 0])
+
+
+@pytest.mark.parametrize("T,n_routed,n_shared,k", [(64, 15, 1, 3), (5, 7, 1, 1), (128, 31, 1, 3), (33, 63, 1, 3), (16, 8, 0, 2), (1, 15, 1, 3),
+                                                   (256, 15, 1, 3)])
+def test_moe_route(T, n_routed, n_shared, k):
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"moe_route T{T} routed{n_routed} shared{n_shared} k{k}")
+    rng = np.random.default_rng(T + n_routed)
+    logits = rng.standard_normal((T, n_routed)).astype(np.float32)
+    logits[0, :] = 0.25  # all tied: the lowest indices win
+    if T > 2:
+        logits[2, 1::2] = logits[2, 0]  # ties with the maximum candidate
+    scores, groups, row_map, dest = F.moe_route(U.t_f32(logits), n_routed, n_shared, k)
+    w_scores, w_active, w_groups = O.route_tokens(logits, k, n_routed, n_shared)
+    w_perm, w_dest = O.bpermute(w_active, w_groups, n_routed + n_shared)
+    assert np.array_equal(groups.cpu().numpy(), w_groups)
+    assert np.array_equal(dest.cpu().numpy(), w_dest)
+    assert np.array_equal(row_map.cpu().numpy(), w_perm // (k + n_shared))
+    np.testing.assert_allclose(scores.cpu().numpy(), w_scores, atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("T,topk,C", [(64, 4, 2048), (3, 2, 256), (17, 4, 4096)])
+def test_moe_combine(T, topk, C):
+    from lyra_amd.kernels import decode_fused as F
+
+    rng = np.random.default_rng(T)
+    rows = O.bf16_round(rng.standard_normal((T * topk, C), dtype=np.float32))
+    x = O.bf16_round(rng.standard_normal((T, C), dtype=np.float32))
+    scores = rng.random((T, topk)).astype(np.float32)
+    dest = rng.permutation(T * topk).astype(np.int32)
+    rs = 0.1767766952966369
+    out = F.moe_combine(U.t_bf16(rows), U.t_f32(scores), torch.from_numpy(dest).to(U.dev()), U.t_bf16(x), rs)
+    t = O.bf16_round(O.combine(rows, scores, dest))
+    t = O.bf16_round(t * np.float32(rs))
+    want = x + t
+    _bf16_close(U.to_np(out), want, "combine")
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("M,G,K,N,swiglu", [(64, 1, 2048, 2048, False), (256, 16, 2048, 4096, True), (48, 8, 1024, 2048, False)])
+def test_gemm_row_map_and_residual_epilogue(fp8, M, G, K, N, swiglu):
+    """The fused variants must equal the plain kernel composed with the torch ops they replace, bit for bit."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import quantize
+
+    _say(f"gemm_ex fp8={fp8} M{M} G{G} K{K} N{N} swiglu={swiglu}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(M + G)
+    tokens = max(1, M // 4)
+    x = torch.randn(tokens, K, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(G, K, N, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    if fp8:
+        w = quantize(w, torch.float8_e4m3fn, (K, 1))
+    row_map = torch.randint(0, tokens, (M,), generator=g, device=dev, dtype=torch.int32)
+    sizes = torch.zeros(G, dtype=torch.int32, device=dev)
+    cuts = torch.sort(torch.randint(0, M + 1, (G - 1,), generator=g, device=dev)).values if G > 1 else torch.zeros(0, dtype=torch.int64, device=dev)
+    bounds = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), cuts, torch.full((1,), M, dtype=torch.int64, device=dev)])
+    sizes.copy_((bounds[1:] - bounds[:-1]).to(torch.int32))
+    plain = F.gemm(x[row_map.long()].contiguous(), w, sizes, fused_swiglu=swiglu)
+    gathered = F.gemm(x, w, sizes, rows=M, row_map=row_map, fused_swiglu=swiglu)
+    assert torch.equal(plain, gathered)
+    NO = plain.shape[1]
+    res = torch.randn(M, NO, generator=g, device=dev).to(torch.bfloat16)
+    scale = 0.1767766952966369
+    fused = F.gemm(x, w, sizes, rows=M, row_map=row_map, fused_swiglu=swiglu, residual=res, out_scale=scale)
+    assert torch.equal(fused, res + plain * scale)
+    scaled = F.gemm(x, w, sizes, rows=M, row_map=row_map, fused_swiglu=swiglu, out_scale=scale)
+    assert torch.equal(scaled, plain * scale)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fused_model_matches_unfused(fp8):
+    """Whole decode step: the fused launches against the same step built from torch ops around the two kernels."""
+    from dataclasses import replace
+
+    from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights, model_apply
+
+    cfg = replace(MODEL_VARIANTS["dev"], sliding_window=128, use_sdpa_output_gate=True, seq_len=512)
+    if fp8:
+        cfg = apply_inference_overrides(cfg, fp8=True, fp8_attn=True)
+    dev = U.dev()
+    w = init_weights(cfg, dev, seed=3)
+    B, S, start = 5, 512, 300
+    outs = []
+    for fused in (True, False):
+        c = replace(cfg, fused_glue=fused)
+        cache = init_cache(c, B, S, dev)
+        cache.pos.fill_(start)
+        tok = torch.arange(B, device=dev) * 7 + 1
+        steps = []
+        for _ in range(2):
+            logits, _ = model_apply(tok, w, cache, c)
+            steps.append(U.to_np(logits[:, : cfg.vocab_size]))
+            tok = logits.argmax(-1)
+        outs.append(steps)
+    for a, b in zip(*outs):
+        U.assert_close(a, b, atol=3e-2, rtol=2e-2, what="fused vs unfused logits")
