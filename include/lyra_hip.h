@@ -124,11 +124,12 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
  * bf16 array.
  *
  * lyra_rmsnorm_proj: h = bf16(x * rsqrt(mean(x^2) + eps) * scale) (lyra/model.py:189-191), optionally followed by a
- *   narrow float32 projection of f32(h): y = h @ proj (+ bias), proj [C,n] float32.
+ *   narrow float32 projection of f32(h): y[j] = sum_c h[c] * proj_t[j,c] (+ bias[j]); proj_t [n,C] float32 is the
+ *   reference's [C,n] parameter transposed once at load time so that each output reads a contiguous row.  C % 4 == 0.
  *   mode 1: y -> bf16(2 * sigmoid(y)), the per-head output gate (model.py:343-347), y is bf16 [B,n];
- *   mode 2: y float32 [B,n], the router logits (model.py:455-457).  proj NULL: norm only.
+ *   mode 2: y float32 [B,n], the router logits (model.py:455-457).  proj_t NULL: norm only.
  */
-int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj, const float* bias, void* y, int B, int C,
+int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C,
                       int n, int mode, float eps, lyra_stream_t stream);
 
 /*

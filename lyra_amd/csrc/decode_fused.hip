@@ -22,54 +22,69 @@ __device__ __forceinline__ float block_sum(float v, float* sm) {  // blockDim.x 
 
 // ---- RMS norm (+ a narrow float32 projection of the normalised row) ---------------------------------------
 // h = bf16(x * rsqrt(mean(x^2) + eps) * scale)                      lyra/model.py:189-191
-// y[j] = sum_c f32(h[c]) * P[c, j] (+ bias[j]), j < n                router logits (model.py:455-457) or the
+// y[j] = sum_c f32(h[c]) * Pt[j, c] (+ bias[j]), j < n               router logits (model.py:455-457) or the
 // gate = bf16(2 * sigmoid(y))                                        output gate (model.py:343-347)
+// One workgroup per row.  The normalised row stays in LDS; each wavefront then takes output columns in turn and
+// reads that column's weights (a contiguous row of the transposed projection) 16 bytes per lane.
 struct NormProjParams {
     const uint16_t* x;
     const float* scale;
     uint16_t* h;
-    const float* proj;  // [C, n] or null
-    const float* bias;  // [n] or null
-    void* y;            // mode 1: bf16 [B, n] gate; mode 2: float32 [B, n]
+    const float* proj_t;  // [n, C] or null
+    const float* bias;    // [n] or null
+    void* y;              // mode 1: bf16 [B, n] gate; mode 2: float32 [B, n]
     int C, n, mode;
     float eps;
 };
 
-__global__ __launch_bounds__(256) void rmsnorm_proj_kernel(NormProjParams p) {
-    __shared__ float sm[64];
+constexpr int kNormThreads = 512;
+
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjParams p) {
+    extern __shared__ float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
+    float* sm_red = sm_h + p.C;
     const int b = blockIdx.x;
     const uint16_t* xr = p.x + (size_t)b * p.C;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
-        const float v = bf16_bits_to_f32(xr[c]);
-        ss += v * v;
+    for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // C % 4 == 0
+        const u32x2 d = *(const u32x2*)(xr + c);
+        const float v0 = __uint_as_float(d[0] << 16), v1 = __uint_as_float(d[0] & 0xFFFF0000u);
+        const float v2 = __uint_as_float(d[1] << 16), v3 = __uint_as_float(d[1] & 0xFFFF0000u);
+        sm_h[c] = v0; sm_h[c + 1] = v1; sm_h[c + 2] = v2; sm_h[c + 3] = v3;
+        ss += v0 * v0 + v1 * v1 + v2 * v2 + v3 * v3;
     }
-    ss = block_sum(ss, sm);
+    ss = block_sum(ss, sm_red);
     const float inv = rsqrtf(ss / (float)p.C + p.eps);
-    for (int c = threadIdx.x; c < p.C; c += blockDim.x)
-        p.h[(size_t)b * p.C + c] = f32_to_bf16_bits(bf16_bits_to_f32(xr[c]) * inv * p.scale[c]);
-    if (!p.proj) return;
-    for (int j0 = 0; j0 < p.n; j0 += 16) {  // 16 output columns per sweep over the row
-        float acc[16];
+    for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // each thread revisits its own elements
+        const f32x4 sc = *(const f32x4*)(p.scale + c);
+        float v[4];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-        for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
-            const float hv = bf16r(bf16_bits_to_f32(xr[c]) * inv * p.scale[c]);
-            const float* pr = p.proj + (size_t)c * p.n + j0;
-#pragma unroll
-            for (int j = 0; j < 16; ++j)
-                if (j0 + j < p.n) acc[j] += hv * pr[j];
+        for (int i = 0; i < 4; ++i) v[i] = sm_h[c + i] * inv * sc[i];
+        u32x2 d;
+        d[0] = pack_bf16(v[0], v[1]);
+        d[1] = pack_bf16(v[2], v[3]);
+        *(u32x2*)(p.h + (size_t)b * p.C + c) = d;
+        sm_h[c] = __uint_as_float(d[0] << 16);
+        sm_h[c + 1] = __uint_as_float(d[0] & 0xFFFF0000u);
+        sm_h[c + 2] = __uint_as_float(d[1] << 16);
+        sm_h[c + 3] = __uint_as_float(d[1] & 0xFFFF0000u);
+    }
+    if (!p.proj_t) return;
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int j = wave; j < p.n; j += kNormThreads / 64) {
+        const float* pr = p.proj_t + (size_t)j * p.C;
+        float acc = 0.f;
+        for (int c = lane * 4; c < p.C; c += 256) {
+            const f32x4 w = *(const f32x4*)(pr + c);
+            const f32x4 hv = *(const f32x4*)(sm_h + c);
+            acc += hv[0] * w[0] + hv[1] * w[1] + hv[2] * w[2] + hv[3] * w[3];
         }
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            if (j0 + j >= p.n) break;
-            float v = block_sum(acc[j], sm);
-            if (threadIdx.x == 0) {
-                if (p.bias) v += p.bias[j0 + j];
-                const size_t o = (size_t)b * p.n + j0 + j;
-                if (p.mode == 1) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(2.f / (1.f + __expf(-v)));
-                else ((float*)p.y)[o] = v;
-            }
+        float v = wave_sum(acc);
+        if (lane == 0) {
+            if (p.bias) v += p.bias[j];
+            const size_t o = (size_t)b * p.n + j;
+            if (p.mode == 1) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(2.f / (1.f + __expf(-v)));
+            else ((float*)p.y)[o] = v;
         }
     }
 }
@@ -264,13 +279,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
 
 }  // namespace lyra
 
-extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj, const float* bias, void* y,
+extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
                                  int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
     using namespace lyra;
     if (!x || !scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
-    if (proj && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
-    NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj, bias, y, C, proj ? n : 0, mode, eps};
-    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B), dim3(256), 0, (hipStream_t)stream, p);
+    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
+    NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps};
+    const size_t lds = ((size_t)C + 16) * sizeof(float);
+    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 

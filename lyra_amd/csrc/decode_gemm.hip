@@ -374,11 +374,174 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
     }
 }
 
+
+// ---- small weight sets: one group, a few MB of weights (the dense projections of a decode layer) -----------------
+// Such a product is bound by latency, not bandwidth: what counts is how many weight rows are in flight.  A workgroup
+// owns one 16-row x 128-column output tile; its 8 wavefronts interleave over K in steps of 32 rows, each keeping
+// DEPTH steps of weights and activations in flight (activations come straight from global memory, they are L2
+// resident), and their partial tiles are summed through LDS in a fixed order.  No split over workgroups, no second
+// pass, no workspace.  Rows at or beyond group_sizes[0] multiply zeros (epilogue(0), lax.ragged_dot semantics).
+constexpr int kSmallWaves = 8;
+
+template <bool FP8, int DEPTH>
+__global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(GemmParams p) {
+    constexpr int ES = FP8 ? 1 : 2;
+    extern __shared__ float sm_part[];  // [kSmallWaves][16][128]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int x = lane & 15, kb = lane >> 4;
+    const int span = blockIdx.x, row0 = blockIdx.y * 16;
+    const int cnt = min(p.group_sizes[0], p.M);
+
+    int ncol;
+    const bool is_lin_lane = p.swiglu && x >= 8;
+    if (p.swiglu) ncol = (is_lin_lane ? (p.N >> 1) : 0) + span * 64 + 8 * (x & 7);
+    else ncol = span * 128 + 8 * x;
+
+    const int row_bytes = p.N * ES;
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+    const int wvoff = 8 * kb * row_bytes + ncol * ES;
+
+    // activations of this lane: row row0 + x, 8 consecutive k of k-group kb
+    const int arow = row0 + x;
+    const bool a_ok = arow < cnt;
+    const int asrc = a_ok ? (p.row_map ? p.row_map[arow] : arow) : 0;
+    const uint16_t* aptr = p.lhs + (size_t)asrc * p.K + 8 * kb;
+
+    const int steps = p.K >> 5;
+    const int n_my = (steps - wave + kSmallWaves - 1) / kSmallWaves;  // steps wave, wave + 8, ...
+    const bool step_scales = FP8 && p.scale_mode == 1 && p.bk < p.K;
+    const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (ncol >> p.bn_shift) : nullptr;
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    RawW<FP8> w[DEPTH];
+    u32x4 a[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        a[d] = u32x4{0u, 0u, 0u, 0u};
+        if (d < n_my) {
+            const int kk = (wave + kSmallWaves * d) << 5;
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) load_w_pair<FP8>(w[d], pr, wrsrc, wvoff, kk, row_bytes);
+            if (a_ok) a[d] = *(const u32x4*)(aptr + kk);
+        }
+    }
+    for (int base = 0; base < n_my; base += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int idx = base + d;
+            if (idx < n_my) {
+                const int kk = (wave + kSmallWaves * idx) << 5;
+                const int kk_next = kk + ((kSmallWaves * DEPTH) << 5);
+                const bool more = idx + DEPTH < n_my;
+                Pack8 bop[8], av;
+                av.u[0] = a[d][0]; av.u[1] = a[d][1]; av.u[2] = a[d][2]; av.u[3] = a[d][3];
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    convert_pair<FP8>(w[d], pr, bop);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (more) load_w_pair<FP8>(w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (more && a_ok) a[d] = *(const u32x4*)(aptr + kk_next);
+                if (step_scales) {
+                    const float sc = sc_lane[(size_t)(kk / p.bk) * p.NB];
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                        acc[c][0] += t[0] * sc;
+                        acc[c][1] += t[1] * sc;
+                        acc[c][2] += t[2] * sc;
+                        acc[c][3] += t[3] * sc;
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) acc[c] = mfma_16x16x32(av.v, bop[c].v, acc[c]);
+                }
+            }
+        }
+    }
+
+    float colscale[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
+    if (FP8 && p.scale_mode == 1 && !step_scales) {
+        const float sc = *sc_lane;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = sc;
+    } else if (FP8 && p.scale_mode == 2) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(ncol + c) >> p.bn_shift];
+    }
+    float* mine = sm_part + wave * (16 * 128);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float* dst = mine + (4 * kb + r) * 128 + 8 * x;
+        *(f32x4*)dst = f32x4{acc[0][r] * colscale[0], acc[1][r] * colscale[1], acc[2][r] * colscale[2], acc[3][r] * colscale[3]};
+        *(f32x4*)(dst + 4) = f32x4{acc[4][r] * colscale[4], acc[5][r] * colscale[5], acc[6][r] * colscale[6], acc[7][r] * colscale[7]};
+    }
+    __syncthreads();
+
+    // thread t finishes row t / 32 of the tile: 4 columns (2 gate + 2 linear columns with SwiGLU)
+    const int r = threadIdx.x >> 5, q = threadIdx.x & 31;
+    const int row = row0 + r;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.swiglu) {
+#pragma unroll
+        for (int wv = 0; wv < kSmallWaves; ++wv) {
+            const float* src = sm_part + wv * (16 * 128) + r * 128 + 2 * q;
+            const f32x2 g2 = *(const f32x2*)src, l2 = *(const f32x2*)(src + 64);
+            v[0] += g2[0]; v[1] += g2[1]; v[2] += l2[0]; v[3] += l2[1];
+        }
+    } else {
+#pragma unroll
+        for (int wv = 0; wv < kSmallWaves; ++wv) {
+            const f32x4 t = *(const f32x4*)(sm_part + wv * (16 * 128) + r * 128 + 4 * q);
+            v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+        }
+    }
+    if (row >= p.M) return;
+    if (p.swiglu) {
+        const int NO = p.N >> 1, oc = span * 64 + 2 * q;
+        if (p.bias) {
+            v[0] += p.bias[oc]; v[1] += p.bias[oc + 1]; v[2] += p.bias[NO + oc]; v[3] += p.bias[NO + oc + 1];
+        }
+        float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
+        const size_t idx = (size_t)row * NO + oc;
+        if (p.post_scale) {
+            o[0] = residual_epilogue(p, o[0], idx);
+            o[1] = residual_epilogue(p, o[1], idx + 1);
+        }
+        if (p.out_f32) *(f32x2*)((float*)p.out + idx) = f32x2{o[0], o[1]};
+        else *(uint32_t*)((uint16_t*)p.out + idx) = pack_bf16(o[0], o[1]);
+    } else {
+        const int oc = span * 128 + 4 * q;
+        const size_t idx = (size_t)row * p.N + oc;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (p.bias) v[c] += p.bias[oc + c];
+            if (p.post_scale) v[c] = residual_epilogue(p, v[c], idx + c);
+        }
+        if (p.out_f32) {
+            *(f32x4*)((float*)p.out + idx) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+            u32x2 d;
+            d[0] = pack_bf16(v[0], v[1]);
+            d[1] = pack_bf16(v[2], v[3]);
+            *(u32x2*)((uint16_t*)p.out + idx) = d;
+        }
+    }
+}
+
 struct GemmPlan {
     int mt;       // 16-row tiles held in registers per pass
     int row_par;  // row blocks of one group spread over this many workgroups
     int spans;    // 128-column spans (64+64 with SwiGLU)
     int ksplit, kpart;
+    bool one_pass;  // single group with a few MB of weights: decode_gemm_small_kernel
 };
 
 // Shape-only plan (group sizes live on the device).  Large weight sets are streamed once: wide row blocks, K
@@ -393,6 +556,16 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     GemmPlan pl;
     const int touched = std::max(1, std::min(G, M));
     const double weight_bytes = (double)touched * K * N;
+    static const bool no_one_pass = getenv("LYRA_GEMM_NO_ONE_PASS") != nullptr;  // tuning override
+    pl.one_pass = G == 1 && weight_bytes <= 48e6 && !no_one_pass;
+    if (pl.one_pass) {
+        pl.mt = 1;
+        pl.row_par = (M + 15) / 16;
+        pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
+        pl.ksplit = 1;
+        pl.kpart = K;
+        return pl;
+    }
     const bool small = weight_bytes <= 48e6 && M > 16;
     pl.mt = M <= 16 ? 1 : (small ? 1 : (M <= 32 ? 2 : 4));
     pl.row_par = small ? std::min(8, (M / std::max(1, touched) + 15) / 16) : 1;
@@ -485,6 +658,13 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     }
 
     hipStream_t st = (hipStream_t)stream;
+    if (pl.one_pass) {
+        const dim3 sgrid(pl.spans, pl.row_par), sblock(kSmallWaves * 64);
+        const size_t slds = (size_t)kSmallWaves * 16 * 128 * sizeof(float);
+        if (fp8) hipLaunchKernelGGL((decode_gemm_small_kernel<true, 4>), sgrid, sblock, slds, st, p);
+        else hipLaunchKernelGGL((decode_gemm_small_kernel<false, 2>), sgrid, sblock, slds, st, p);
+        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+    }
     const dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
     const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t);
 #define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p)

@@ -28,6 +28,19 @@ def _f32(t):
     return t
 
 
+_TRANSPOSED: dict = {}
+
+
+def _transposed(w: torch.Tensor) -> torch.Tensor:
+    """[C,n] parameter -> contiguous [n,C] copy, made once per weight tensor (weights do not change while decoding)."""
+    key = (w.data_ptr(), tuple(w.shape), w.device)
+    hit = _TRANSPOSED.get(key)
+    if hit is None or hit[0] is not w:
+        hit = (w, w.t().contiguous())
+        _TRANSPOSED[key] = hit
+    return hit[1]
+
+
 def rmsnorm_proj(x: torch.Tensor, scale: torch.Tensor, eps: float, proj: torch.Tensor | None = None,
                  bias: torch.Tensor | None = None, gate: bool = False):
     """rms_norm (lyra/model.py:189-191) of x [B,C] bf16; with ``proj`` [C,n] f32 also f32(h) @ proj (+ bias) as
@@ -39,7 +52,7 @@ def rmsnorm_proj(x: torch.Tensor, scale: torch.Tensor, eps: float, proj: torch.T
     if proj is not None:
         n = proj.shape[1]
         y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=x.device)
-        _f32(proj)
+        proj = _f32(_transposed(proj))
     rc = _L.lyra_rmsnorm_proj(x.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
                               1 if gate else 2, float(eps), _stream(x.device))
     _lib.check(rc, "lyra_rmsnorm_proj")
