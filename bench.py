@@ -115,6 +115,20 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, launches=100):
     return start.elapsed_time(stop) * 1e-3 / launches  # seconds per launch
 
 
+def traffic_probe(device, mib=256, repeats=4):
+    """A plain streaming kernel of known HBM traffic (reads `mib` MiB, writes `mib` MiB per launch), launched a few
+    times so that a hardware-counter run of this script can scale FETCH_SIZE / WRITE_SIZE against it."""
+    import torch
+
+    n = mib * (1 << 20) // 4
+    src = torch.arange(n, dtype=torch.int32, device=device)
+    dst = torch.empty_like(src)
+    for _ in range(repeats):
+        torch.add(src, 1, out=dst)
+    torch.cuda.synchronize()
+    return {"kernel": "torch add(int32, 1)", "read_bytes": n * 4, "write_bytes": n * 4, "launches": repeats}
+
+
 def cpu_baseline(cfg, weights, cache, ctx, sample_batch):
     """The CPU restatement of the reference decode step (oracle/decode_step.py, threaded C contractions) on the first
     `sample_batch` sequences of the same workload: one full step, all layers, context 4096."""
@@ -155,6 +169,8 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--cpu-sample", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch a copy-like kernel of known size (reference point for rocprofv3 --pmc runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's decode path; run with --gpus 1 (no multi-GPU figure exists).")
@@ -208,6 +224,8 @@ def main():
             "us_per_launch": t_attn * 1e6,
         },
     }
+    if args.traffic_probe:
+        result["traffic_probe"] = traffic_probe(dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, weights, cache, args.ctx, min(args.cpu_sample, args.batch))
     print(json.dumps(result))
