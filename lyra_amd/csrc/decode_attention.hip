@@ -105,16 +105,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 }
 
 template <int H, bool FP8>
-__device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base) {
+__device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base, bool live) {
     constexpr int ES = RawK<H, FP8>::ES;
     constexpr int KW = RawK<H, FP8>::KW;
     constexpr int RB = H * ES;  // bytes per cached row
-    const int soff = __builtin_amdgcn_readfirstlane(base * RB);
+    const int soff = __builtin_amdgcn_readfirstlane(live ? base * RB : 0);
+    const int voff = live ? sl.voff_k : kNoLoad;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int w = 0; w < KW; w += 4) {
-            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, sl.voff_k + j * 16 * RB + w * 4, soff, 0);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, voff + j * 16 * RB + w * 4, soff, 0);
             t.k[j][w] = d[0];
             t.k[j][w + 1] = d[1];
             t.k[j][w + 2] = d[2];
@@ -123,13 +124,14 @@ __device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base
 }
 
 template <bool VEC4>
-__device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base) {
-    const int ssoff = __builtin_amdgcn_readfirstlane(base * 4);
+__device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base, bool live) {
+    const int ssoff = __builtin_amdgcn_readfirstlane(live ? base * 4 : 0);
+    const int voff = live ? sl.voff_s : kNoLoad;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         if constexpr (VEC4) {
-            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(sl.ks, sl.voff_s + j * 64, ssoff, 0);
-            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(sl.vs, sl.voff_s + j * 64, ssoff, 0);
+            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(sl.ks, voff + j * 64, ssoff, 0);
+            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(sl.vs, voff + j * 64, ssoff, 0);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 t.ks[4 * j + r] = __uint_as_float(a[r]);
@@ -138,22 +140,23 @@ __device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base) {
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                t.ks[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.ks, sl.voff_s + j * 64 + r * 4, ssoff, 0));
-                t.vs[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.vs, sl.voff_s + j * 64 + r * 4, ssoff, 0));
+                t.ks[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.ks, voff + j * 64 + r * 4, ssoff, 0));
+                t.vs[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.vs, voff + j * 64 + r * 4, ssoff, 0));
             }
         }
     }
 }
 
 template <int H, bool FP8>
-__device__ __forceinline__ void load_v(RawV<H, FP8>& t, const Slab& sl, int base) {
+__device__ __forceinline__ void load_v(RawV<H, FP8>& t, const Slab& sl, int base, bool live) {
     constexpr int ES = RawV<H, FP8>::ES;
     constexpr int VW = RawV<H, FP8>::VW;
     constexpr int RB = H * ES;
-    const int soff = __builtin_amdgcn_readfirstlane(base * RB);
+    const int soff = __builtin_amdgcn_readfirstlane(live ? base * RB : 0);
+    const int voff = live ? sl.voff_v : kNoLoad;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int off = sl.voff_v + (16 * (i >> 2) + (i & 3)) * RB;
+        const int off = voff + (16 * (i >> 2) + (i & 3)) * RB;
         if constexpr (VW == 1) {
             t.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(sl.v, off, soff, 0);
         } else if constexpr (VW == 2) {
@@ -347,10 +350,11 @@ void decode_attention_kernel(AttnParams p) {
     RawS rs;
     RawV<H, FP8> rv;
     int tile = wave;
-    if (tile < n_tiles) {
-        load_k<H, FP8>(rk, sl, c_lo + tile * kTile);
-        if constexpr (FP8) load_s<VEC4>(rs, sl, c_lo + tile * kTile);
-        load_v<H, FP8>(rv, sl, c_lo + tile * kTile);
+    {  // (a wavefront without tiles issues the same loads with an offset outside the slab: they fetch nothing)
+        const bool live = tile < n_tiles;
+        load_k<H, FP8>(rk, sl, c_lo + tile * kTile, live);
+        if constexpr (FP8) load_s<VEC4>(rs, sl, c_lo + tile * kTile, live);
+        load_v<H, FP8>(rv, sl, c_lo + tile * kTile, live);
     }
 
     // q of this kv head's G query heads, padded to 16 rows of zeros, in LDS: the Q^T operand of lane
@@ -371,6 +375,9 @@ void decode_attention_kernel(AttnParams p) {
     for (int c = 0; c < CB; ++c) acc.o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
 
+    // Loads for a tile past the end are issued all the same, with a lane offset no buffer contains (they return zeros
+    // without touching memory): the number of loads in flight is then identical on every path and each wait covers
+    // exactly the loads it needs.
     // Software pipeline over this wavefront's tiles (wave, wave + WAVES, ...: a fixed assignment, so results are
     // bit-reproducible from run to run) with a single register set: each operand of the
     // next tile is requested right after the last use of the current one, so the loads fly during the rest
@@ -384,21 +391,19 @@ void decode_attention_kernel(AttnParams p) {
         f32x4 s[2];
         tile_logits<H, FP8>(rk, sm_q, lane, s);
         __builtin_amdgcn_sched_barrier(0);
-        if (more) load_k<H, FP8>(rk, sl, next);
+        load_k<H, FP8>(rk, sl, next, more);
         __builtin_amdgcn_sched_barrier(0);
         uint32_t vis;
         bf16x8 pop;
         if (full) pop = tile_softmax<H, FP8, false>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
         else pop = tile_softmax<H, FP8, true>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (FP8) {
-            if (more) load_s<VEC4>(rs, sl, next);
-        }
+        if constexpr (FP8) load_s<VEC4>(rs, sl, next, more);
         __builtin_amdgcn_sched_barrier(0);
         if (full) tile_values<H, FP8, false>(rv, pop, vis, acc);
         else tile_values<H, FP8, true>(rv, pop, vis, acc);
         __builtin_amdgcn_sched_barrier(0);
-        if (more) load_v<H, FP8>(rv, sl, next);
+        load_v<H, FP8>(rv, sl, next, more);
         __builtin_amdgcn_sched_barrier(0);
         tile = next_tile;
     }

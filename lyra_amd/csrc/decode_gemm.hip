@@ -89,6 +89,17 @@ __device__ __forceinline__ void load_w_pair(RawW<FP8>& t, int pair, __amdgpu_buf
     }
 }
 
+// Loads that may
+// run past the end of the data are issued unconditionally with the lane offset kNoLoad instead of being branched around, so
+// that the number of loads in flight is the same on every path and each wait covers exactly the loads it needs
+// (a load inside a branch makes the compiler wait for every outstanding load at the next use).
+
+template <bool FP8>
+__device__ __forceinline__ void load_w_pair_if(bool live, RawW<FP8>& t, int pair, __amdgpu_buffer_rsrc_t rsrc, int voff, int kk,
+                                               int row_bytes) {
+    load_w_pair<FP8>(t, pair, rsrc, live ? voff : kNoLoad, live ? kk : 0, live ? row_bytes : 0);
+}
+
 // Element `pair` of the K-major B operands of all 8 column phases: pairing two weight rows in the bf16 pack
 // step transposes the row-major weights for free.
 template <bool FP8>
@@ -383,14 +394,13 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
 // pass, no workspace.  Rows at or beyond group_sizes[0] multiply zeros (epilogue(0), lax.ragged_dot semantics).
 constexpr int kSmallWaves = 8;
 
-template <bool FP8, int DEPTH>
+template <bool FP8, int DEPTH, bool STEP_SCALES, bool ONE_ROUND>
 __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSmallWaves][16][128]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
     const int span = blockIdx.x, row0 = blockIdx.y * 16;
-    const int cnt = min(p.group_sizes[0], p.M);
 
     int ncol;
     const bool is_lin_lane = p.swiglu && x >= 8;
@@ -402,73 +412,42 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
         const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
     const int wvoff = 8 * kb * row_bytes + ncol * ES;
 
-    // activations of this lane: row row0 + x, 8 consecutive k of k-group kb
+    // Everything the kernel reads is requested before anything is waited for, in the order it is consumed
+    // (loads return in order): activations, weights, then what the epilogue needs.
+    // Activations of this lane: row row0 + x, 8 consecutive k of k-group kb.  Whether the row belongs to the group
+    // is only known once group_sizes[0] has arrived; the values are zeroed then, the loads do not wait for it.
     const int arow = row0 + x;
-    const bool a_ok = arow < cnt;
-    const int asrc = a_ok ? (p.row_map ? p.row_map[arow] : arow) : 0;
-    const uint16_t* aptr = p.lhs + (size_t)asrc * p.K + 8 * kb;
+    const int asrc = arow < p.M ? (p.row_map ? p.row_map[arow] : arow) : 0;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
+    const int avoff = arow < p.M ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
 
     const int steps = p.K >> 5;
     const int n_my = (steps - wave + kSmallWaves - 1) / kSmallWaves;  // steps wave, wave + 8, ...
-    const bool step_scales = FP8 && p.scale_mode == 1 && p.bk < p.K;
     const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (ncol >> p.bn_shift) : nullptr;
-
-    f32x4 acc[8];
-#pragma unroll
-    for (int c = 0; c < 8; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     RawW<FP8> w[DEPTH];
     u32x4 a[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        a[d] = u32x4{0u, 0u, 0u, 0u};
-        if (d < n_my) {
-            const int kk = (wave + kSmallWaves * d) << 5;
-#pragma unroll
-            for (int pr = 0; pr < 4; ++pr) load_w_pair<FP8>(w[d], pr, wrsrc, wvoff, kk, row_bytes);
-            if (a_ok) a[d] = *(const u32x4*)(aptr + kk);
-        }
+        const bool live = d < n_my;
+        const int kk = (wave + kSmallWaves * d) << 5;
+        a[d] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff : kNoLoad, __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0), 0);
     }
-    for (int base = 0; base < n_my; base += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int idx = base + d;
-            if (idx < n_my) {
-                const int kk = (wave + kSmallWaves * idx) << 5;
-                const int kk_next = kk + ((kSmallWaves * DEPTH) << 5);
-                const bool more = idx + DEPTH < n_my;
-                Pack8 bop[8], av;
-                av.u[0] = a[d][0]; av.u[1] = a[d][1]; av.u[2] = a[d][2]; av.u[3] = a[d][3];
+    for (int d = 0; d < DEPTH; ++d) {
+        const bool live = d < n_my;
+        const int kk = (wave + kSmallWaves * d) << 5;
 #pragma unroll
-                for (int pr = 0; pr < 4; ++pr) {
-                    convert_pair<FP8>(w[d], pr, bop);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (more) load_w_pair<FP8>(w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                if (more && a_ok) a[d] = *(const u32x4*)(aptr + kk_next);
-                if (step_scales) {
-                    const float sc = sc_lane[(size_t)(kk / p.bk) * p.NB];
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) {
-                        const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
-                        acc[c][0] += t[0] * sc;
-                        acc[c][1] += t[1] * sc;
-                        acc[c][2] += t[2] * sc;
-                        acc[c][3] += t[3] * sc;
-                    }
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) acc[c] = mfma_16x16x32(av.v, bop[c].v, acc[c]);
-                }
-            }
-        }
+        for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
     }
+    __builtin_amdgcn_sched_barrier(0);
 
+    // epilogue inputs: the scales of this lane's 8 columns; bias and residual of the 4 outputs thread t finishes
+    // (row t / 32 of the tile; 4 columns, or 2 gate + 2 linear columns with SwiGLU)
     float colscale[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
-    if (FP8 && p.scale_mode == 1 && !step_scales) {
+    if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
         const float sc = *sc_lane;
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = sc;
@@ -476,6 +455,82 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(ncol + c) >> p.bn_shift];
     }
+    const int er = threadIdx.x >> 5, eq = threadIdx.x & 31;
+    const int erow = row0 + er;
+    const bool e_ok = erow < p.M;
+    const int NO = p.swiglu ? p.N >> 1 : p.N;
+    const int oc = p.swiglu ? span * 64 + 2 * eq : span * 128 + 4 * eq;
+    const size_t oidx = (size_t)erow * NO + oc;
+    float ebias[4] = {0.f, 0.f, 0.f, 0.f}, eres[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+        if (p.swiglu) {
+            ebias[0] = p.bias[oc]; ebias[1] = p.bias[oc + 1]; ebias[2] = p.bias[NO + oc]; ebias[3] = p.bias[NO + oc + 1];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) ebias[c] = p.bias[oc + c];
+        }
+    }
+    if (p.residual && e_ok) {
+        if (p.swiglu) {
+            const uint32_t d = *(const uint32_t*)(p.residual + oidx);
+            eres[0] = __uint_as_float(d << 16); eres[1] = __uint_as_float(d & 0xFFFF0000u);
+        } else {
+            const u32x2 d = *(const u32x2*)(p.residual + oidx);
+            eres[0] = __uint_as_float(d[0] << 16); eres[1] = __uint_as_float(d[0] & 0xFFFF0000u);
+            eres[2] = __uint_as_float(d[1] << 16); eres[3] = __uint_as_float(d[1] & 0xFFFF0000u);
+        }
+    }
+    const int cnt = min(p.group_sizes[0], p.M);
+    const bool a_ok = arow < cnt;
+    __builtin_amdgcn_sched_barrier(0);
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // every pass issues the same loads (past the end they fetch nothing) and multiplies zeros there
+    for (int base = 0; base < (ONE_ROUND ? 1 : n_my); base += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int idx = base + d;
+            const int kk = (wave + kSmallWaves * idx) << 5;
+            const int kk_next = kk + ((kSmallWaves * DEPTH) << 5);
+            const bool more = idx + DEPTH < n_my;
+            Pack8 bop[8], av;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av.u[i] = a_ok ? a[d][i] : 0u;
+            if constexpr (!ONE_ROUND) {
+                __builtin_amdgcn_sched_barrier(0);
+                a[d] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff : kNoLoad,
+                                                             __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0), 0);
+            }
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {
+                convert_pair<FP8>(w[d], pr, bop);
+                if constexpr (!ONE_ROUND) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_w_pair_if<FP8>(more, w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if constexpr (STEP_SCALES) {
+                const float sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                    acc[c][0] += t[0] * sc;
+                    acc[c][1] += t[1] * sc;
+                    acc[c][2] += t[2] * sc;
+                    acc[c][3] += t[3] * sc;
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[c] = mfma_16x16x32(av.v, bop[c].v, acc[c]);
+            }
+            if constexpr (ONE_ROUND) __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
     float* mine = sm_part + wave * (16 * 128);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -486,52 +541,44 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
     __syncthreads();
 
     // thread t finishes row t / 32 of the tile: 4 columns (2 gate + 2 linear columns with SwiGLU)
-    const int r = threadIdx.x >> 5, q = threadIdx.x & 31;
-    const int row = row0 + r;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (p.swiglu) {
 #pragma unroll
         for (int wv = 0; wv < kSmallWaves; ++wv) {
-            const float* src = sm_part + wv * (16 * 128) + r * 128 + 2 * q;
+            const float* src = sm_part + wv * (16 * 128) + er * 128 + 2 * eq;
             const f32x2 g2 = *(const f32x2*)src, l2 = *(const f32x2*)(src + 64);
             v[0] += g2[0]; v[1] += g2[1]; v[2] += l2[0]; v[3] += l2[1];
         }
     } else {
 #pragma unroll
         for (int wv = 0; wv < kSmallWaves; ++wv) {
-            const f32x4 t = *(const f32x4*)(sm_part + wv * (16 * 128) + r * 128 + 4 * q);
+            const f32x4 t = *(const f32x4*)(sm_part + wv * (16 * 128) + er * 128 + 4 * eq);
             v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
         }
     }
-    if (row >= p.M) return;
-    if (p.swiglu) {
-        const int NO = p.N >> 1, oc = span * 64 + 2 * q;
-        if (p.bias) {
-            v[0] += p.bias[oc]; v[1] += p.bias[oc + 1]; v[2] += p.bias[NO + oc]; v[3] += p.bias[NO + oc + 1];
-        }
-        float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
-        const size_t idx = (size_t)row * NO + oc;
-        if (p.post_scale) {
-            o[0] = residual_epilogue(p, o[0], idx);
-            o[1] = residual_epilogue(p, o[1], idx + 1);
-        }
-        if (p.out_f32) *(f32x2*)((float*)p.out + idx) = f32x2{o[0], o[1]};
-        else *(uint32_t*)((uint16_t*)p.out + idx) = pack_bf16(o[0], o[1]);
-    } else {
-        const int oc = span * 128 + 4 * q;
-        const size_t idx = (size_t)row * p.N + oc;
+    if (!e_ok) return;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (p.bias) v[c] += p.bias[oc + c];
-            if (p.post_scale) v[c] = residual_epilogue(p, v[c], idx + c);
+    for (int c = 0; c < 4; ++c) v[c] += ebias[c];
+    if (p.swiglu) {
+        float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
+        if (p.post_scale) {
+            o[0] = round_bf16(round_bf16(o[0]) * p.out_scale) + eres[0];
+            o[1] = round_bf16(round_bf16(o[1]) * p.out_scale) + eres[1];
+        }
+        if (p.out_f32) *(f32x2*)((float*)p.out + oidx) = f32x2{o[0], o[1]};
+        else *(uint32_t*)((uint16_t*)p.out + oidx) = pack_bf16(o[0], o[1]);
+    } else {
+        if (p.post_scale) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = round_bf16(round_bf16(v[c]) * p.out_scale) + eres[c];
         }
         if (p.out_f32) {
-            *(f32x4*)((float*)p.out + idx) = f32x4{v[0], v[1], v[2], v[3]};
+            *(f32x4*)((float*)p.out + oidx) = f32x4{v[0], v[1], v[2], v[3]};
         } else {
             u32x2 d;
             d[0] = pack_bf16(v[0], v[1]);
             d[1] = pack_bf16(v[2], v[3]);
-            *(u32x2*)((uint16_t*)p.out + idx) = d;
+            *(u32x2*)((uint16_t*)p.out + oidx) = d;
         }
     }
 }
@@ -661,8 +708,24 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     if (pl.one_pass) {
         const dim3 sgrid(pl.spans, pl.row_par), sblock(kSmallWaves * 64);
         const size_t slds = (size_t)kSmallWaves * 16 * 128 * sizeof(float);
-        if (fp8) hipLaunchKernelGGL((decode_gemm_small_kernel<true, 4>), sgrid, sblock, slds, st, p);
-        else hipLaunchKernelGGL((decode_gemm_small_kernel<false, 2>), sgrid, sblock, slds, st, p);
+        const int per_wave = (K / 32 + kSmallWaves - 1) / kSmallWaves;  // steps of 32 rows each wavefront walks
+        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+#define LYRA_SMALL(F, D, S, O) hipLaunchKernelGGL((decode_gemm_small_kernel<F, D, S, O>), sgrid, sblock, slds, st, p)
+        if (step_scales) {
+            if (per_wave <= 4) LYRA_SMALL(true, 4, true, true);
+            else LYRA_SMALL(true, 4, true, false);
+        } else if (fp8) {
+            if (per_wave <= 2) LYRA_SMALL(true, 2, false, true);
+            else if (per_wave <= 4) LYRA_SMALL(true, 4, false, true);
+            else if (per_wave <= 6) LYRA_SMALL(true, 6, false, true);
+            else if (per_wave <= 8) LYRA_SMALL(true, 8, false, true);
+            else LYRA_SMALL(true, 6, false, false);
+        } else {
+            if (per_wave <= 2) LYRA_SMALL(false, 2, false, true);
+            else if (per_wave <= 4) LYRA_SMALL(false, 4, false, true);
+            else LYRA_SMALL(false, 4, false, false);
+        }
+#undef LYRA_SMALL
         return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
     }
     const dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);

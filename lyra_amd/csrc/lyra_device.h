@@ -19,6 +19,10 @@ typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
 constexpr int kWave = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 
+// A buffer-load lane offset beyond any buffer descriptor used here (all are shorter than 2 GiB; the constant
+// offsets added to it stay far below 4 GiB): such a load returns zeros without touching memory.
+constexpr int kNoLoad = (int)0x80000000u;
+
 // D(16x16,f32) += A(16x32,bf16) * B(32x16,bf16).  Lane l supplies row (l & 15) of A and column
 // (l & 15) of B, each as the 8 consecutive k-slots of k-group (l >> 4); both operands use the same
 // slot -> k mapping, so only "same k in the same slot" matters.  Lane l receives D[4*(l>>4)+r][l&15]
