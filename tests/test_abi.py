@@ -1,0 +1,77 @@
+"""The C-ABI shared library: every function include/lyra_hip.h declares is exported, the Python binding table covers
+them all, and argument validation answers before anything touches a GPU (no compute is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lyra_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lyra_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("lyra_decode_attention", "lyra_decode_attention_workspace", "lyra_decode_gemm", "lyra_decode_gemm_workspace",
+                 "lyra_strerror", "lyra_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from lyra_amd import _lib
+
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(raw, name), f"{name} is declared in include/lyra_hip.h but not exported by liblyra_hip.so"
+    assert set(_lib.SIGNATURES) == set(declared_functions())
+
+
+def test_abi_version_and_error_strings():
+    from lyra_amd import _lib
+
+    text = open(HEADER).read()
+    assert _lib.lib.lyra_abi_version() == int(re.search(r"#define LYRA_ABI_VERSION (\d+)", text).group(1)) == _lib.ABI_VERSION
+    seen = set()
+    for code in (0, -1, -2, -3, -4):
+        msg = _lib.lib.lyra_strerror(code).decode()
+        assert msg and msg not in seen
+        seen.add(msg)
+    with pytest.raises(_lib.LyraHipError):
+        _lib.check(-2, "probe")
+
+
+def test_argument_validation_needs_no_gpu():
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    bad = L.lyra_decode_attention(None, None, None, None, None, None, None, 0, None, None, None, 0, 1, 16, 4, 512, 128, 0.1, 0, 0, 0, None)
+    assert bad == -1
+    one = ctypes.c_void_p(256)  # never dereferenced: shapes are rejected first
+    assert L.lyra_decode_attention(one, one, one, None, None, one, one, 0, None, one, None, 0, 1, 16, 5, 512, 128, 0.1, 0, 0, 0, None) == -1  # N % K
+    assert L.lyra_decode_attention(one, one, one, None, None, one, one, 0, None, one, None, 0, 1, 16, 4, 512, 96, 0.1, 0, 0, 0, None) == -2  # head dim
+    assert L.lyra_decode_gemm(None, None, None, 0, 0, None, None, None, None, 0, 4, 1, 64, 128, 0, 0, 0, 1.702, 7.0, None) == -1
+    assert L.lyra_decode_gemm(one, one, None, 0, 0, one, None, one, None, 0, 4, 1, 48, 128, 0, 0, 0, 1.702, 7.0, None) == -2  # K % 32
+    assert L.lyra_decode_gemm(one, one, None, 0, 0, one, None, one, None, 0, 4, 1, 64, 128, 1, 0, 0, 1.702, 7.0, None) == -1  # fp8 without scales
+    assert L.lyra_rmsnorm_proj(None, None, None, None, None, None, 1, 64, 0, 2, 1e-5, None) == -1
+    assert L.lyra_qkv_post(one, None, None, one, one, one, 0, one, one, one, None, None, 1, 4, 2, 16, 96, 16, 0, 1e-5, None) == -2
+    assert L.lyra_moe_route(one, one, one, one, one, 4, 15, 1, 9, None) == -2  # more than 8 routed picks
+    assert L.lyra_moe_combine(None, None, None, None, None, 1, 1, 1, 1.0, None) == -1
+
+
+def test_workspace_sizes_are_host_arithmetic():
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    small = L.lyra_decode_attention_workspace(1, 16, 4, 512, 128, 0)
+    big = L.lyra_decode_attention_workspace(64, 16, 4, 4096, 128, 0)
+    assert small % 256 == 0 and big % 256 == 0 and big >= small > 0
+    assert L.lyra_decode_attention_workspace(0, 16, 4, 512, 128, 0) == 0
+    moe = L.lyra_decode_gemm_workspace(256, 16, 2048, 4096, 1)
+    assert moe % 256 == 0 and moe >= 256
+    assert L.lyra_decode_gemm_workspace(64, 1, 2048, 3072, 0) == 256  # dense projections run in one pass, no partials

@@ -1,0 +1,177 @@
+"""Host-side mirror of the reference's plugin interface on CPU tensors: QArray arithmetic, dispatch contract, the
+plain-framework ("xla") paths of both operators and the decode-step driver, each against the oracle."""
+from dataclasses import replace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decode_step as D
+from oracle import lyra_oracle as O
+
+
+def _bf16(x):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16)
+
+
+def test_quantize_dequantize_bit_exact_with_oracle():
+    from lyra_amd.nn.quant import QArray, dequantize, qupdate, quantize
+
+    rng = np.random.default_rng(7)
+    x = O.bf16_round(rng.standard_normal((2, 3, 8, 64), dtype=np.float32) * 5)
+    x[0, 0, 0] = 0
+    q = quantize(_bf16(x), torch.float8_e4m3fn, (1, 64))
+    oq, osc = O.quantize(x, (1, 64))
+    assert np.array_equal(q.qval.view(torch.uint8).numpy(), oq) and np.array_equal(q.scale.numpy(), osc)
+    assert q.scale.shape == (2, 3, 8, 1) and q.block == (1, 64) and q.dtype == torch.float8_e4m3fn and q.shape == (2, 3, 8, 64)
+    assert np.array_equal(dequantize(q, torch.bfloat16).float().numpy(), O.dequantize(oq, osc, (1, 64)))
+    w = O.bf16_round(rng.standard_normal((2, 512, 256), dtype=np.float32) * 0.05)
+    qw = quantize(_bf16(w), torch.float8_e4m3fn, (256, 256))
+    ow, ows = O.quantize(w, (256, 256))
+    assert np.array_equal(qw.qval.view(torch.uint8).numpy(), ow) and np.array_equal(qw.scale.numpy(), ows) and qw.scale.shape == (2, 2, 1)
+    # functional update of one token, inputs untouched (quant.py:89-98)
+    new = O.bf16_round(rng.standard_normal((2, 3, 1, 64), dtype=np.float32))
+    before = q.qval.view(torch.uint8).clone()
+    upd = qupdate(q, _bf16(new), (0, 0, 5, 0))
+    assert torch.equal(q.qval.view(torch.uint8), before) and isinstance(upd, QArray)
+    nq, ns = O.quantize(new, (1, 64))
+    assert np.array_equal(upd.qval.view(torch.uint8)[:, :, 5].numpy(), nq[:, :, 0]) and np.array_equal(upd.scale[:, :, 5].numpy(), ns[:, :, 0])
+    with pytest.raises(ValueError):
+        quantize(q, torch.float8_e4m3fn, (1, 32))
+    with pytest.raises(ValueError):
+        quantize(_bf16(x), torch.bfloat16, (1, 64))
+
+
+def test_dispatch_contract():
+    from lyra_amd.kernels.common import dispatch_kernel
+
+    calls = []
+    k = lambda: calls.append("kernel") or torch.zeros(1)
+    r = lambda: calls.append("reference") or torch.zeros(1)
+    common = dict(shape="s", tiling="t", kernel=k, reference=r)
+    dispatch_kernel("op", implementation="auto", config=object(), **common)
+    dispatch_kernel("op", implementation="pallas", config=object(), **common)
+    dispatch_kernel("op", implementation="xla", config=object(), **common)
+    dispatch_kernel("op", implementation="auto", config=None, **common)
+    assert calls == ["kernel", "kernel", "reference", "reference"]
+    with pytest.raises(ValueError, match="no HIP kernel configuration supports inputs"):
+        dispatch_kernel("op", implementation="pallas", config=None, **common)
+    with pytest.raises(ValueError):
+        dispatch_kernel("op", implementation="cuda", config=None, **common)
+
+
+def test_operator_selectors_are_decode_only():
+    from lyra_amd.kernels.op import Mode, attn_op, gmm_op
+
+    assert attn_op(Mode.DECODE, "xla").keywords == {"implementation": "xla"}
+    assert gmm_op(Mode.DECODE, "auto").func.__name__ == "decode_gemm"
+    for mode in Mode:
+        if mode is not Mode.DECODE:
+            with pytest.raises((ValueError, NotImplementedError)):
+                attn_op(mode, "auto")
+
+
+@pytest.mark.parametrize("fp8,sw", [(False, 0), (True, 0), (True, 128)])
+def test_decode_attention_plain_path_on_cpu_matches_oracle(fp8, sw):
+    from lyra_amd.kernels.decode_attention import decode_attention
+    from lyra_amd.nn.quant import QArray
+
+    rng = np.random.default_rng(3)
+    B, N, K, S, H = 2, 8, 2, 384, 64
+    q = O.bf16_round(rng.standard_normal((B, N, 1, H), dtype=np.float32))
+    k = O.bf16_round(rng.standard_normal((B, K, S, H), dtype=np.float32))
+    v = O.bf16_round(rng.standard_normal((B, K, S, H), dtype=np.float32))
+    sinks = rng.standard_normal(N).astype(np.float32)
+    pos = 300
+    if fp8:
+        (kq, ks), (vq, vs) = O.quantize(k, (1, H)), O.quantize(v, (1, H))
+        kt = QArray(torch.from_numpy(kq).view(torch.float8_e4m3fn), torch.from_numpy(ks), (1, H))
+        vt = QArray(torch.from_numpy(vq).view(torch.float8_e4m3fn), torch.from_numpy(vs), (1, H))
+        want = O.decode_attention_reference(q, (kq, ks), (vq, vs), sinks, H**-0.5, sw, pos, mode="fp32")
+    else:
+        kt, vt = _bf16(k), _bf16(v)
+        want = O.decode_attention_reference(q, k, v, sinks, H**-0.5, sw, pos, mode="fp32")
+    got = decode_attention(_bf16(q), kt, vt, torch.from_numpy(sinks), H**-0.5, sw, torch.tensor(pos, dtype=torch.int32), implementation="auto")
+    assert got.shape == (B, N, 1, H) and got.dtype == torch.bfloat16
+    np.testing.assert_allclose(got.float().numpy(), want, atol=2e-2, rtol=1e-2)
+    with pytest.raises(ValueError):  # CPU tensors have no HIP kernel
+        decode_attention(_bf16(q), kt, vt, torch.from_numpy(sinks), H**-0.5, sw, torch.tensor(pos, dtype=torch.int32), implementation="pallas")
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_decode_gemm_plain_path_on_cpu_matches_oracle(fp8):
+    from lyra_amd.kernels.decode_gemm import decode_gemm
+    from lyra_amd.nn.quant import quantize
+
+    rng = np.random.default_rng(4)
+    sizes = np.asarray([3, 0, 2, 4], np.int32)
+    M, K, N = 11, 128, 256  # two rows past the last group
+    lhs = O.bf16_round(rng.standard_normal((M, K), dtype=np.float32))
+    w = O.bf16_round((rng.standard_normal((4, K, N)) * 0.05).astype(np.float32))
+    bias = rng.standard_normal((4, N)).astype(np.float32)
+    if fp8:
+        wq = quantize(_bf16(w), torch.float8_e4m3fn, (128, 256))
+        got = decode_gemm(_bf16(lhs), wq, torch.from_numpy(sizes), bias=torch.from_numpy(bias), fused_swiglu=True,
+                          quant_dtype=torch.float8_e4m3fn, implementation="xla")
+        want = O.decode_gemm_reference(lhs, O.quantize(w, (128, 256)), sizes, block=(128, 256), bias=bias, fused_swiglu=True, mode="fp32")
+    else:
+        got = decode_gemm(_bf16(lhs), _bf16(w), torch.from_numpy(sizes), bias=torch.from_numpy(bias), fused_swiglu=True, implementation="xla")
+        want = O.decode_gemm_reference(lhs, w, sizes, bias=bias, fused_swiglu=True, mode="fp32")
+    assert got.shape == (M, N // 2) and got.dtype == torch.bfloat16
+    np.testing.assert_allclose(got.float().numpy(), want, atol=2e-2, rtol=1e-2)
+
+
+def test_routing_and_permutation_match_oracle():
+    from lyra_amd.model import MODEL_VARIANTS, MoEWeights, bpermute, route_tokens
+
+    cfg = MODEL_VARIANTS["lyra-small"]
+    rng = np.random.default_rng(9)
+    T, C = 12, 64
+    x = O.bf16_round(rng.standard_normal((T, C), dtype=np.float32))
+    router = (rng.standard_normal((C, cfg.n_routed_experts)) * 0.2).astype(np.float32)
+    rbias = rng.standard_normal(cfg.n_routed_experts).astype(np.float32)
+    w = MoEWeights(router=torch.from_numpy(router), router_bias=torch.from_numpy(rbias), mlp_up=None, mlp_down=None, norm_scale=None)
+    scores, active, groups = route_tokens(_bf16(x), w, cfg)
+    logits = x @ router + rbias
+    o_scores, o_active, o_groups = O.route_tokens(logits, cfg.n_active_routed_experts, cfg.n_routed_experts, cfg.n_shared_experts)
+    assert np.array_equal(active.numpy(), o_active) and np.array_equal(groups.numpy(), o_groups)
+    np.testing.assert_allclose(scores.numpy(), o_scores, atol=1e-6)
+    perm, dest = bpermute(active)
+    o_perm, o_dest = O.bpermute(o_active, o_groups, cfg.n_experts)
+    assert np.array_equal(perm.numpy(), o_perm) and np.array_equal(dest.numpy(), o_dest)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_decode_step_driver_on_cpu_matches_oracle(fp8):
+    """model_apply with the plain-framework operators on CPU tensors: the same op sequence as the oracle's decode step."""
+    from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights, model_apply
+
+    cfg = replace(MODEL_VARIANTS["dev"], implementation="xla", seq_len=128, use_sdpa_output_gate=True, sliding_window=128)
+    if fp8:
+        cfg = apply_inference_overrides(cfg, fp8=True)
+    dev = torch.device("cpu")
+    w = init_weights(cfg, dev, seed=1)
+    cache = init_cache(cfg, 2, 128, dev)
+    cache.pos.fill_(0)
+    wn, cn = D.weights_to_numpy(w, cfg), D.cache_to_numpy(cache)
+    tokens = np.asarray([[3, 900], [17, 5]])
+    for s in range(2):
+        got, _ = model_apply(torch.from_numpy(tokens[s]), w, cache, cfg)
+        want = D.decode_step(tokens[s], wn, cn, s, cfg)
+        assert np.isneginf(got[:, cfg.vocab_size :].numpy()).all()
+        np.testing.assert_allclose(got[:, : cfg.vocab_size].numpy(), want[:, : cfg.vocab_size], atol=6e-2, rtol=2e-2)
+    assert int(cache.pos) == 2
+
+
+def test_sampling():
+    from lyra_amd.generate import sample_token
+    from lyra_amd.model import MODEL_VARIANTS
+
+    logits = torch.tensor([[0.0, 3.0, 3.0, -1.0], [5.0, 1.0, 0.0, 4.9]])
+    greedy = replace(MODEL_VARIANTS["dev"], sample_temperature=0.0)
+    assert sample_token(logits, greedy).tolist() == [1, 0]  # ties: lowest index
+    cfg = replace(MODEL_VARIANTS["dev"], sample_temperature=0.8, sample_topk=2)
+    g = torch.Generator().manual_seed(0)
+    draws = torch.stack([sample_token(logits, cfg, g) for _ in range(200)])
+    assert set(draws[:, 0].tolist()) <= {1, 2} and set(draws[:, 1].tolist()) <= {0, 3}
+    assert len(set(draws[:, 0].tolist())) == 2
