@@ -309,7 +309,7 @@ __device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_
     }
 }
 
-template <int H, bool FP8, bool VEC4, int WAVES>
+template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES >= 8 ? 4 : 3)))
 void decode_attention_kernel(AttnParams p) {
     constexpr int ES = FP8 ? 1 : 2;
@@ -323,18 +323,6 @@ void decode_attention_kernel(AttnParams p) {
     const int c_idx = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
     const int G = p.G;
 
-    const int pos = p.position[(size_t)b * p.pos_stride];
-    const Range rg = visible_range(pos, p.sw, p.S);
-    const int c_lo = rg.start + c_idx * p.chunk;
-    if (c_lo > rg.hi) {  // chunk holds no visible key (whole workgroup leaves together)
-        if (p.n_chunks == 1)  // position < 0: only the sink is attended and its value is 0
-            for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64)
-                store_out(p, ((size_t)b * p.N + kh * G) * H + idx, 0.f, 1.f);
-        return;
-    }
-    const int c_hi = min(c_lo + p.chunk, rg.hi + 1);
-    const int n_tiles = (c_hi - c_lo + kTile - 1) / kTile;
-
     const size_t head_row = ((size_t)b * p.K + kh) * p.S;
     Slab sl;
     sl.k = make_rsrc(p.k + head_row * (H * ES), (uint32_t)p.S * (H * ES));
@@ -345,12 +333,44 @@ void decode_attention_kernel(AttnParams p) {
     sl.voff_v = 4 * kb * (H * ES) + x * (H * ES / 16);
     sl.voff_s = 16 * kb;
 
-    // first tile of this wavefront: request it before anything else so it overlaps the q staging
+    // q of this kv head's G query heads (thread t: row t / (H/8), 16-byte piece t % (H/8); rows >= G lie past the end of
+    // the descriptor and read as zeros) and the sink logits: requested first, so that their arrival does not wait for
+    // the cache tiles behind them (loads return in order).
+    const __amdgpu_buffer_rsrc_t qrsrc = make_rsrc(p.q + ((size_t)b * p.N + kh * G) * H, (uint32_t)(G * H * 2));
+    const int q_row = threadIdx.x / (H / 8), q_piece = threadIdx.x % (H / 8);
+    const u32x4 q_raw = __builtin_amdgcn_raw_buffer_load_b128(qrsrc, (q_row * H + q_piece * 8) * 2, 0, 0);
+    const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(p.sinks + kh * G, (uint32_t)(G * 4));
+    const float sink_raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(srsrc, x * 4, 0, 0));
+    __builtin_amdgcn_sched_barrier(0);
+
+    // First tile of this wavefront: requested next.  Without a sliding window the chunk starts at a
+    // key that does not depend on the position, so the request does not wait for the position to arrive (keys past
+    // the end of the slab read as zeros, tiles past the visible range are simply not used).
     RawK<H, FP8> rk;
     RawS rs;
     RawV<H, FP8> rv;
     int tile = wave;
-    {  // (a wavefront without tiles issues the same loads with an offset outside the slab: they fetch nothing)
+    constexpr bool early = EARLY;  // no sliding window
+    const int early_base = c_idx * p.chunk + tile * kTile;
+    if constexpr (early) {
+        load_k<H, FP8>(rk, sl, early_base, true);
+        if constexpr (FP8) load_s<VEC4>(rs, sl, early_base, true);
+        load_v<H, FP8>(rv, sl, early_base, true);
+    }
+
+    const int pos = p.position[(size_t)b * p.pos_stride];
+    const Range rg = visible_range(pos, p.sw, p.S);
+    const int c_lo = rg.start + c_idx * p.chunk;
+    if (c_lo > rg.hi) {  // chunk holds no visible key (whole workgroup leaves together)
+        if (p.n_chunks == 1)  // position < 0: only the sink is attended and its value is 0
+            for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64)
+                store_out(p, ((size_t)b * p.N + kh * G) * H + idx, 0.f, 1.f);
+        wait_all_memory();
+        return;
+    }
+    const int c_hi = min(c_lo + p.chunk, rg.hi + 1);
+    const int n_tiles = (c_hi - c_lo + kTile - 1) / kTile;
+    if constexpr (!early) {  // sliding window: the first key follows from the position
         const bool live = tile < n_tiles;
         load_k<H, FP8>(rk, sl, c_lo + tile * kTile, live);
         if constexpr (FP8) load_s<VEC4>(rs, sl, c_lo + tile * kTile, live);
@@ -360,15 +380,11 @@ void decode_attention_kernel(AttnParams p) {
     // q of this kv head's G query heads, padded to 16 rows of zeros, in LDS: the Q^T operand of lane
     // (head x, k-group kb) is q[x][kb*H/4 + 8c .. +8], the same columns the K lanes hold.
     uint16_t* sm_q = (uint16_t*)smem;
-    for (int idx = threadIdx.x; idx < 16 * (H / 8); idx += WAVES * 64) {
-        const int row = idx / (H / 8), piece = idx - row * (H / 8);
-        u32x4 d = u32x4{0u, 0u, 0u, 0u};
-        if (row < G) d = *(const u32x4*)(p.q + ((size_t)b * p.N + kh * G + row) * H + piece * 8);
-        *(u32x4*)(sm_q + row * QP + piece * 8) = d;
-    }
+    static_assert(WAVES * 64 >= 16 * (H / 8), "one q piece per thread");
+    *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = q_raw;  // every thread stores (rows >= G hold zeros; rows >= 16 are never read)
 
     Acc<H> acc;
-    const float sink2 = x < G ? p.sinks[kh * G + x] * kLog2e : 0.f;
+    const float sink2 = x < G ? sink_raw * kLog2e : 0.f;
     acc.m = fmaxf(sink2, -1e30f);  // finite start: fully masked tiles cannot produce inf - inf
     acc.lsum = 0.f;
 #pragma unroll
@@ -560,7 +576,7 @@ static AttnPlan plan_attention(int B, int K, int S, int sliding_window) {
     if (waves_env == 4 || waves_env == 8 || waves_env == 16) pl.waves = (int)waves_env;
     const int unit = pl.waves * kTile;
     const int max_chunks = (span + unit - 1) / unit;
-    const long target = target_env > 0 ? target_env : 512;  // workgroups
+    const long target = target_env > 0 ? target_env : 256;  // workgroups: one per compute unit
     long want = (target + pairs - 1) / pairs;
     if (span <= 2 * 128) want = 1;  // a window of a few tiles: one workgroup, no merge
     if (pairs > kMaxSplitPairs) want = 1;
@@ -662,11 +678,14 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(pl.n_chunks, K, B), block(pl.waves * 64);
     const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16) * sizeof(float);
-    const size_t lds_q = (size_t)16 * (H + 8) * sizeof(uint16_t);
+    const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
     const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
     const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
-#define LYRA_LAUNCH_ATTN_W(HH, F, V, W) \
-    hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W>), grid, block, lds, st, p)
+#define LYRA_LAUNCH_ATTN_W(HH, F, V, W)                                                                        \
+    do {                                                                                                      \
+        if (sliding_window == 0) hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, true>), grid, block, lds, st, p); \
+        else hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, false>), grid, block, lds, st, p);      \
+    } while (0)
 #define LYRA_LAUNCH_ATTN(HH, F, V)                              \
     do {                                                        \
         if (pl.waves == 4) LYRA_LAUNCH_ATTN_W(HH, F, V, 4);     \
