@@ -309,8 +309,8 @@ __device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_
     }
 }
 
-template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES >= 8 ? 4 : 3)))
+template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY, int DEPTH>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(DEPTH > 1 ? 2 : (WAVES >= 8 ? 4 : 3))))
 void decode_attention_kernel(AttnParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int CB = H / 16;
@@ -346,16 +346,19 @@ void decode_attention_kernel(AttnParams p) {
     // First tile of this wavefront: requested next.  Without a sliding window the chunk starts at a
     // key that does not depend on the position, so the request does not wait for the position to arrive (keys past
     // the end of the slab read as zeros, tiles past the visible range are simply not used).
-    RawK<H, FP8> rk;
-    RawS rs;
-    RawV<H, FP8> rv;
+    RawK<H, FP8> rk[DEPTH];
+    RawS rs[DEPTH];
+    RawV<H, FP8> rv[DEPTH];
     int tile = wave;
     constexpr bool early = EARLY;  // no sliding window
-    const int early_base = c_idx * p.chunk + tile * kTile;
     if constexpr (early) {
-        load_k<H, FP8>(rk, sl, early_base, true);
-        if constexpr (FP8) load_s<VEC4>(rs, sl, early_base, true);
-        load_v<H, FP8>(rv, sl, early_base, true);
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int early_base = c_idx * p.chunk + (tile + d * WAVES) * kTile;
+            load_k<H, FP8>(rk[d], sl, early_base, true);
+            if constexpr (FP8) load_s<VEC4>(rs[d], sl, early_base, true);
+            load_v<H, FP8>(rv[d], sl, early_base, true);
+        }
     }
 
     const int pos = p.position[(size_t)b * p.pos_stride];
@@ -371,14 +374,16 @@ void decode_attention_kernel(AttnParams p) {
     const int c_hi = min(c_lo + p.chunk, rg.hi + 1);
     const int n_tiles = (c_hi - c_lo + kTile - 1) / kTile;
     if constexpr (!early) {  // sliding window: the first key follows from the position
-        const bool live = tile < n_tiles;
-        load_k<H, FP8>(rk, sl, c_lo + tile * kTile, live);
-        if constexpr (FP8) load_s<VEC4>(rs, sl, c_lo + tile * kTile, live);
-        load_v<H, FP8>(rv, sl, c_lo + tile * kTile, live);
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const bool live = tile + d * WAVES < n_tiles;
+            const int base = c_lo + (tile + d * WAVES) * kTile;
+            load_k<H, FP8>(rk[d], sl, base, live);
+            if constexpr (FP8) load_s<VEC4>(rs[d], sl, base, live);
+            load_v<H, FP8>(rv[d], sl, base, live);
+        }
     }
 
-    // q of this kv head's G query heads, padded to 16 rows of zeros, in LDS: the Q^T operand of lane
-    // (head x, k-group kb) is q[x][kb*H/4 + 8c .. +8], the same columns the K lanes hold.
     uint16_t* sm_q = (uint16_t*)smem;
     static_assert(WAVES * 64 >= 16 * (H / 8), "one q piece per thread");
     *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = q_raw;  // every thread stores (rows >= G hold zeros; rows >= 16 are never read)
@@ -395,33 +400,42 @@ void decode_attention_kernel(AttnParams p) {
     // without touching memory): the number of loads in flight is then identical on every path and each wait covers
     // exactly the loads it needs.
     // Software pipeline over this wavefront's tiles (wave, wave + WAVES, ...: a fixed assignment, so results are
-    // bit-reproducible from run to run) with a single register set: each operand of the
-    // next tile is requested right after the last use of the current one, so the loads fly during the rest
-    // of the iteration and no registers are spent on a second buffer.
+    // bit-reproducible from run to run) with DEPTH register sets (1 as instantiated: two tiles in flight per wavefront
+    // measured no faster): each operand of the next tile of a set is requested right after the last use of the
+    // current one, so the loads fly during the rest of the iteration.
     while (tile < n_tiles) {
-        const int next_tile = tile + WAVES;
-        const int base = c_lo + tile * kTile;
-        const int next = c_lo + next_tile * kTile;
-        const bool more = next_tile < n_tiles;
-        const bool full = base >= rg.lo && base + kTile - 1 <= rg.hi;
-        f32x4 s[2];
-        tile_logits<H, FP8>(rk, sm_q, lane, s);
-        __builtin_amdgcn_sched_barrier(0);
-        load_k<H, FP8>(rk, sl, next, more);
-        __builtin_amdgcn_sched_barrier(0);
-        uint32_t vis;
-        bf16x8 pop;
-        if (full) pop = tile_softmax<H, FP8, false>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
-        else pop = tile_softmax<H, FP8, true>(s, rs, base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (FP8) load_s<VEC4>(rs, sl, next, more);
-        __builtin_amdgcn_sched_barrier(0);
-        if (full) tile_values<H, FP8, false>(rv, pop, vis, acc);
-        else tile_values<H, FP8, true>(rv, pop, vis, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        load_v<H, FP8>(rv, sl, next, more);
-        __builtin_amdgcn_sched_barrier(0);
-        tile = next_tile;
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int cur = tile + d * WAVES;         // tile held in register set d (zeros past the end: skipped)
+            const int next_tile = cur + DEPTH * WAVES;  // tile requested into the same set
+            const int base = c_lo + cur * kTile;
+            const int next = c_lo + next_tile * kTile;
+            const bool more = next_tile < n_tiles;
+            const bool live = cur < n_tiles;
+            const bool full = base >= rg.lo && base + kTile - 1 <= rg.hi;
+            f32x4 s[2];
+            if (live) tile_logits<H, FP8>(rk[d], sm_q, lane, s);
+            __builtin_amdgcn_sched_barrier(0);
+            load_k<H, FP8>(rk[d], sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+            uint32_t vis = 0;
+            bf16x8 pop;
+            if (live) {
+                if (full) pop = tile_softmax<H, FP8, false>(s, rs[d], base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
+                else pop = tile_softmax<H, FP8, true>(s, rs[d], base, rg.lo, rg.hi, p.scale_log2, lane, acc, vis);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (FP8) load_s<VEC4>(rs[d], sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+            if (live) {
+                if (full) tile_values<H, FP8, false>(rv[d], pop, vis, acc);
+                else tile_values<H, FP8, true>(rv[d], pop, vis, acc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            load_v<H, FP8>(rv[d], sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        tile += DEPTH * WAVES;
     }
     acc.lsum = group4_sum(acc.lsum);
 
@@ -572,7 +586,6 @@ static AttnPlan plan_attention(int B, int K, int S, int sliding_window) {
     const long pairs = (long)B * K;
     AttnPlan pl;
     pl.waves = 4;
-    if (pairs >= 192 && span >= 2048) pl.waves = 8;  // one big workgroup per pair instead of chunks
     if (waves_env == 4 || waves_env == 8 || waves_env == 16) pl.waves = (int)waves_env;
     const int unit = pl.waves * kTile;
     const int max_chunks = (span + unit - 1) / unit;
@@ -683,8 +696,8 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
 #define LYRA_LAUNCH_ATTN_W(HH, F, V, W)                                                                        \
     do {                                                                                                      \
-        if (sliding_window == 0) hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, true>), grid, block, lds, st, p); \
-        else hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, false>), grid, block, lds, st, p);      \
+        if (sliding_window == 0) hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, true, 1>), grid, block, lds, st, p); \
+        else hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, false, 1>), grid, block, lds, st, p);      \
     } while (0)
 #define LYRA_LAUNCH_ATTN(HH, F, V)                              \
     do {                                                        \

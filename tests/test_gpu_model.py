@@ -25,9 +25,13 @@ def _run_steps(cfg, B, S, steps, start):
     # a synthetic history: every cached row below `start` holds N(0,1) keys/values
     from lyra_amd.nn.quant import QArray, quantize
 
+    # (seeded: top-1 routing is a discontinuous function of the activations, so an unlucky history can put a router
+    # logit pair within bf16 noise of a tie and send one token to a different expert than the float32-exact oracle)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2024)
     for layer in cache.layers:
         for name in ("k", "v"):
-            hist = torch.randn(B, cfg.n_kv_heads, start, cfg.head_dim, device=dev).to(torch.bfloat16)
+            hist = torch.randn(B, cfg.n_kv_heads, start, cfg.head_dim, device=dev, generator=gen).to(torch.bfloat16)
             dst = getattr(layer, name)
             if isinstance(dst, QArray):
                 q = quantize(hist, dst.dtype, dst.block)
