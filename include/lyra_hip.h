@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 3
+#define LYRA_ABI_VERSION 4
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -160,6 +160,16 @@ int lyra_moe_route(const float* logits, float* scores, int32_t* groups, int32_t*
                    int n_routed, int n_shared, int k_routed, lyra_stream_t stream);
 int lyra_moe_combine(const void* rows, const float* scores, const int32_t* dest, const void* x, void* out, int tokens, int topk,
                      int C, float residual_scale, lyra_stream_t stream);
+
+/*
+ * Greedy sampling (lyra/generate.py:46-53 with temperature <= 0): out[r] = first index of the maximum of
+ * x[r, 0:cols], x float32 [rows, ld] (ld >= cols is the padded vocabulary; the padding is not looked at).
+ * workspace: lyra_argmax_workspace bytes, 256-byte aligned, zero on first use (it holds arrival counters that
+ * every call returns to zero, like the attention workspace).  ld % 4 == 0, x 16-byte aligned.
+ */
+int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols, int ld,
+                lyra_stream_t stream);
+size_t lyra_argmax_workspace(int rows, int cols);
 
 /*
  * Self-check of the matrix-core register layouts and FP8 conversions the kernels rely on.

@@ -37,7 +37,7 @@ struct NormProjParams {
     float eps;
 };
 
-constexpr int kNormThreads = 512;
+constexpr int kNormThreads = 1024;
 
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjParams p) {
     extern __shared__ float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
@@ -72,12 +72,22 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int j = wave; j < p.n; j += kNormThreads / 64) {
-        const float* pr = p.proj_t + (size_t)j * p.C;
+        // one output per wavefront at a time; its weight row is requested 8 x 16 bytes per lane at once (offsets past
+        // the row read as zeros), so a row of up to 2048 columns costs one memory round trip
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.proj_t) + (size_t)j * p.C, 0,
+                                                                            (uint32_t)p.C * 4u, 0x00020000);
         float acc = 0.f;
-        for (int c = lane * 4; c < p.C; c += 256) {
-            const f32x4 w = *(const f32x4*)(pr + c);
-            const f32x4 hv = *(const f32x4*)(sm_h + c);
-            acc += hv[0] * w[0] + hv[1] * w[1] + hv[2] * w[2] + hv[3] * w[3];
+        for (int c0 = 0; c0 < p.C; c0 += 2048) {
+            u32x4 w[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (c0 + i * 256 + lane * 4) * 4, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = min(c0 + i * 256 + lane * 4, p.C - 4);  // (clamped reads meet zero weights)
+                const f32x4 hv = *(const f32x4*)(sm_h + c);
+                acc += hv[0] * __uint_as_float(w[i][0]) + hv[1] * __uint_as_float(w[i][1]) + hv[2] * __uint_as_float(w[i][2]) +
+                       hv[3] * __uint_as_float(w[i][3]);
+            }
         }
         float v = wave_sum(acc);
         if (lane == 0) {
@@ -185,6 +195,7 @@ struct RouteParams {
     int32_t* row_map;     // [tokens * topk]: token of each sorted row   (permute_map // topk)
     int32_t* dest;        // [tokens * topk]: sorted row of each assignment (unpermute_map)
     int tokens, n_routed, n_shared, k_routed;
+    int stage_logits;
 };
 
 __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
@@ -193,10 +204,13 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
     int* sm_expert = sm_i;        // [M]
     int* sm_count = sm_i + M;     // [E]
     int* sm_start = sm_count + E; // [E]
+    float* sm_logits = (float*)(sm_start + E);  // [tokens * n_routed] when p.stage_logits (coalesced copy, then row reads)
     for (int e = threadIdx.x; e < E; e += blockDim.x) sm_count[e] = 0;
+    if (p.stage_logits)
+        for (int i = threadIdx.x; i < p.tokens * p.n_routed; i += blockDim.x) sm_logits[i] = p.logits[i];
     __syncthreads();
     for (int t = threadIdx.x; t < p.tokens; t += blockDim.x) {
-        const float* lg = p.logits + (size_t)t * p.n_routed;
+        const float* lg = (p.stage_logits ? sm_logits : p.logits) + (size_t)t * p.n_routed;
         float top[8];
         int idx[8];
         unsigned long long taken_lo = 0ull, taken_hi = 0ull;  // up to 128 routed experts
@@ -266,15 +280,95 @@ struct CombineParams {
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
     const int f = blockIdx.x;
-    for (int c = threadIdx.x; c < p.C; c += blockDim.x) {
-        float acc = 0.f;
+    for (int c = threadIdx.x * 8; c < p.C; c += blockDim.x * 8) {  // C % 8 == 0: 16 bytes per thread and row
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
         for (int k = 0; k < p.topk; ++k) {
             const int r = p.dest[f * p.topk + k];
-            acc += bf16_bits_to_f32(p.rows[(size_t)r * p.C + c]) * p.scores[f * p.topk + k];
+            const float sc = p.scores[f * p.topk + k];
+            const u32x4 d = *(const u32x4*)(p.rows + (size_t)r * p.C + c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] += __uint_as_float(d[i] << 16) * sc;
+                acc[2 * i + 1] += __uint_as_float(d[i] & 0xFFFF0000u) * sc;
+            }
         }
-        const float t = bf16r(bf16r(acc) * p.residual_scale);
-        p.out[(size_t)f * p.C + c] = f32_to_bf16_bits(bf16_bits_to_f32(p.x[(size_t)f * p.C + c]) + t);
+        const u32x4 xd = *(const u32x4*)(p.x + (size_t)f * p.C + c);
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float t0 = bf16r(bf16r(acc[2 * i]) * p.residual_scale), t1 = bf16r(bf16r(acc[2 * i + 1]) * p.residual_scale);
+            o[i] = pack_bf16(__uint_as_float(xd[i] << 16) + t0, __uint_as_float(xd[i] & 0xFFFF0000u) + t1);
+        }
+        *(u32x4*)(p.out + (size_t)f * p.C + c) = o;
     }
+}
+
+// ---- greedy sampling: first index of the row maximum ---------------------------------------------------------
+// lyra/generate.py:46-53 with temperature 0 (argmax over the vocabulary; columns >= cols, the padding of the
+// vocabulary, are not looked at).  Grid (chunks, rows): every workgroup reduces one chunk of a row to (max, first
+// index) and publishes it; the workgroup that arrives last for the row picks among the chunks.
+struct ArgmaxParams {
+    const float* x;
+    int32_t* out;
+    float* part_v;   // [rows, chunks]
+    int* part_i;     // [rows, chunks]
+    int* arrivals;   // [rows] zero on entry, zero again on exit
+    int rows, cols, ld, chunks, chunk_len;
+};
+
+__device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) {
+        bv = v;
+        bi = i;
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
+    __shared__ float sm_v[4];
+    __shared__ int sm_i[4];
+    __shared__ int sm_last;
+    const int c = blockIdx.x, row = blockIdx.y;
+    const float* xr = p.x + (size_t)row * p.ld;
+    const int lo = c * p.chunk_len, hi = min(lo + p.chunk_len, p.cols);
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = lo + threadIdx.x * 4; i < hi; i += 1024) {  // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads
+        if (i + 4 <= hi) {
+            const f32x4 v = *(const f32x4*)(xr + i);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) take_better(bv, bi, v[k], i + k);
+        } else {
+            for (int k = 0; i + k < hi; ++k) take_better(bv, bi, xr[i + k], i + k);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) {
+        sm_v[wave] = bv;
+        sm_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w) take_better(bv, bi, sm_v[w], sm_i[w]);
+        store_agent(&p.part_v[row * p.chunks + c], bv);
+        store_agent(&p.part_i[row * p.chunks + c], bi);
+        wait_all_memory();
+        const int seen = add_agent(&p.arrivals[row], 1);
+        sm_last = seen == p.chunks - 1;
+        if (sm_last) store_agent(&p.arrivals[row], 0);
+    }
+    __syncthreads();
+    if (!sm_last || threadIdx.x >= 64) return;
+    bv = -INFINITY;
+    bi = 0x7FFFFFFF;
+    for (int k = threadIdx.x; k < p.chunks; k += 64)
+        take_better(bv, bi, load_agent(&p.part_v[row * p.chunks + k]), __hip_atomic_load(&p.part_i[row * p.chunks + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+    if (threadIdx.x == 0) p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
 }
 
 }  // namespace lyra
@@ -318,9 +412,12 @@ extern "C" int lyra_moe_route(const float* logits, float* scores, int32_t* group
     if (tokens <= 0 || n_routed <= 0 || n_shared < 0 || k_routed <= 0) return LYRA_E_BADARG;
     if (k_routed > 8 || k_routed > n_routed || n_routed > 128) return LYRA_E_UNSUPPORTED;
     const int topk = k_routed + n_shared, E = n_routed + n_shared;
-    const size_t lds = ((size_t)tokens * topk + 2 * E) * sizeof(int);
+    size_t lds = ((size_t)tokens * topk + 2 * E) * sizeof(int);
     if (lds > 60000) return LYRA_E_UNSUPPORTED;
-    RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed};
+    const size_t staged = (size_t)tokens * n_routed * sizeof(float);
+    const int stage = lds + staged <= 64000;
+    if (stage) lds += staged;
+    RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed, stage};
     const int threads = std::min(1024, std::max(64, (tokens * topk + 63) / 64 * 64));
     hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
@@ -330,7 +427,47 @@ extern "C" int lyra_moe_combine(const void* rows, const float* scores, const int
                                 int topk, int C, float residual_scale, lyra_stream_t stream) {
     using namespace lyra;
     if (!rows || !scores || !dest || !x || !out || tokens <= 0 || topk <= 0 || C <= 0) return LYRA_E_BADARG;
+    if (C % 8) return LYRA_E_UNSUPPORTED;
     CombineParams p{(const uint16_t*)rows, scores, dest, (const uint16_t*)x, (uint16_t*)out, tokens, topk, C, residual_scale};
     hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+namespace lyra {
+// The arrival counters take a fixed region at the start of the workspace whatever the shape, so that calls of
+// different shapes sharing one workspace never leave partial results where another call expects zeroed counters.
+constexpr size_t kArgmaxCounterBytes = 65536 * sizeof(int);
+static int argmax_chunks(int rows, int cols) {
+    const int want = std::max(1, 512 / std::max(1, rows));             // ~2 workgroups per compute unit
+    const int most = std::max(1, (cols + 4095) / 4096);                // at least 4096 columns per workgroup
+    return std::min(std::min(want, most), 64);
+}
+}  // namespace lyra
+
+extern "C" size_t lyra_argmax_workspace(int rows, int cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    return lyra::kArgmaxCounterBytes + ((size_t)rows * lyra::argmax_chunks(rows, cols) * 8 + 255) / 256 * 256;
+}
+
+extern "C" int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols, int ld,
+                           lyra_stream_t stream) {
+    using namespace lyra;
+    if (!x || !out || rows <= 0 || cols <= 0 || ld < cols) return LYRA_E_BADARG;
+    if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535) return LYRA_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < lyra_argmax_workspace(rows, cols) || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
+    ArgmaxParams p;
+    p.x = x;
+    p.out = out;
+    p.rows = rows;
+    p.cols = cols;
+    p.ld = ld;
+    p.chunks = argmax_chunks(rows, cols);
+    p.chunk_len = ((cols + p.chunks - 1) / p.chunks + 3) / 4 * 4;
+    p.chunks = (cols + p.chunk_len - 1) / p.chunk_len;
+    const size_t counters = kArgmaxCounterBytes;
+    p.arrivals = (int*)workspace;
+    p.part_v = (float*)((char*)workspace + counters);
+    p.part_i = (int*)(p.part_v + (size_t)rows * argmax_chunks(rows, cols));
+    hipLaunchKernelGGL(argmax_kernel, dim3(p.chunks, rows), dim3(256), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }

@@ -236,10 +236,8 @@ void decode_gemm_kernel(GemmParams p) {
         // One register set of raw weights: a pair of rows is requested again (for the next step) as soon as it
         // has been converted, so weight loads are in flight during the whole step.
         RawW<FP8> w;
-        if (k0 < k1) {
 #pragma unroll
-            for (int pr = 0; pr < 4; ++pr) load_w_pair<FP8>(w, pr, wrsrc, wvoff, k0, row_bytes);
-        }
+        for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(k0 < k1, w, pr, wrsrc, wvoff, k0, row_bytes);
 
         for (int kc = k0; kc < k1; kc += KC) {
             const int kc_end = min(kc + KC, k1);
@@ -285,7 +283,7 @@ void decode_gemm_kernel(GemmParams p) {
                 for (int pr = 0; pr < 4; ++pr) {
                     convert_pair<FP8>(w, pr, bop);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (more) load_w_pair<FP8>(w, pr, wrsrc, wvoff, kk + 32, row_bytes);
+                    load_w_pair_if<FP8>(more, w, pr, wrsrc, wvoff, kk + 32, row_bytes);
                     __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll

@@ -1,6 +1,8 @@
 """Generation driver for decode mode (lyra/generate.py of the reference, minus tokenizer and REPL)."""
 from __future__ import annotations
 
+from dataclasses import replace
+
 import torch
 
 from lyra_amd.model import ModelCache, ModelConfig, ModelWeights, model_apply
@@ -10,6 +12,10 @@ def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Genera
     """lyra/generate.py:46-53 applied to each row of ``logits`` [B, V]: greedy when temperature <= 0, else
     temperature scaling, top-k masking (lowest index wins ties, like lax.top_k) and a categorical draw."""
     if cfg.sample_temperature <= 0:
+        if logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla":
+            from lyra_amd.kernels.decode_fused import argmax
+
+            return argmax(logits, min(cfg.vocab_size, logits.shape[-1]))
         return torch.argmax(logits, dim=-1).to(torch.int32)
     logits = logits.to(torch.float32) / cfg.sample_temperature
     if 0 < cfg.sample_topk < logits.shape[-1]:
@@ -56,7 +62,7 @@ class GraphedDecoder:
     def _step(self):
         logits, _ = model_apply(self.tokens, self.model, self.cache, self.cfg)
         self.logits = logits
-        self.next_tokens.copy_(torch.argmax(logits, dim=-1))
+        self.next_tokens.copy_(sample_token(logits, replace(self.cfg, sample_temperature=0.0)))
 
     def step(self) -> torch.Tensor:
         """Run one decode step on ``self.tokens``; returns the greedy next tokens (device, int32)."""

@@ -151,3 +151,17 @@ def moe_combine(rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, x:
                              float(residual_scale), _stream(x.device))
     _lib.check(rc, "lyra_moe_combine")
     return out
+
+
+def argmax(logits: torch.Tensor, cols: int | None = None) -> torch.Tensor:
+    """Greedy token choice (lyra/generate.py:46-53 at temperature 0): first index of each row's maximum over the first
+    ``cols`` columns of float32 ``logits`` [rows, ld]; returns int32 [rows]."""
+    rows, ld = logits.shape
+    cols = ld if cols is None else cols
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    stream = _stream(logits.device)
+    ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_argmax_workspace(rows, cols))
+    rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, stream)
+    _lib.check(rc, "lyra_argmax")
+    return out

@@ -62,6 +62,8 @@ def test_argument_validation_needs_no_gpu():
     assert L.lyra_qkv_post(one, None, None, one, one, one, 0, one, one, one, None, None, 1, 4, 2, 16, 96, 16, 0, 1e-5, None) == -2
     assert L.lyra_moe_route(one, one, one, one, one, 4, 15, 1, 9, None) == -2  # more than 8 routed picks
     assert L.lyra_moe_combine(None, None, None, None, None, 1, 1, 1, 1.0, None) == -1
+    assert L.lyra_argmax(None, None, None, 0, 1, 1, 4, None) == -1
+    assert L.lyra_argmax(one, one, None, 0, 2, 10, 6, None) == -1  # leading dimension shorter than the row
 
 
 def test_workspace_sizes_are_host_arithmetic():
@@ -70,7 +72,8 @@ def test_workspace_sizes_are_host_arithmetic():
     L = _lib.lib
     small = L.lyra_decode_attention_workspace(1, 16, 4, 512, 128, 0)
     big = L.lyra_decode_attention_workspace(64, 16, 4, 4096, 128, 0)
-    assert small % 256 == 0 and big % 256 == 0 and big >= small > 0
+    assert small % 256 == 0 and big % 256 == 0 and small > 0 and big > 0  # (a launch that is not chunked needs no partials)
+    assert L.lyra_argmax_workspace(64, 201088) % 256 == 0 and L.lyra_argmax_workspace(0, 5) == 0
     assert L.lyra_decode_attention_workspace(0, 16, 4, 512, 128, 0) == 0
     moe = L.lyra_decode_gemm_workspace(256, 16, 2048, 4096, 1)
     assert moe % 256 == 0 and moe >= 256

@@ -247,3 +247,26 @@ def test_fused_model_matches_unfused(fp8):
         outs.append(steps)
     for a, b in zip(*outs):
         U.assert_close(a, b, atol=3e-2, rtol=2e-2, what="fused vs unfused logits")
+
+
+@pytest.mark.parametrize("rows,cols,ld", [(64, 201088, 204800), (3, 1000, 1024), (1, 7, 8), (5, 4097, 4100), (130, 50000, 50000)])
+def test_argmax_first_maximum(rows, cols, ld):
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"argmax rows{rows} cols{cols} ld{ld}")
+    g = torch.Generator(device=U.dev())
+    g.manual_seed(rows + cols)
+    x = torch.randn(rows, ld, generator=g, device=U.dev())
+    x[:, cols:] = 100.0  # padding columns must not win
+    x[0, : min(cols, 5)] = 50.0  # ties: the first index wins
+    if rows > 1:
+        x[1, :cols] = float("-inf")  # a fully masked row picks index 0
+    if rows > 2:
+        x[2, cols - 1] = 60.0  # the last valid column
+    for _ in range(2):  # twice: the arrival counters must be back at zero
+        got = F.argmax(x, cols).cpu().numpy()
+        want = torch.argmax(x[:, :cols], dim=-1).cpu().numpy()
+        want[0] = 0
+        if rows > 1:
+            want[1] = 0
+        assert np.array_equal(got, want)
