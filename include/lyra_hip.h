@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 4
+#define LYRA_ABI_VERSION 5
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -119,6 +119,21 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
                         lyra_stream_t stream);
 
 /*
+ * A dense projection (one group, a few MB of weights) runs split over K across all compute units; the float32
+ * slices [splits, M, N] are summed by whoever consumes the result.  lyra_decode_gemm(_ex) sums them itself in a
+ * second launch.  A decode step saves that launch by handing the unsummed slices to the next kernel of the layer
+ * (lyra_qkv_post_sum after the q/k/v projection, lyra_rmsnorm_proj_sum after the output and down projections):
+ *   lyra_decode_gemm_splits    number of slices for (M, K, N, bk) - shape only; 0 = this shape does not run split
+ *   lyra_decode_gemm_partials  partials[s] = lhs[:, slice s] @ rhs[slice s, :] (weight scales applied), no epilogue;
+ *                              partials holds splits * M * N floats, 16-byte aligned.
+ * The sum over slices is taken in slice order in float32, then rounded as the projection's bf16 output would be.
+ */
+int lyra_decode_gemm_splits(int M, int K, int N, int bk);
+int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
+                              const int32_t* group_sizes, float* partials, size_t partials_bytes, int M, int K, int N,
+                              int rhs_dtype, lyra_stream_t stream);
+
+/*
  * The elementwise steps of a decode layer between the two kernels above, one launch each.  They follow the
  * reference's dtype flow exactly: float32 arithmetic inside an op, a bf16 rounding wherever its JAX code holds a
  * bf16 array.
@@ -131,6 +146,11 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
  */
 int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C,
                       int n, int mode, float eps, lyra_stream_t stream);
+/* Same, but the row to normalise is first formed from unsummed projection slices (lyra/model.py:371-374, 631-636):
+ * x_out = bf16(residual + bf16(bf16(sum_s partials[s]) * out_scale)), partials [splits, B, C] float32; x is ignored. */
+int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale, void* x_out,
+                          const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C, int n,
+                          int mode, float eps, lyra_stream_t stream);
 
 /*
  * lyra_qkv_post: everything between the fused q/k/v projection and the attention kernel (model.py:309-336):
@@ -145,6 +165,11 @@ int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const
                   const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache, float* k_scale,
                   float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype, float eps,
                   lyra_stream_t stream);
+/* Same, reading the projection as unsummed slices partials [splits, B, (N+2K)*H] float32 (qkv is ignored). */
+int lyra_qkv_post_sum(const void* qkv, const float* partials, int splits, const float* qnorm, const float* knorm,
+                      const float* cos_t, const float* sin_t, const int32_t* position, int position_stride, void* q_out,
+                      void* k_cache, void* v_cache, float* k_scale, float* v_scale, int B, int N, int K, int S, int H,
+                      int rope_rows, int kv_dtype, float eps, lyra_stream_t stream);
 
 /*
  * lyra_moe_route: router top-k, softmax over the chosen logits, shared experts appended with score 1, and the stable

@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _c = ctypes
 SIGNATURES = {
@@ -37,6 +37,19 @@ SIGNATURES = {
     ),
     "lyra_moe_route": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 4 + [_c.c_void_p]),
     "lyra_moe_combine": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 3 + [_c.c_float, _c.c_void_p]),
+    "lyra_decode_gemm_splits": (_c.c_int, [_c.c_int] * 4),
+    "lyra_decode_gemm_partials": (
+        _c.c_int,
+        [_c.c_void_p] * 3 + [_c.c_int] * 2 + [_c.c_void_p] * 2 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_void_p],
+    ),
+    "lyra_rmsnorm_proj_sum": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
+    ),
+    "lyra_qkv_post_sum": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
+    ),
     "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p]),
     "lyra_argmax_workspace": (_c.c_size_t, [_c.c_int] * 2),
     "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),

@@ -35,6 +35,13 @@ struct NormProjParams {
     void* y;              // mode 1: bf16 [B, n] gate; mode 2: float32 [B, n]
     int C, n, mode;
     float eps;
+    // optional: the row to normalise is not x but bf16(residual + bf16(bf16(sum_s partials[s]) * out_scale)), the
+    // residual update that follows a projection whose K slices have not been summed yet; it is written to x_out
+    const float* partials;  // [splits, B, C] or null
+    int splits, B;
+    const uint16_t* residual;
+    float out_scale;
+    uint16_t* x_out;
 };
 
 constexpr int kNormThreads = 1024;
@@ -46,7 +53,22 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     const uint16_t* xr = p.x + (size_t)b * p.C;
     float ss = 0.f;
     for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // C % 4 == 0
-        const u32x2 d = *(const u32x2*)(xr + c);
+        u32x2 d;
+        if (p.partials) {
+            f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int sidx = 0; sidx < p.splits; ++sidx) {
+                const f32x4 u = *(const f32x4*)(p.partials + ((size_t)sidx * p.B + b) * p.C + c);
+                t[0] += u[0]; t[1] += u[1]; t[2] += u[2]; t[3] += u[3];
+            }
+            const u32x2 r = *(const u32x2*)(p.residual + (size_t)b * p.C + c);
+            const float r0 = __uint_as_float(r[0] << 16), r1 = __uint_as_float(r[0] & 0xFFFF0000u);
+            const float r2 = __uint_as_float(r[1] << 16), r3 = __uint_as_float(r[1] & 0xFFFF0000u);
+            d[0] = pack_bf16(r0 + bf16r(bf16r(t[0]) * p.out_scale), r1 + bf16r(bf16r(t[1]) * p.out_scale));
+            d[1] = pack_bf16(r2 + bf16r(bf16r(t[2]) * p.out_scale), r3 + bf16r(bf16r(t[3]) * p.out_scale));
+            *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
+        } else {
+            d = *(const u32x2*)(xr + c);
+        }
         const float v0 = __uint_as_float(d[0] << 16), v1 = __uint_as_float(d[0] & 0xFFFF0000u);
         const float v2 = __uint_as_float(d[1] << 16), v3 = __uint_as_float(d[1] & 0xFFFF0000u);
         sm_h[c] = v0; sm_h[c + 1] = v1; sm_h[c + 2] = v2; sm_h[c + 3] = v3;
@@ -120,6 +142,8 @@ struct QkvPostParams {
     float* v_scale;
     int B, N, K, S, H, seq;
     float eps;
+    const float* partials;  // [splits, B, (N + 2K) * H] K slices of the projection not summed yet, or null (then qkv)
+    int splits;
 };
 
 __device__ __forceinline__ uint8_t f32_to_e4m3fn(float v) {  // round to nearest even; |v| <= 448 by construction
@@ -135,9 +159,23 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
     const int b = item / heads, hd = item - b * heads;
     const int half = p.H >> 1;
     const bool active = lane < half;
-    const uint16_t* src = p.qkv + ((size_t)b * heads + hd) * p.H;
-    float a = active ? bf16_bits_to_f32(src[lane]) : 0.f;
-    float c = active ? bf16_bits_to_f32(src[lane + half]) : 0.f;
+    float a = 0.f, c = 0.f;
+    if (p.partials) {
+        if (active) {
+            const size_t slab = (size_t)p.B * heads * p.H;
+            const float* src = p.partials + ((size_t)b * heads + hd) * p.H;
+            for (int sidx = 0; sidx < p.splits; ++sidx) {
+                a += src[sidx * slab + lane];
+                c += src[sidx * slab + lane + half];
+            }
+            a = bf16r(a);  // the projection's output is a bf16 array
+            c = bf16r(c);
+        }
+    } else if (active) {
+        const uint16_t* src = p.qkv + ((size_t)b * heads + hd) * p.H;
+        a = bf16_bits_to_f32(src[lane]);
+        c = bf16_bits_to_f32(src[lane + half]);
+    }
     const int pos = p.position[(size_t)b * p.pos_stride];
     const bool is_q = hd < p.N, is_k = !is_q && hd < p.N + p.K;
     if (is_q || is_k) {
@@ -375,11 +413,19 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
 
 extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
                                  int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
+    return lyra_rmsnorm_proj_sum(x, nullptr, 0, nullptr, 1.0f, nullptr, scale, h, proj_t, bias, y, B, C, n, mode, eps, stream);
+}
+
+extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale,
+                                     void* x_out, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
+                                     int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
     using namespace lyra;
-    if (!x || !scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
+    if (partials ? (!residual || !x_out || splits <= 0) : !x) return LYRA_E_BADARG;
+    if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
-    NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps};
+    NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
+                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out};
     const size_t lds = ((size_t)C + 16) * sizeof(float);
     hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
@@ -389,8 +435,17 @@ extern "C" int lyra_qkv_post(const void* qkv, const float* qnorm, const float* k
                              const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache,
                              float* k_scale, float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype,
                              float eps, lyra_stream_t stream) {
+    return lyra_qkv_post_sum(qkv, nullptr, 0, qnorm, knorm, cos_t, sin_t, position, position_stride, q_out, k_cache, v_cache, k_scale,
+                             v_scale, B, N, K, S, H, rope_rows, kv_dtype, eps, stream);
+}
+
+extern "C" int lyra_qkv_post_sum(const void* qkv, const float* partials, int splits, const float* qnorm, const float* knorm,
+                                 const float* cos_t, const float* sin_t, const int32_t* position, int position_stride, void* q_out,
+                                 void* k_cache, void* v_cache, float* k_scale, float* v_scale, int B, int N, int K, int S, int H,
+                                 int rope_rows, int kv_dtype, float eps, lyra_stream_t stream) {
     using namespace lyra;
-    if (!qkv || !cos_t || !sin_t || !position || !q_out || !k_cache || !v_cache) return LYRA_E_BADARG;
+    if (partials ? splits <= 0 : !qkv) return LYRA_E_BADARG;
+    if (!cos_t || !sin_t || !position || !q_out || !k_cache || !v_cache) return LYRA_E_BADARG;
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || rope_rows <= 0) return LYRA_E_BADARG;
     if (H != 64 && H != 128) return LYRA_E_UNSUPPORTED;
     if ((qnorm == nullptr) != (knorm == nullptr)) return LYRA_E_BADARG;
@@ -399,7 +454,7 @@ extern "C" int lyra_qkv_post(const void* qkv, const float* qnorm, const float* k
     if (fp8 != (k_scale != nullptr) || fp8 != (v_scale != nullptr)) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
     QkvPostParams p{(const uint16_t*)qkv, qnorm, knorm, cos_t, sin_t, position, position_stride, (uint16_t*)q_out,
-                    k_cache, v_cache, k_scale, v_scale, B, N, K, S, H, rope_rows, eps};
+                    k_cache, v_cache, k_scale, v_scale, B, N, K, S, H, rope_rows, eps, partials, splits};
     const int items = B * (N + 2 * K);
     hipLaunchKernelGGL(qkv_post_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;

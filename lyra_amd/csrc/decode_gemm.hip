@@ -581,12 +581,153 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
     }
 }
 
+// ---- one group, a few MB of weights, up to a few dozen rows: split over K across all compute units ----------------
+// A compute unit ingests only ~30-50 GB/s, so a dense projection (4-13 MB of weights) must be spread over all of
+// them with as few bytes per unit as possible.  A workgroup owns 64 rows x 128 columns x one K slice: it reads 1/ks of
+// one column span of the weights once and the matching slice of the activations once (about equal byte counts at 64
+// rows).  Its 4 wavefronts interleave over the slice in steps of 32 rows with everything requested up front; their
+// partial tiles are summed through LDS in a fixed order and the float32 result goes to slice ks of the partial
+// buffer [ks, M, N].  Bias / SwiGLU / residual are applied by whoever sums the slices (the finish kernel, or the
+// next kernel of the decode step when the caller defers the sum to it).
+constexpr int kSplitWaves = 4;
+constexpr int kSplitPitch = 132;  // floats per row of a partial tile in LDS (128 + padding against bank conflicts)
+
+template <bool FP8, int DEPTH, bool STEP_SCALES>
+__global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(GemmParams p) {
+    constexpr int ES = FP8 ? 1 : 2;
+    extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int x = lane & 15, kb = lane >> 4;
+    const int span = blockIdx.x, ks = blockIdx.y, row0 = blockIdx.z * 64;
+    const int ncol = span * 128 + 8 * x;
+    const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
+    const int steps = (k1 - k0) >> 5;
+    const int n_my = (steps - wave + kSplitWaves - 1) / kSplitWaves;  // steps wave, wave + 4, ... of the slice (<= DEPTH)
+
+    const int row_bytes = p.N * ES;
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+    const int wvoff = 8 * kb * row_bytes + ncol * ES;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
+    int avoff[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int arow = row0 + mt * 16 + x;
+        const int asrc = arow < p.M ? (p.row_map ? p.row_map[arow] : arow) : 0;
+        avoff[mt] = arow < p.M ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
+    }
+    const int n_mt = min(4, (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
+
+    // all operands are requested before anything is waited for, in the order they are consumed
+    u32x4 a[DEPTH][4];
+    RawW<FP8> w[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        const bool live = d < n_my;
+        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+        const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        const bool live = d < n_my;
+        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    float colscale[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
+    const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (ncol >> p.bn_shift) : nullptr;
+    if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
+        const float sc = *sc_lane;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = sc;
+    } else if (FP8 && p.scale_mode == 2) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(ncol + c) >> p.bn_shift];
+    }
+    const int cnt = min(p.group_sizes[0], p.M);  // rows at or beyond it multiply zeros (lax.ragged_dot)
+    __builtin_amdgcn_sched_barrier(0);
+
+    f32x4 acc[4][8];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+        Pack8 bop[8];
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) convert_pair<FP8>(w[d], pr, bop);
+        float sc = 1.f;
+        if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            if (mt < n_mt) {
+                Pack8 av;
+                const bool a_ok = row0 + mt * 16 + x < cnt;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) av.u[i] = a_ok ? a[d][mt][i] : 0u;
+                if constexpr (STEP_SCALES) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                        acc[mt][c][0] += t[0] * sc;
+                        acc[mt][c][1] += t[1] * sc;
+                        acc[mt][c][2] += t[2] * sc;
+                        acc[mt][c][3] += t[3] * sc;
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av.v, bop[c].v, acc[mt][c]);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    float* mine = sm_part + wave * (64 * kSplitPitch);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        if (mt < n_mt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* dst = mine + (mt * 16 + 4 * kb + r) * kSplitPitch + 8 * x;
+                *(f32x4*)dst = f32x4{acc[mt][0][r] * colscale[0], acc[mt][1][r] * colscale[1], acc[mt][2][r] * colscale[2],
+                                     acc[mt][3][r] * colscale[3]};
+                *(f32x4*)(dst + 4) = f32x4{acc[mt][4][r] * colscale[4], acc[mt][5][r] * colscale[5], acc[mt][6][r] * colscale[6],
+                                           acc[mt][7][r] * colscale[7]};
+            }
+        }
+    }
+    __syncthreads();
+    // thread t sums 4 columns of rows t / 32, t / 32 + 8, ... over the wavefronts and writes the slice's partial
+    const int q = threadIdx.x & 31;
+    for (int r = threadIdx.x >> 5; r < 16 * n_mt; r += 8) {
+        const int row = row0 + r;
+        if (row >= p.M) break;
+        f32x4 v = *(const f32x4*)(sm_part + r * kSplitPitch + 4 * q);
+#pragma unroll
+        for (int wv = 1; wv < kSplitWaves; ++wv) {
+            const f32x4 t = *(const f32x4*)(sm_part + wv * (64 * kSplitPitch) + r * kSplitPitch + 4 * q);
+            v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+        }
+        *(f32x4*)(p.part + ((size_t)ks * p.M + row) * p.N + span * 128 + 4 * q) = v;
+    }
+}
+
 struct GemmPlan {
     int mt;       // 16-row tiles held in registers per pass
     int row_par;  // row blocks of one group spread over this many workgroups
     int spans;    // 128-column spans (64+64 with SwiGLU)
     int ksplit, kpart;
-    bool one_pass;  // single group with a few MB of weights: decode_gemm_small_kernel
+    bool one_pass;  // single group with a few MB of weights, swiglu tile layout: decode_gemm_small_kernel
+    bool split_k;   // single group with a few MB of weights: decode_gemm_splitk_kernel + a sum over the K slices
 };
 
 // Shape-only plan (group sizes live on the device).  Large weight sets are streamed once: wide row blocks, K
@@ -601,7 +742,25 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     GemmPlan pl;
     const int touched = std::max(1, std::min(G, M));
     const double weight_bytes = (double)touched * K * N;
-    static const bool no_one_pass = getenv("LYRA_GEMM_NO_ONE_PASS") != nullptr;  // tuning override
+    static const bool no_one_pass = getenv("LYRA_GEMM_NO_ONE_PASS") != nullptr;  // tuning overrides
+    static const bool no_split_k = getenv("LYRA_GEMM_NO_SPLIT_K") != nullptr;
+    pl.one_pass = false;
+    pl.split_k = G == 1 && weight_bytes <= 48e6 && M <= 256 && K % 128 == 0 && !no_split_k;
+    if (pl.split_k) {
+        // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
+        pl.mt = 4;
+        pl.row_par = (M + 63) / 64;
+        pl.spans = (N + 127) / 128;
+        int unit = 128;
+        if (bk > 0 && bk < K) unit = std::max(unit, (bk + 127) / 128 * 128);
+        const long want = std::max(1L, 256L / ((long)pl.spans * pl.row_par));
+        int kpart = (int)((K + want - 1) / want);
+        kpart = std::min(512, (kpart + unit - 1) / unit * unit);
+        if (unit > 512 || (bk > 0 && bk < K && kpart % bk)) pl.split_k = false;  // scale blocks that do not tile a slice
+        pl.kpart = kpart;
+        pl.ksplit = (K + kpart - 1) / kpart;
+        if (pl.split_k) return pl;
+    }
     pl.one_pass = G == 1 && weight_bytes <= 48e6 && !no_one_pass;
     if (pl.one_pass) {
         pl.mt = 1;
@@ -629,13 +788,41 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     return pl;
 }
 
+// Launches the K-split kernel of a plan with split_k set; p.part receives [ksplit, M, N] float32 slices.
+static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st) {
+    const dim3 grid(pl.spans, pl.ksplit, pl.row_par), block(kSplitWaves * 64);
+    const size_t lds = (size_t)kSplitWaves * 64 * kSplitPitch * sizeof(float);
+    const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4
+    const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+#define LYRA_SPLITK(F, D, S)                                                                                          \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S>,          \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S>), grid, block, lds, st, p);                            \
+    } while (0)
+#define LYRA_SPLITK_D(F, S)                   \
+    do {                                      \
+        if (depth <= 1) LYRA_SPLITK(F, 1, S); \
+        else if (depth == 2) LYRA_SPLITK(F, 2, S); \
+        else if (depth == 3) LYRA_SPLITK(F, 3, S); \
+        else LYRA_SPLITK(F, 4, S);            \
+    } while (0)
+    if (step_scales) LYRA_SPLITK_D(true, true);
+    else if (fp8) LYRA_SPLITK_D(true, false);
+    else LYRA_SPLITK_D(false, false);
+#undef LYRA_SPLITK_D
+#undef LYRA_SPLITK
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
 }  // namespace lyra
 
 extern "C" size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu) {
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return 0;
     // the split factor may depend on the scale block; size for the largest split the plan can choose
     const lyra::GemmPlan pl = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu);
-    if (pl.ksplit == 1) return 256;
+    if (pl.ksplit == 1 && !pl.split_k) return 256;
     return ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
 }
 
@@ -696,13 +883,21 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
     p.post_scale = post_scale != 0;
-    if (pl.ksplit > 1) {
+    if (pl.ksplit > 1 || pl.split_k) {
         const size_t need = ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
         if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
         p.part = (float*)workspace;
     }
 
     hipStream_t st = (hipStream_t)stream;
+    if (pl.split_k) {
+        const int rc = launch_split_k(p, pl, fp8, st);
+        if (rc != LYRA_OK) return rc;
+        const int NO = fused_swiglu ? N / 2 : N;
+        const long threads = (long)M * (NO / 4);
+        hipLaunchKernelGGL(decode_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p);
+        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+    }
     if (pl.one_pass) {
         const dim3 sgrid(pl.spans, pl.row_par), sblock(kSmallWaves * 64);
         const size_t slds = (size_t)kSmallWaves * 16 * 128 * sizeof(float);
@@ -748,4 +943,45 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
     }
     return LYRA_OK;
+}
+
+extern "C" int lyra_decode_gemm_splits(int M, int K, int N, int bk) {
+    if (M <= 0 || K <= 0 || N <= 0 || K % 32 || N % 128) return 0;
+    const lyra::GemmPlan pl = lyra::plan_gemm(M, 1, K, N, bk, 0);
+    return pl.split_k ? pl.ksplit : 0;
+}
+
+extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
+                                         const int32_t* group_sizes, float* partials, size_t partials_bytes, int M, int K, int N,
+                                         int rhs_dtype, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!lhs || !rhs || !group_sizes || !partials || M <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
+    if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
+    if (K % 32 || N % 128) return LYRA_E_UNSUPPORTED;
+    GemmParams p = {};
+    p.bk = p.bn = p.KB = p.NB = 1;
+    if (fp8) {
+        if (bk <= 0 || bn <= 0 || K % bk || N % bn) return LYRA_E_BADARG;
+        if (bn & (bn - 1)) return LYRA_E_UNSUPPORTED;
+        p.bk = bk; p.bn = bn; p.KB = K / bk; p.NB = N / bn;
+        p.bn_shift = __builtin_ctz((unsigned)bn);
+        if (bn % 8 == 0 && (bk % 32 == 0 || bk == K)) p.scale_mode = 1;
+        else if (bk == K) p.scale_mode = 2;
+        else return LYRA_E_UNSUPPORTED;
+    }
+    const GemmPlan pl = plan_gemm(M, 1, K, N, fp8 ? bk : 0, 0);
+    if (!pl.split_k) return LYRA_E_UNSUPPORTED;
+    if (partials_bytes < (size_t)pl.ksplit * M * N * sizeof(float) || ((uintptr_t)partials % 16)) return LYRA_E_WORKSPACE;
+    p.lhs = (const uint16_t*)lhs;
+    p.rhs = (const uint8_t*)rhs;
+    p.scale = rhs_scale;
+    p.group_sizes = group_sizes;
+    p.part = partials;
+    p.M = M; p.G = 1; p.K = K; p.N = N;
+    p.ksplit = pl.ksplit;
+    p.kpart = pl.kpart;
+    p.row_par = pl.row_par;
+    return launch_split_k(p, pl, fp8, (hipStream_t)stream);
 }

@@ -41,10 +41,60 @@ def _transposed(w: torch.Tensor) -> torch.Tensor:
     return hit[1]
 
 
-def rmsnorm_proj(x: torch.Tensor, scale: torch.Tensor, eps: float, proj: torch.Tensor | None = None,
+class Unsummed:
+    """A projection whose K slices are still separate: ``partials`` [splits, M, N] float32, plus the residual update that
+    follows it (``residual`` [M, N] bf16 and ``scale``), to be applied by the kernel that consumes it."""
+
+    __slots__ = ("partials", "residual", "scale")
+
+    def __init__(self, partials: torch.Tensor, residual: torch.Tensor | None = None, scale: float = 1.0):
+        self.partials, self.residual, self.scale = partials, residual, scale
+
+
+def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed | None:
+    """lyra_decode_gemm_partials for a one-group projection; None when the shape does not run split over K."""
+    M, K = lhs.shape
+    G, _, N = rhs.shape
+    fp8 = isinstance(rhs, QArray)
+    bk, bn = rhs.block if fp8 else (0, 0)
+    if G != 1 or K % 32 or N % 128:
+        return None
+    splits = _L.lyra_decode_gemm_splits(M, K, N, bk)
+    if splits <= 0:
+        return None
+    assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous()
+    part = torch.empty((splits, M, N), dtype=torch.float32, device=lhs.device)
+    rv = rhs.qval if fp8 else rhs
+    rc = _L.lyra_decode_gemm_partials(lhs.data_ptr(), rv.data_ptr(), _f32(rhs.scale).data_ptr() if fp8 else None, bk, bn,
+                                      group_sizes.data_ptr(), part.data_ptr(), part.numel() * 4, M, K, N,
+                                      _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _stream(lhs.device))
+    _lib.check(rc, "lyra_decode_gemm_partials")
+    return Unsummed(part)
+
+
+def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None = None,
                  bias: torch.Tensor | None = None, gate: bool = False):
     """rms_norm (lyra/model.py:189-191) of x [B,C] bf16; with ``proj`` [C,n] f32 also f32(h) @ proj (+ bias) as
-    float32 logits, or bf16 ``2*sigmoid`` gates when ``gate`` is set (model.py:343-347).  Returns (h, y | None)."""
+    float32 logits, or bf16 ``2*sigmoid`` gates when ``gate`` is set (model.py:343-347).  Returns (h, y | None).
+
+    ``x`` may be an ``Unsummed`` projection with its residual: the row is then first formed as
+    ``bf16(residual + bf16(bf16(sum of slices) * scale))`` and returned as a third value."""
+    if isinstance(x, Unsummed):
+        u = x
+        splits, B, C = u.partials.shape
+        assert u.residual is not None and u.residual.dtype == torch.bfloat16 and u.residual.is_contiguous()
+        x_out = torch.empty_like(u.residual)
+        h = torch.empty_like(u.residual)
+        y, n = None, 0
+        if proj is not None:
+            n = proj.shape[1]
+            y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=h.device)
+            proj = _f32(_transposed(proj))
+        rc = _L.lyra_rmsnorm_proj_sum(None, u.partials.data_ptr(), splits, u.residual.data_ptr(), float(u.scale), x_out.data_ptr(),
+                                      _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
+                                      1 if gate else 2, float(eps), _stream(h.device))
+        _lib.check(rc, "lyra_rmsnorm_proj_sum")
+        return h, y, x_out
     B, C = x.shape
     assert x.dtype == torch.bfloat16 and x.is_contiguous()
     h = torch.empty_like(x)
@@ -59,16 +109,24 @@ def rmsnorm_proj(x: torch.Tensor, scale: torch.Tensor, eps: float, proj: torch.T
     return h, y
 
 
-def qkv_post(qkv: torch.Tensor, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
+def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
              n_heads: int, n_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
     """QK norm + rotary embedding + KV-cache append (quantising for an FP8 cache) for one new token per sequence
     (lyra/model.py:309-336); ``pos`` is an int32 device scalar or a [B] tensor.  Returns q [B,N,H] bf16; the caches
     are updated in place."""
-    B = qkv.shape[0]
     N, K, H = n_heads, n_kv_heads, head_dim
-    assert qkv.dtype == torch.bfloat16 and qkv.is_contiguous() and qkv.shape[1] == (N + 2 * K) * H
+    unsummed = isinstance(qkv, Unsummed)
+    if unsummed:  # the projection arrives as K slices; they are summed while reading
+        part = qkv.partials
+        splits, B, width = part.shape
+        assert width == (N + 2 * K) * H and qkv.residual is None
+        dev = part.device
+    else:
+        B = qkv.shape[0]
+        assert qkv.dtype == torch.bfloat16 and qkv.is_contiguous() and qkv.shape[1] == (N + 2 * K) * H
+        dev = qkv.device
     assert pos.dtype == torch.int32
-    q = torch.empty((B, N, H), dtype=torch.bfloat16, device=qkv.device)
+    q = torch.empty((B, N, H), dtype=torch.bfloat16, device=dev)
     fp8 = isinstance(cache_k, QArray)
     if fp8:
         assert tuple(cache_k.block) == (1, H) and cache_k.scale.dtype == torch.float32
@@ -79,11 +137,12 @@ def qkv_post(qkv: torch.Tensor, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.
         S = kq.shape[2]
         assert kq.dtype == torch.bfloat16
     assert kq.is_contiguous() and vq.is_contiguous() and tuple(kq.shape) == (B, K, S, H)
-    rc = _L.lyra_qkv_post(qkv.data_ptr(), _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(), _f32(sin_t).data_ptr(), pos.data_ptr(),
-                          0 if pos.numel() == 1 else 1, q.data_ptr(), kq.data_ptr(), vq.data_ptr(), _ptr(ks), _ptr(vs),
-                          B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
-                          _stream(qkv.device))
-    _lib.check(rc, "lyra_qkv_post")
+    rc = _L.lyra_qkv_post_sum(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None, splits if unsummed else 0,
+                              _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(), _f32(sin_t).data_ptr(), pos.data_ptr(),
+                              0 if pos.numel() == 1 else 1, q.data_ptr(), kq.data_ptr(), vq.data_ptr(), _ptr(ks), _ptr(vs),
+                              B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
+                              _stream(dev))
+    _lib.check(rc, "lyra_qkv_post_sum")
     return q
 
 

@@ -397,29 +397,42 @@ _ONE_GROUP: dict = {}
 
 
 def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
-    """attention_apply as 5-7 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append | attention |
-    output matmul with the scaled residual add in its epilogue."""
+    """attention_apply as 5 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append | attention | output matmul.
+    ``x`` is the residual stream or an ``Unsummed`` projection that still has to be added to it; the return value likewise
+    (dense projections run split over K and leave the sum of their slices to the kernel that consumes them)."""
     from lyra_amd.kernels import decode_fused as F
 
-    B = x.shape[0]
     H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
+    if isinstance(x, F.Unsummed):
+        h, gate, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+    else:
+        h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+    B = x.shape[0]
     one = _one_group(B, x.device)
-    h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
-    qkv = F.gemm(h, w.qkv, one)
+    qkv = F.gemm_unsummed(h, w.qkv, one)
+    if qkv is None:
+        qkv = F.gemm(h, w.qkv, one)
     q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps)
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     attn = attn_op(cfg.mode, cfg.implementation)
-    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate)
-    return F.gemm(t.reshape(B, N * H), w.out, one, residual=x, out_scale=cfg.residual_scale), cache
+    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate).reshape(B, N * H)
+    out = F.gemm_unsummed(t, w.out, one)
+    if out is None:
+        return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache
+    out.residual, out.scale = x, cfg.residual_scale
+    return out, cache
 
 
 def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
     """moe_apply as norm+router | routing | up matmul (token gather fused) | down matmul | combine+residual."""
     from lyra_amd.kernels import decode_fused as F
 
-    B = x.shape[0]
     topk = cfg.n_active_experts
-    xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+    if isinstance(x, F.Unsummed):
+        xn, logits, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+    else:
+        xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+    B = x.shape[0]
     scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
     t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
                swiglu_limit=cfg.swiglu_limit)
@@ -430,10 +443,17 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
 def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     from lyra_amd.kernels import decode_fused as F
 
+    if isinstance(x, F.Unsummed):
+        t, _, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
+    else:
+        t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     one = _one_group(x.shape[0], x.device)
-    t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit)
-    return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)
+    down = F.gemm_unsummed(t, w.mlp_down, one)
+    if down is None:
+        return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)
+    down.residual, down.scale = x, cfg.dense_residual_scale
+    return down
 
 
 def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
@@ -456,7 +476,7 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
         h = moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
-    h, _ = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)
+    h = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)[0]
     logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True)
     logits[:, cfg.vocab_size :] = float("-inf")
     cache.pos += 1

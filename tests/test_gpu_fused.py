@@ -270,3 +270,48 @@ def test_argmax_first_maximum(rows, cols, ld):
         if rows > 1:
             want[1] = 0
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("B,C,N,K,H", [(64, 2048, 16, 4, 128), (5, 256, 2, 1, 64)])
+def test_unsummed_projection_consumers_equal_summed_path(fp8, B, C, N, K, H):
+    """Handing the K slices of a dense projection to the next kernel must give bit for bit what summing them first gives."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray, quantize
+
+    _say(f"unsummed fp8={fp8} B{B} C{C}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(B + C)
+    rnd = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).to(torch.bfloat16)
+    width = (N + 2 * K) * H
+    w_qkv, w_out = rnd(1, C, width, std=0.03), rnd(1, N * H, C, std=0.03)
+    if fp8:
+        w_qkv, w_out = quantize(w_qkv, torch.float8_e4m3fn, (C, 1)), quantize(w_out, torch.float8_e4m3fn, (min(N * H, 256), 256))
+    one = torch.full((1,), B, dtype=torch.int32, device=dev)
+    h, x = rnd(B, C), rnd(B, C)
+    S = 64
+    cos_t, sin_t = (U.t_f32(t) for t in O.rope_tables(S, H))
+    qn = torch.ones(H, device=dev) * 1.1
+    pos = torch.tensor(7, dtype=torch.int32, device=dev)
+    mk = lambda: QArray(torch.zeros((B, K, S, H), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn),
+                        torch.ones((B, K, S, 1), dtype=torch.float32, device=dev), (1, H))
+    # q/k/v projection -> QK norm, RoPE, cache append
+    un = F.gemm_unsummed(h, w_qkv, one)
+    assert un is not None and un.partials.shape[1:] == (B, width)
+    ck1, cv1, ck2, cv2 = mk(), mk(), mk(), mk()
+    q1 = F.qkv_post(un, qn, qn, cos_t, sin_t, pos, ck1, cv1, N, K, H, 1e-5)
+    q2 = F.qkv_post(F.gemm(h, w_qkv, one), qn, qn, cos_t, sin_t, pos, ck2, cv2, N, K, H, 1e-5)
+    assert torch.equal(q1, q2)
+    assert torch.equal(ck1.qval.view(torch.uint8), ck2.qval.view(torch.uint8)) and torch.equal(cv1.scale, cv2.scale)
+    # output projection -> residual update -> next norm (+ router logits)
+    t = rnd(B, N * H)
+    un = F.gemm_unsummed(t, w_out, one)
+    assert un is not None
+    un.residual, un.scale = x, 0.1767766952966369
+    scale = torch.rand(C, generator=g, device=dev) + 0.5
+    router = torch.randn(C, 7, generator=g, device=dev) * 0.05
+    h1, y1, x1 = F.rmsnorm_proj(un, scale, 1e-5, router, None)
+    x2 = F.gemm(t, w_out, one, residual=x, out_scale=0.1767766952966369)
+    h2, y2 = F.rmsnorm_proj(x2, scale, 1e-5, router, None)
+    assert torch.equal(x1, x2) and torch.equal(h1, h2) and torch.equal(y1, y2)
