@@ -55,10 +55,21 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // C % 4 == 0
         u32x2 d;
         if (p.partials) {
+            // slices are requested 8 at a time (slices past the last read as zeros) and added in slice order
+            const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(p.partials), 0, (uint32_t)((size_t)p.splits * p.B * p.C * 4), 0x00020000);
+            const int slab = p.B * p.C * 4, mine = (b * p.C + c) * 4;
             f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
-            for (int sidx = 0; sidx < p.splits; ++sidx) {
-                const f32x4 u = *(const f32x4*)(p.partials + ((size_t)sidx * p.B + b) * p.C + c);
-                t[0] += u[0]; t[1] += u[1]; t[2] += u[2]; t[3] += u[3];
+            for (int s0 = 0; s0 < p.splits; s0 += 8) {
+                u32x4 u[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    u[j] = __builtin_amdgcn_raw_buffer_load_b128(pr, s0 + j < p.splits ? (s0 + j) * slab + mine : kNoLoad, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    t[0] += __uint_as_float(u[j][0]); t[1] += __uint_as_float(u[j][1]);
+                    t[2] += __uint_as_float(u[j][2]); t[3] += __uint_as_float(u[j][3]);
+                }
             }
             const u32x2 r = *(const u32x2*)(p.residual + (size_t)b * p.C + c);
             const float r0 = __uint_as_float(r[0] << 16), r1 = __uint_as_float(r[0] & 0xFFFF0000u);
@@ -164,9 +175,21 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
         if (active) {
             const size_t slab = (size_t)p.B * heads * p.H;
             const float* src = p.partials + ((size_t)b * heads + hd) * p.H;
-            for (int sidx = 0; sidx < p.splits; ++sidx) {
-                a += src[sidx * slab + lane];
-                c += src[sidx * slab + lane + half];
+            for (int s0 = 0; s0 < p.splits; s0 += 8) {  // 8 slices in flight; added in slice order
+                float ua[8], uc[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int sidx = min(s0 + j, p.splits - 1);
+                    ua[j] = src[sidx * slab + lane];
+                    uc[j] = src[sidx * slab + lane + half];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (s0 + j < p.splits) {
+                        a += ua[j];
+                        c += uc[j];
+                    }
+                }
             }
             a = bf16r(a);  // the projection's output is a bf16 array
             c = bf16r(c);
@@ -421,6 +444,7 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
                                      int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
     using namespace lyra;
     if (partials ? (!residual || !x_out || splits <= 0) : !x) return LYRA_E_BADARG;
+    if (partials && (double)splits * B * C * 4 >= 2147483648.0) return LYRA_E_UNSUPPORTED;
     if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
