@@ -721,6 +721,225 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     }
 }
 
+// Finishes 4 accumulated columns of one output row (2 gate + 2 linear columns with SwiGLU): bias, SwiGLU, residual
+// epilogue, cast, store.  oc = first output column.
+__device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&v)[4], int g, int row, int oc, int NO) {
+    const size_t oidx = (size_t)row * NO + oc;
+    if (p.swiglu) {
+        if (p.bias) {
+            const float* bp = p.bias + (size_t)g * p.N;
+            v[0] += bp[oc]; v[1] += bp[oc + 1]; v[2] += bp[NO + oc]; v[3] += bp[NO + oc + 1];
+        }
+        float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
+        if (p.post_scale) {
+            o[0] = residual_epilogue(p, o[0], oidx);
+            o[1] = residual_epilogue(p, o[1], oidx + 1);
+        }
+        if (p.out_f32) *(f32x2*)((float*)p.out + oidx) = f32x2{o[0], o[1]};
+        else *(uint32_t*)((uint16_t*)p.out + oidx) = pack_bf16(o[0], o[1]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (p.bias) v[c] += p.bias[(size_t)g * p.N + oc + c];
+            if (p.post_scale) v[c] = residual_epilogue(p, v[c], oidx + c);
+        }
+        if (p.out_f32) {
+            *(f32x4*)((float*)p.out + oidx) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+            u32x2 d;
+            d[0] = pack_bf16(v[0], v[1]);
+            d[1] = pack_bf16(v[2], v[3]);
+            *(u32x2*)((uint16_t*)p.out + oidx) = d;
+        }
+    }
+}
+
+// ---- several groups (MoE experts), a handful of rows each: one workgroup per (expert, 128-column span) --------------
+// The workgroup streams the whole K extent of its span once: its 4 wavefronts interleave over K in steps of 32 rows
+// with DEPTH steps of weights and activations in flight each, accumulate 64 rows of the expert per pass, and their partial
+// tiles are summed through LDS in a fixed order; bias / SwiGLU / residual follow in the same kernel.  Experts without
+// rows return at once (their weights are never read), so there are no float32 partials in global memory and no
+// second pass.  With SwiGLU a span is 64 gate + 64 linear columns.
+// ROUNDS passes over the DEPTH register sets are unrolled per trip of the K loop: in straight-line code every wait counts
+// exactly the loads issued after the one it needs, whereas the wait at the head of a loop drains nearly everything in
+// flight, so the longer the straight-line stretch the better (4 when the number of passes allows, else 2 or 1).
+constexpr int kGroupTiles = 4;  // 16-row tiles a workgroup accumulates per pass over its weights (64 rows)
+
+template <bool FP8, bool STEP_SCALES, int ROUNDS>
+__global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
+    constexpr int MTM = kGroupTiles;
+    constexpr int ES = FP8 ? 1 : 2;
+    constexpr int DEPTH = FP8 ? 4 : 2;
+    extern __shared__ float sm_part[];  // [kSplitWaves][16 * MTM][kSplitPitch]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int x = lane & 15, kb = lane >> 4;
+    // With SwiGLU a span reads half of each 128-byte line of a weight row (64 gate bytes, 64 linear bytes with FP8); the
+    // span next to it reads the other half.  Workgroups go to the 8 dies round robin by launch index, and each die has
+    // its own L2: the two spans of a pair are placed half the grid apart (a multiple of 8), so they share an L2.
+    int span = blockIdx.x;
+    if (p.swiglu && (gridDim.x & 15) == 0) span = (blockIdx.x % (gridDim.x >> 1)) * 2 + blockIdx.x / (gridDim.x >> 1);
+    // groups are launched last to first: shared experts, which every token visits and whose workgroups therefore carry
+    // the most rows (the most activation bytes), are the last groups (lyra/model.py:470-476) and should start first
+    const int g = p.G - 1 - blockIdx.y;
+
+    // rows of this group: [off, off + cnt); the last group also owns the rows past the end of all groups
+    int part_sum = 0;
+    for (int i = lane; i < g; i += 64) part_sum += p.group_sizes[i];
+    part_sum = (int)wave_sum((float)part_sum);  // (row counts are far below 2^24: exact in float32)
+    const int off = min(part_sum, p.M);
+    const int cnt = min(p.group_sizes[g], p.M - off);
+    const int pad_from = g == p.G - 1 ? off + cnt : p.M;
+    if (cnt <= 0 && pad_from >= p.M) return;
+
+    int ncol;
+    const bool is_lin_lane = p.swiglu && x >= 8;
+    if (p.swiglu) ncol = (is_lin_lane ? (p.N >> 1) : 0) + span * 64 + 8 * (x & 7);
+    else ncol = span * 128 + 8 * x;
+    const int row_bytes = p.N * ES;
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+    const int wvoff = 8 * kb * row_bytes + ncol * ES;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
+    const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (size_t)g * p.KB * p.NB + (ncol >> p.bn_shift) : nullptr;
+    const int steps = p.K >> 5;
+    const int n_my = (steps - wave + kSplitWaves - 1) / kSplitWaves;
+    const int NO = p.swiglu ? p.N >> 1 : p.N;
+    const int q = threadIdx.x & 31;
+    const int oc = p.swiglu ? span * 64 + 2 * q : span * 128 + 4 * q;
+
+    for (int rb = 0; rb < cnt; rb += 16 * MTM) {
+        const int rows_here = min(16 * MTM, cnt - rb);
+        const int n_mt = (rows_here + 15) >> 4;
+        int avoff[MTM];
+#pragma unroll
+        for (int mt = 0; mt < MTM; ++mt) {
+            const int r = rb + mt * 16 + x;
+            const int src = r < cnt ? (p.row_map ? p.row_map[off + r] : off + r) : 0;
+            avoff[mt] = r < cnt ? (src * p.K + 8 * kb) * 2 : kNoLoad;
+        }
+        u32x4 a[DEPTH][MTM];
+        RawW<FP8> w[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const bool live = d < n_my;
+            const int kk = (wave + kSplitWaves * d) << 5;
+            const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
+#pragma unroll
+            for (int mt = 0; mt < MTM; ++mt)
+                a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live && mt < n_mt ? avoff[mt] : kNoLoad, soff, 0);
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
+        }
+        // column scales: requested behind the first operands, needed only when the tile is written out
+        float colscale[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
+        if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
+            const float sc = *sc_lane;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) colscale[c] = sc;
+        } else if (FP8 && p.scale_mode == 2) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)g * p.NB + ((ncol + c) >> p.bn_shift)];
+        }
+        f32x4 acc[MTM][8];
+#pragma unroll
+        for (int mt = 0; mt < MTM; ++mt)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // every pass issues the same loads (past the end they fetch nothing) and multiplies zeros there
+        const int n_rounds = (n_my + DEPTH - 1) / DEPTH;  // a multiple of ROUNDS (the host checks)
+        for (int round0 = 0; round0 < n_rounds; round0 += ROUNDS) {
+#pragma unroll
+          for (int ur = 0; ur < ROUNDS; ++ur) {
+            const int base = (round0 + ur) * DEPTH;
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int idx = base + d;
+                const int kk = (wave + kSplitWaves * idx) << 5;
+                const int kk_next = kk + ((kSplitWaves * DEPTH) << 5);
+                const bool more = idx + DEPTH < n_my;
+                Pack8 bop[8], av[MTM];
+#pragma unroll
+                for (int mt = 0; mt < MTM; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) av[mt].u[i] = a[d][mt][i];
+                __builtin_amdgcn_sched_barrier(0);
+                const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
+#pragma unroll
+                for (int mt = 0; mt < MTM; ++mt)
+                    a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more && mt < n_mt ? avoff[mt] : kNoLoad, soff, 0);
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    convert_pair<FP8>(w[d], pr, bop);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_w_pair_if<FP8>(more, w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                float sc = 1.f;
+                if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+#pragma unroll
+                for (int mt = 0; mt < MTM; ++mt) {
+                    if (mt < n_mt) {
+                        if constexpr (STEP_SCALES) {
+#pragma unroll
+                            for (int c = 0; c < 8; ++c) {
+                                const f32x4 t = mfma_16x16x32(av[mt].v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                                acc[mt][c][0] += t[0] * sc;
+                                acc[mt][c][1] += t[1] * sc;
+                                acc[mt][c][2] += t[2] * sc;
+                                acc[mt][c][3] += t[3] * sc;
+                            }
+                        } else {
+#pragma unroll
+                            for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
+                        }
+                    }
+                }
+            }
+          }
+        }
+
+        __syncthreads();  // (the previous row block's sums have been read)
+        float* mine = sm_part + wave * (16 * MTM * kSplitPitch);
+#pragma unroll
+        for (int mt = 0; mt < MTM; ++mt) {
+            if (mt < n_mt) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float* dst = mine + (mt * 16 + 4 * kb + r) * kSplitPitch + 8 * x;
+                    *(f32x4*)dst = f32x4{acc[mt][0][r] * colscale[0], acc[mt][1][r] * colscale[1], acc[mt][2][r] * colscale[2],
+                                         acc[mt][3][r] * colscale[3]};
+                    *(f32x4*)(dst + 4) = f32x4{acc[mt][4][r] * colscale[4], acc[mt][5][r] * colscale[5],
+                                               acc[mt][6][r] * colscale[6], acc[mt][7][r] * colscale[7]};
+                }
+            }
+        }
+        __syncthreads();
+        for (int r = threadIdx.x >> 5; r < rows_here; r += 8) {
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int wv = 0; wv < kSplitWaves; ++wv) {
+                const float* src = sm_part + wv * (16 * MTM * kSplitPitch) + r * kSplitPitch;
+                if (p.swiglu) {
+                    const f32x2 g2 = *(const f32x2*)(src + 2 * q), l2 = *(const f32x2*)(src + 64 + 2 * q);
+                    v[0] += g2[0]; v[1] += g2[1]; v[2] += l2[0]; v[3] += l2[1];
+                } else {
+                    const f32x4 t = *(const f32x4*)(src + 4 * q);
+                    v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+                }
+            }
+            group_epilogue(p, v, g, off + rb + r, oc, NO);
+        }
+    }
+    // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
+    for (int row = pad_from + (threadIdx.x >> 5); row < p.M; row += 8) {
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        group_epilogue(p, v, g, row, oc, NO);
+    }
+}
+
 struct GemmPlan {
     int mt;       // 16-row tiles held in registers per pass
     int row_par;  // row blocks of one group spread over this many workgroups
@@ -728,6 +947,7 @@ struct GemmPlan {
     int ksplit, kpart;
     bool one_pass;  // single group with a few MB of weights, swiglu tile layout: decode_gemm_small_kernel
     bool split_k;   // single group with a few MB of weights: decode_gemm_splitk_kernel + a sum over the K slices
+    bool grouped;   // several groups: decode_gemm_group_kernel, one pass
 };
 
 // Shape-only plan (group sizes live on the device).  Large weight sets are streamed once: wide row blocks, K
@@ -745,6 +965,17 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     static const bool no_one_pass = getenv("LYRA_GEMM_NO_ONE_PASS") != nullptr;  // tuning overrides
     static const bool no_split_k = getenv("LYRA_GEMM_NO_SPLIT_K") != nullptr;
     pl.one_pass = false;
+    static const bool no_grouped = getenv("LYRA_GEMM_NO_GROUPED") != nullptr;
+    pl.grouped = G > 1 && !no_grouped;
+    if (pl.grouped) {
+        pl.mt = 4;
+        pl.row_par = 1;
+        pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
+        pl.ksplit = 1;
+        pl.kpart = K;
+        pl.split_k = false;
+        return pl;
+    }
     pl.split_k = G == 1 && weight_bytes <= 48e6 && M <= 256 && K % 128 == 0 && !no_split_k;
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
@@ -890,6 +1121,31 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     }
 
     hipStream_t st = (hipStream_t)stream;
+    if (pl.grouped) {
+        const dim3 ggrid(pl.spans, G), gblock(kSplitWaves * 64);
+        const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
+        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+#define LYRA_GROUP_R(F, S, R)                                                                                         \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R>,           \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R>), ggrid, gblock, glds, st, p);                          \
+    } while (0)
+#define LYRA_GROUP(F, S, DEPTH_)                                                          \
+    do {                                                                                  \
+        const int per_wave = (K / 32 + kSplitWaves - 1) / kSplitWaves;                    \
+        const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
+        if (K % (kSplitWaves * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);        \
+        else LYRA_GROUP_R(F, S, 1);                                                       \
+    } while (0)
+        if (step_scales) LYRA_GROUP(true, true, 4);
+        else if (fp8) LYRA_GROUP(true, false, 4);
+        else LYRA_GROUP(false, false, 2);
+#undef LYRA_GROUP
+#undef LYRA_GROUP_R
+        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+    }
     if (pl.split_k) {
         const int rc = launch_split_k(p, pl, fp8, st);
         if (rc != LYRA_OK) return rc;
