@@ -79,7 +79,7 @@ __device__ __forceinline__ void store_out(const AttnParams& p, size_t idx, float
 template <int H, bool FP8>
 struct RawK {
     static constexpr int ES = FP8 ? 1 : 2;
-    static constexpr int KW = ES * H / 16;  // dwords of one K row held by a lane (a quarter row)
+    static constexpr int KW = ES * H / 16;  // dwords of one K row held by a lane: 16-byte pieces at p * 64 + kb * 16
     uint32_t k[2][KW];
 };
 struct RawS {  // per-token scales of the 8 tokens whose logits this lane holds
@@ -115,7 +115,7 @@ __device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int w = 0; w < KW; w += 4) {
-            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, voff + j * 16 * RB + w * 4, soff, 0);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, voff + j * 16 * RB + (w / 4) * 64, soff, 0);
             t.k[j][w] = d[0];
             t.k[j][w + 1] = d[1];
             t.k[j][w + 2] = d[2];
@@ -189,7 +189,12 @@ __device__ __forceinline__ void tile_logits(const RawK<H, FP8>& t, const uint16_
     const int x = lane & 15, kb = lane >> 4;
     bf16x8 qop[NC];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) qop[c] = *(const bf16x8*)(sm_q + x * QP + kb * (H / 4) + 8 * c);
+    for (int c = 0; c < NC; ++c) {
+        // k index of the 8 values chunk c takes from this lane's K pieces: piece p of a lane is the 16 bytes at
+        // p * 64 + kb * 16 of the row, so that one load instruction covers a contiguous 64 bytes of each of its 16 rows
+        const int k0 = FP8 ? (c >> 1) * 64 + kb * 16 + 8 * (c & 1) : c * 32 + kb * 8;
+        qop[c] = *(const bf16x8*)(sm_q + x * QP + k0);
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -329,7 +334,7 @@ void decode_attention_kernel(AttnParams p) {
     sl.v = make_rsrc(p.v + head_row * (H * ES), (uint32_t)p.S * (H * ES));
     sl.ks = make_rsrc(FP8 ? p.ks + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
     sl.vs = make_rsrc(FP8 ? p.vs + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
-    sl.voff_k = x * (H * ES) + kb * (H * ES / 4);
+    sl.voff_k = x * (H * ES) + kb * 16;
     sl.voff_v = 4 * kb * (H * ES) + x * (H * ES / 16);
     sl.voff_s = 16 * kb;
 
