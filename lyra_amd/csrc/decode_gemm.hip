@@ -721,116 +721,182 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     }
 }
 
-// Finishes 4 accumulated columns of one output row (2 gate + 2 linear columns with SwiGLU): bias, SwiGLU, residual
-// epilogue, cast, store.  oc = first output column.
-__device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&v)[4], int g, int row, int oc, int NO) {
+// Finishes 4 consecutive output columns of one row: vg holds the accumulated columns (the gate columns with SwiGLU, vl
+// then holds the matching linear columns): bias, SwiGLU, residual epilogue, cast, store.  oc = first output column.
+__device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[4], float (&vl)[4], int g, int row, int oc, int NO) {
     const size_t oidx = (size_t)row * NO + oc;
-    if (p.swiglu) {
-        if (p.bias) {
-            const float* bp = p.bias + (size_t)g * p.N;
-            v[0] += bp[oc]; v[1] += bp[oc + 1]; v[2] += bp[NO + oc]; v[3] += bp[NO + oc + 1];
-        }
-        float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
-        if (p.post_scale) {
-            o[0] = residual_epilogue(p, o[0], oidx);
-            o[1] = residual_epilogue(p, o[1], oidx + 1);
-        }
-        if (p.out_f32) *(f32x2*)((float*)p.out + oidx) = f32x2{o[0], o[1]};
-        else *(uint32_t*)((uint16_t*)p.out + oidx) = pack_bf16(o[0], o[1]);
-    } else {
+    float o[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (p.bias) v[c] += p.bias[(size_t)g * p.N + oc + c];
-            if (p.post_scale) v[c] = residual_epilogue(p, v[c], oidx + c);
+    for (int c = 0; c < 4; ++c) {
+        float a = vg[c];
+        if (p.bias) a += p.bias[(size_t)g * p.N + oc + c];
+        if (p.swiglu) {
+            float l = vl[c];
+            if (p.bias) l += p.bias[(size_t)g * p.N + NO + oc + c];
+            a = swiglu_one(a, l, p.beta, p.limit);
         }
-        if (p.out_f32) {
-            *(f32x4*)((float*)p.out + oidx) = f32x4{v[0], v[1], v[2], v[3]};
-        } else {
-            u32x2 d;
-            d[0] = pack_bf16(v[0], v[1]);
-            d[1] = pack_bf16(v[2], v[3]);
-            *(u32x2*)((uint16_t*)p.out + oidx) = d;
-        }
+        if (p.post_scale) a = residual_epilogue(p, a, oidx + c);
+        o[c] = a;
+    }
+    if (p.out_f32) {
+        *(f32x4*)((float*)p.out + oidx) = f32x4{o[0], o[1], o[2], o[3]};
+    } else {
+        u32x2 d;
+        d[0] = pack_bf16(o[0], o[1]);
+        d[1] = pack_bf16(o[2], o[3]);
+        *(u32x2*)((uint16_t*)p.out + oidx) = d;
     }
 }
 
-// ---- several groups (MoE experts), a handful of rows each: one workgroup per (expert, 128-column span) --------------
-// The workgroup streams the whole K extent of its span once: its 4 wavefronts interleave over K in steps of 32 rows
-// with DEPTH steps of weights and activations in flight each, accumulate 64 rows of the expert per pass, and their partial
-// tiles are summed through LDS in a fixed order; bias / SwiGLU / residual follow in the same kernel.  Experts without
-// rows return at once (their weights are never read), so there are no float32 partials in global memory and no
-// second pass.  With SwiGLU a span is 64 gate + 64 linear columns.
+// ---- several groups (MoE experts), a handful of rows each: workgroups walk a list of (row block, column span) units -----
+// A unit is up to 64 rows of one expert times one 128-column span over the whole K extent (256-1024 KB of weights).
+// Every workgroup first builds the same unit list in LDS from group_sizes (experts without rows contribute nothing, so
+// their weights are never read; the last groups - shared experts, which carry the most rows - come first) and then takes
+// units blockIdx.x, blockIdx.x + gridDim.x, ...  Within a unit its 4 wavefronts interleave over K in steps of 32 rows
+// with DEPTH steps of weights and activations in flight each; their partial tiles are summed through LDS in a fixed
+// order and bias / SwiGLU / residual follow.  The first operands of the next unit are requested before the current
+// unit's tile is summed and written, so a compute unit keeps streaming across unit boundaries.  No float32 partials
+// in global memory, no second pass, results independent of the grid size.  With SwiGLU a span is 128 gate columns
+// (wavefronts 0, 1, interleaved over K) plus the matching 128 linear columns (wavefronts 2, 3), so every load covers whole
+// 128-byte lines of a weight row; 64 + 64 columns per wavefront would fetch twice as many lines per byte.
 // ROUNDS passes over the DEPTH register sets are unrolled per trip of the K loop: in straight-line code every wait counts
 // exactly the loads issued after the one it needs, whereas the wait at the head of a loop drains nearly everything in
-// flight, so the longer the straight-line stretch the better (4 when the number of passes allows, else 2 or 1).
-constexpr int kGroupTiles = 4;  // 16-row tiles a workgroup accumulates per pass over its weights (64 rows)
+// flight, so the longer the straight-line stretch the better.
+constexpr int kGroupTiles = 4;      // 16-row tiles a unit accumulates (64 rows)
+constexpr int kMaxStreamGroups = 256;
+constexpr int kMaxRowBlocks = 512;  // units / spans the LDS table holds
+
+struct StreamUnit {
+    int g, row0, rows;  // group, first row (in the sorted lhs), rows in this block (0: no unit)
+};
 
 template <bool FP8, bool STEP_SCALES, int ROUNDS>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
-    constexpr int MTM = kGroupTiles;
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int DEPTH = FP8 ? 4 : 2;
+    constexpr int MTM = kGroupTiles;
     extern __shared__ float sm_part[];  // [kSplitWaves][16 * MTM][kSplitPitch]
+    __shared__ int sm_blk[kMaxRowBlocks][3];  // (group, first row, rows) of every row block, heavy groups first
+    __shared__ int sm_scan[8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
-    // With SwiGLU a span reads half of each 128-byte line of a weight row (64 gate bytes, 64 linear bytes with FP8); the
-    // span next to it reads the other half.  Workgroups go to the 8 dies round robin by launch index, and each die has
-    // its own L2: the two spans of a pair are placed half the grid apart (a multiple of 8), so they share an L2.
-    int span = blockIdx.x;
-    if (p.swiglu && (gridDim.x & 15) == 0) span = (blockIdx.x % (gridDim.x >> 1)) * 2 + blockIdx.x / (gridDim.x >> 1);
-    // groups are launched last to first: shared experts, which every token visits and whose workgroups therefore carry
-    // the most rows (the most activation bytes), are the last groups (lyra/model.py:470-476) and should start first
-    const int g = p.G - 1 - blockIdx.y;
 
-    // rows of this group: [off, off + cnt); the last group also owns the rows past the end of all groups
-    int part_sum = 0;
-    for (int i = lane; i < g; i += 64) part_sum += p.group_sizes[i];
-    part_sum = (int)wave_sum((float)part_sum);  // (row counts are far below 2^24: exact in float32)
-    const int off = min(part_sum, p.M);
-    const int cnt = min(p.group_sizes[g], p.M - off);
-    const int pad_from = g == p.G - 1 ? off + cnt : p.M;
-    if (cnt <= 0 && pad_from >= p.M) return;
+    // ---- unit list: thread t looks at group G-1-t ----
+    const int t = threadIdx.x;
+    int my_cnt = 0, my_before = 0;  // rows of "my" group and rows of all groups before it (in lhs order)
+    {
+        // rows before group g = sum of sizes of groups < g: an inclusive scan over groups in natural order
+        const int gnat = t;  // natural order for the scan
+        int v = gnat < p.G ? p.group_sizes[gnat] : 0;
+        int incl = v;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int u = __shfl_up(incl, o, kWave);
+            if (lane >= o) incl += u;
+        }
+        if (lane == 63) sm_scan[wave] = incl;
+        __syncthreads();
+        int base = 0;
+        for (int wv = 0; wv < wave; ++wv) base += sm_scan[wv];
+        const int before = base + incl - v;
+        // hand (before, size) of natural group gnat to the thread that owns it in heavy-first order: thread G-1-gnat
+        __syncthreads();
+        int* tmp = (int*)sm_part;  // scratch before the tiles are used
+        if (gnat < p.G) {
+            tmp[2 * (p.G - 1 - gnat)] = min(before, p.M);
+            tmp[2 * (p.G - 1 - gnat) + 1] = max(0, min(v, p.M - min(before, p.M)));
+        }
+        __syncthreads();
+        if (t < p.G) {
+            my_before = tmp[2 * t];
+            my_cnt = tmp[2 * t + 1];
+        }
+    }
+    const int my_blocks = (my_cnt + 16 * MTM - 1) / (16 * MTM);
+    int blk_incl = my_blocks;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int u = __shfl_up(blk_incl, o, kWave);
+        if (lane >= o) blk_incl += u;
+    }
+    __syncthreads();
+    if (lane == 63) sm_scan[4 + wave] = blk_incl;
+    __syncthreads();
+    int blk_base = 0;
+    for (int wv = 0; wv < wave; ++wv) blk_base += sm_scan[4 + wv];
+    const int n_blocks = min(kMaxRowBlocks, sm_scan[4] + sm_scan[5] + sm_scan[6] + sm_scan[7]);
+    for (int i = 0; i < my_blocks; ++i) {
+        const int j = blk_base + blk_incl - my_blocks + i;
+        if (j < kMaxRowBlocks) {
+            sm_blk[j][0] = p.G - 1 - t;
+            sm_blk[j][1] = my_before + i * 16 * MTM;
+            sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
+        }
+    }
+    __syncthreads();
 
-    int ncol;
-    const bool is_lin_lane = p.swiglu && x >= 8;
-    if (p.swiglu) ncol = (is_lin_lane ? (p.N >> 1) : 0) + span * 64 + 8 * (x & 7);
-    else ncol = span * 128 + 8 * x;
-    const int row_bytes = p.N * ES;
-    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-    const int wvoff = 8 * kb * row_bytes + ncol * ES;
-    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
-    const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (size_t)g * p.KB * p.NB + (ncol >> p.bn_shift) : nullptr;
-    const int steps = p.K >> 5;
-    const int n_my = (steps - wave + kSplitWaves - 1) / kSplitWaves;
+    const int spans = p.swiglu ? (p.N >> 1) / 128 : p.N / 128;
+    const int kw = p.swiglu ? 2 : kSplitWaves;             // wavefronts that interleave over K for one set of columns
+    const int wslot = p.swiglu ? (wave & 1) : wave, half = p.swiglu ? (wave >> 1) : 0;
+    const int n_units = n_blocks * spans;
     const int NO = p.swiglu ? p.N >> 1 : p.N;
     const int q = threadIdx.x & 31;
-    const int oc = p.swiglu ? span * 64 + 2 * q : span * 128 + 4 * q;
+    const int row_bytes = p.N * ES;
+    const int steps = p.K >> 5;
+    const int n_my = (steps - wslot + kw - 1) / kw;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
 
-    for (int rb = 0; rb < cnt; rb += 16 * MTM) {
-        const int rows_here = min(16 * MTM, cnt - rb);
-        const int n_mt = (rows_here + 15) >> 4;
-        int avoff[MTM];
+    // state of the unit whose operands are in flight / being consumed
+    int u = blockIdx.x;
+    int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
+    __amdgpu_buffer_rsrc_t wrsrc;
+    u32x4 a[DEPTH][MTM];
+    RawW<FP8> w[DEPTH];
+
+    // Looks unit `uu` up and requests its first DEPTH steps (a unit past the end requests nothing).
+    auto open_unit = [&](int uu) {
+        const bool valid = uu < n_units;
+        const int blk = valid ? uu / spans : 0;
+        span = valid ? uu - blk * spans : 0;
+        g = valid ? sm_blk[blk][0] : 0;
+        row0 = valid ? sm_blk[blk][1] : 0;
+        rows = valid ? sm_blk[blk][2] : 0;
+        ncol = half * (p.N >> 1) + span * 128 + 8 * x;
+        wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
+                                                  (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+        wvoff = valid ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) {
-            const int r = rb + mt * 16 + x;
-            const int src = r < cnt ? (p.row_map ? p.row_map[off + r] : off + r) : 0;
-            avoff[mt] = r < cnt ? (src * p.K + 8 * kb) * 2 : kNoLoad;
+            const int r = mt * 16 + x;
+            int src = row0 + min(r, max(rows - 1, 0));
+            if (p.row_map) src = p.row_map[src];
+            avoff[mt] = r < rows ? (src * p.K + 8 * kb) * 2 : kNoLoad;
         }
-        u32x4 a[DEPTH][MTM];
-        RawW<FP8> w[DEPTH];
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const bool live = d < n_my;
-            const int kk = (wave + kSplitWaves * d) << 5;
+            const int kk = (wslot + kw * d) << 5;
             const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
 #pragma unroll
             for (int mt = 0; mt < MTM; ++mt)
-                a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live && mt < n_mt ? avoff[mt] : kNoLoad, soff, 0);
+                a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
         }
+    };
+
+    open_unit(u);
+    while (u < n_units) {
+        const int cur_g = g, cur_row0 = row0, cur_rows = rows, cur_span = span, cur_ncol = ncol;
+        const int n_mt = (cur_rows + 15) >> 4;
+        const __amdgpu_buffer_rsrc_t cur_wrsrc = wrsrc;
+        const int cur_wvoff = wvoff;
+        int cur_avoff[MTM];
+#pragma unroll
+        for (int mt = 0; mt < MTM; ++mt) cur_avoff[mt] = avoff[mt];
         // column scales: requested behind the first operands, needed only when the tile is written out
+        const float* sc_lane =
+            (FP8 && p.scale_mode == 1) ? p.scale + (size_t)cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift) : nullptr;
         float colscale[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
@@ -840,7 +906,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             for (int c = 0; c < 8; ++c) colscale[c] = sc;
         } else if (FP8 && p.scale_mode == 2) {
 #pragma unroll
-            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)g * p.NB + ((ncol + c) >> p.bn_shift)];
+            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)cur_g * p.NB + ((cur_ncol + c) >> p.bn_shift)];
         }
         f32x4 acc[MTM][8];
 #pragma unroll
@@ -852,56 +918,59 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         const int n_rounds = (n_my + DEPTH - 1) / DEPTH;  // a multiple of ROUNDS (the host checks)
         for (int round0 = 0; round0 < n_rounds; round0 += ROUNDS) {
 #pragma unroll
-          for (int ur = 0; ur < ROUNDS; ++ur) {
-            const int base = (round0 + ur) * DEPTH;
+            for (int ur = 0; ur < ROUNDS; ++ur) {
+                const int base = (round0 + ur) * DEPTH;
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
-                const int idx = base + d;
-                const int kk = (wave + kSplitWaves * idx) << 5;
-                const int kk_next = kk + ((kSplitWaves * DEPTH) << 5);
-                const bool more = idx + DEPTH < n_my;
-                Pack8 bop[8], av[MTM];
+                for (int d = 0; d < DEPTH; ++d) {
+                    const int idx = base + d;
+                    const int kk = (wslot + kw * idx) << 5;
+                    const int kk_next = kk + ((kw * DEPTH) << 5);
+                    const bool more = idx + DEPTH < n_my;
+                    Pack8 bop[8], av[MTM];
 #pragma unroll
-                for (int mt = 0; mt < MTM; ++mt)
+                    for (int mt = 0; mt < MTM; ++mt)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) av[mt].u[i] = a[d][mt][i];
-                __builtin_amdgcn_sched_barrier(0);
-                const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
-#pragma unroll
-                for (int mt = 0; mt < MTM; ++mt)
-                    a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more && mt < n_mt ? avoff[mt] : kNoLoad, soff, 0);
-#pragma unroll
-                for (int pr = 0; pr < 4; ++pr) {
-                    convert_pair<FP8>(w[d], pr, bop);
+                        for (int i = 0; i < 4; ++i) av[mt].u[i] = a[d][mt][i];
                     __builtin_amdgcn_sched_barrier(0);
-                    load_w_pair_if<FP8>(more, w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                float sc = 1.f;
-                if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+                    const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
 #pragma unroll
-                for (int mt = 0; mt < MTM; ++mt) {
-                    if (mt < n_mt) {
-                        if constexpr (STEP_SCALES) {
+                    for (int mt = 0; mt < MTM; ++mt)
+                        a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? cur_avoff[mt] : kNoLoad, soff, 0);
 #pragma unroll
-                            for (int c = 0; c < 8; ++c) {
-                                const f32x4 t = mfma_16x16x32(av[mt].v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
-                                acc[mt][c][0] += t[0] * sc;
-                                acc[mt][c][1] += t[1] * sc;
-                                acc[mt][c][2] += t[2] * sc;
-                                acc[mt][c][3] += t[3] * sc;
+                    for (int pr = 0; pr < 4; ++pr) {
+                        convert_pair<FP8>(w[d], pr, bop);
+                        __builtin_amdgcn_sched_barrier(0);
+                        load_w_pair_if<FP8>(more, w[d], pr, cur_wrsrc, cur_wvoff, kk_next, row_bytes);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    float sc = 1.f;
+                    if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+#pragma unroll
+                    for (int mt = 0; mt < MTM; ++mt) {
+                        if (mt < n_mt) {
+                            if constexpr (STEP_SCALES) {
+#pragma unroll
+                                for (int c = 0; c < 8; ++c) {
+                                    const f32x4 tt = mfma_16x16x32(av[mt].v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                                    acc[mt][c][0] += tt[0] * sc;
+                                    acc[mt][c][1] += tt[1] * sc;
+                                    acc[mt][c][2] += tt[2] * sc;
+                                    acc[mt][c][3] += tt[3] * sc;
+                                }
+                            } else {
+#pragma unroll
+                                for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
                             }
-                        } else {
-#pragma unroll
-                            for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
                         }
                     }
                 }
             }
-          }
         }
 
-        __syncthreads();  // (the previous row block's sums have been read)
+        // the next unit's first operands fly while this unit's tile is summed and written
+        u += gridDim.x;
+        open_unit(u);
+
         float* mine = sm_part + wave * (16 * MTM * kSplitPitch);
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) {
@@ -917,26 +986,38 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             }
         }
         __syncthreads();
-        for (int r = threadIdx.x >> 5; r < rows_here; r += 8) {
-            float v[4] = {0.f, 0.f, 0.f, 0.f};
+        const int oc = cur_span * 128 + 4 * q;
+        constexpr int TS = 16 * MTM * kSplitPitch;  // floats per wavefront tile
+        for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
+            const float* src = sm_part + r * kSplitPitch + 4 * q;
+            const f32x4 t0 = *(const f32x4*)src, t1 = *(const f32x4*)(src + TS), t2 = *(const f32x4*)(src + 2 * TS),
+                        t3 = *(const f32x4*)(src + 3 * TS);
+            float vg[4], vl[4];
 #pragma unroll
-            for (int wv = 0; wv < kSplitWaves; ++wv) {
-                const float* src = sm_part + wv * (16 * MTM * kSplitPitch) + r * kSplitPitch;
+            for (int c = 0; c < 4; ++c) {
                 if (p.swiglu) {
-                    const f32x2 g2 = *(const f32x2*)(src + 2 * q), l2 = *(const f32x2*)(src + 64 + 2 * q);
-                    v[0] += g2[0]; v[1] += g2[1]; v[2] += l2[0]; v[3] += l2[1];
+                    vg[c] = t0[c] + t1[c];
+                    vl[c] = t2[c] + t3[c];
                 } else {
-                    const f32x4 t = *(const f32x4*)(src + 4 * q);
-                    v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+                    vg[c] = ((t0[c] + t1[c]) + t2[c]) + t3[c];
+                    vl[c] = 0.f;
                 }
             }
-            group_epilogue(p, v, g, off + rb + r, oc, NO);
+            group_epilogue(p, vg, vl, cur_g, cur_row0 + r, oc, NO);
         }
+        __syncthreads();  // the tiles are free for the next unit
     }
+    wait_all_memory();  // (requests of a unit past the end return nothing, but must not outlive the wavefront's registers)
+
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
-    for (int row = pad_from + (threadIdx.x >> 5); row < p.M; row += 8) {
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-        group_epilogue(p, v, g, row, oc, NO);
+    const int total = sm_scan[0] + sm_scan[1] + sm_scan[2] + sm_scan[3];
+    const int pad_rows = p.M - min(total, p.M);
+    for (int i = blockIdx.x; i < pad_rows * spans; i += gridDim.x) {
+        if (threadIdx.x < 32) {
+            const int row = min(total, p.M) + i / spans, sp = i % spans;
+            float vg[4] = {0.f, 0.f, 0.f, 0.f}, vl[4] = {0.f, 0.f, 0.f, 0.f};
+            group_epilogue(p, vg, vl, p.G - 1, row, sp * 128 + 4 * q, NO);
+        }
     }
 }
 
@@ -966,11 +1047,11 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     static const bool no_split_k = getenv("LYRA_GEMM_NO_SPLIT_K") != nullptr;
     pl.one_pass = false;
     static const bool no_grouped = getenv("LYRA_GEMM_NO_GROUPED") != nullptr;
-    pl.grouped = G > 1 && !no_grouped;
+    pl.grouped = G > 1 && G <= kMaxStreamGroups && G + M / (16 * kGroupTiles) <= kMaxRowBlocks && !no_grouped;
     if (pl.grouped) {
         pl.mt = 4;
         pl.row_par = 1;
-        pl.spans = fused_swiglu ? (N / 2 + 63) / 64 : (N + 127) / 128;
+        pl.spans = fused_swiglu ? N / 256 : N / 128;
         pl.ksplit = 1;
         pl.kpart = K;
         pl.split_k = false;
@@ -1122,7 +1203,9 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
 
     hipStream_t st = (hipStream_t)stream;
     if (pl.grouped) {
-        const dim3 ggrid(pl.spans, G), gblock(kSplitWaves * 64);
+        // one workgroup per compute unit (more would only queue behind the LDS tiles), fewer when there is less work
+        const long most_units = (long)pl.spans * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
+        const dim3 ggrid((unsigned)std::max(1L, std::min(256L, most_units))), gblock(kSplitWaves * 64);
         const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
         const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
 #define LYRA_GROUP_R(F, S, R)                                                                                         \
@@ -1134,9 +1217,10 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     } while (0)
 #define LYRA_GROUP(F, S, DEPTH_)                                                          \
     do {                                                                                  \
-        const int per_wave = (K / 32 + kSplitWaves - 1) / kSplitWaves;                    \
+        const int kw = fused_swiglu ? 2 : kSplitWaves;                                    \
+        const int per_wave = (K / 32 + kw - 1) / kw;                                      \
         const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
-        if (K % (kSplitWaves * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);        \
+        if (K % (kw * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);                 \
         else LYRA_GROUP_R(F, S, 1);                                                       \
     } while (0)
         if (step_scales) LYRA_GROUP(true, true, 4);
