@@ -36,6 +36,7 @@ struct GemmParams {
     float beta, limit;
     int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
+    int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
     const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
     float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
@@ -835,9 +836,13 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     }
     __syncthreads();
 
-    const int spans = p.swiglu ? (p.N >> 1) / 128 : p.N / 128;
-    const int kw = p.swiglu ? 2 : kSplitWaves;             // wavefronts that interleave over K for one set of columns
-    const int wslot = p.swiglu ? (wave & 1) : wave, half = p.swiglu ? (wave >> 1) : 0;
+    // wide: a unit is two sets of 128 columns, each taken by a pair of wavefronts that interleave over K (gate and linear
+    // columns with SwiGLU, else two adjacent spans); otherwise one set of 128 columns and all 4 wavefronts interleave
+    const bool wide = p.swiglu || p.wide;
+    const int spans = p.swiglu ? (p.N >> 1) / 128 : (wide ? p.N / 256 : p.N / 128);
+    const int kw = wide ? 2 : kSplitWaves;
+    const int wslot = wide ? (wave & 1) : wave, half = wide ? (wave >> 1) : 0;
+    const int half_stride = p.swiglu ? (p.N >> 1) : 128, span_cols = p.swiglu || !wide ? 128 : 256;
     const int n_units = n_blocks * spans;
     const int NO = p.swiglu ? p.N >> 1 : p.N;
     const int q = threadIdx.x & 31;
@@ -861,7 +866,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         g = valid ? sm_blk[blk][0] : 0;
         row0 = valid ? sm_blk[blk][1] : 0;
         rows = valid ? sm_blk[blk][2] : 0;
-        ncol = half * (p.N >> 1) + span * 128 + 8 * x;
+        ncol = half * half_stride + span * span_cols + 8 * x;
         wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
                                                   (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
         wvoff = valid ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
@@ -986,7 +991,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             }
         }
         __syncthreads();
-        const int oc = cur_span * 128 + 4 * q;
+        const int oc = cur_span * span_cols + 4 * q;
         constexpr int TS = 16 * MTM * kSplitPitch;  // floats per wavefront tile
         for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
             const float* src = sm_part + r * kSplitPitch + 4 * q;
@@ -995,7 +1000,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             float vg[4], vl[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                if (p.swiglu) {
+                if (wide) {
                     vg[c] = t0[c] + t1[c];
                     vl[c] = t2[c] + t3[c];
                 } else {
@@ -1003,7 +1008,13 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                     vl[c] = 0.f;
                 }
             }
-            group_epilogue(p, vg, vl, cur_g, cur_row0 + r, oc, NO);
+            if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
+                float zero[4] = {0.f, 0.f, 0.f, 0.f};
+                group_epilogue(p, vg, zero, cur_g, cur_row0 + r, oc, NO);
+                group_epilogue(p, vl, zero, cur_g, cur_row0 + r, oc + 128, NO);
+            } else {
+                group_epilogue(p, vg, vl, cur_g, cur_row0 + r, oc, NO);
+            }
         }
         __syncthreads();  // the tiles are free for the next unit
     }
@@ -1012,9 +1023,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
     const int total = sm_scan[0] + sm_scan[1] + sm_scan[2] + sm_scan[3];
     const int pad_rows = p.M - min(total, p.M);
-    for (int i = blockIdx.x; i < pad_rows * spans; i += gridDim.x) {
+    const int pad_spans = p.swiglu ? spans : p.N / 128;
+    for (int i = blockIdx.x; i < pad_rows * pad_spans; i += gridDim.x) {
         if (threadIdx.x < 32) {
-            const int row = min(total, p.M) + i / spans, sp = i % spans;
+            const int row = min(total, p.M) + i / pad_spans, sp = i % pad_spans;
             float vg[4] = {0.f, 0.f, 0.f, 0.f}, vl[4] = {0.f, 0.f, 0.f, 0.f};
             group_epilogue(p, vg, vl, p.G - 1, row, sp * 128 + 4 * q, NO);
         }
@@ -1029,6 +1041,7 @@ struct GemmPlan {
     bool one_pass;  // single group with a few MB of weights, swiglu tile layout: decode_gemm_small_kernel
     bool split_k;   // single group with a few MB of weights: decode_gemm_splitk_kernel + a sum over the K slices
     bool grouped;   // several groups: decode_gemm_group_kernel, one pass
+    bool wide = false;  // ... with units of 256 plain columns
 };
 
 // Shape-only plan (group sizes live on the device).  Large weight sets are streamed once: wide row blocks, K
@@ -1051,7 +1064,9 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     if (pl.grouped) {
         pl.mt = 4;
         pl.row_par = 1;
-        pl.spans = fused_swiglu ? N / 256 : N / 128;
+        static const bool want_wide = getenv("LYRA_GEMM_WIDE") != nullptr;  // tuning override: measured no faster, off
+        pl.wide = !fused_swiglu && N % 256 == 0 && want_wide;
+        pl.spans = (fused_swiglu || pl.wide) ? N / 256 : N / 128;
         pl.ksplit = 1;
         pl.kpart = K;
         pl.split_k = false;
@@ -1192,6 +1207,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.row_par = pl.row_par;
     p.kpart = pl.kpart;
     p.row_map = lhs_row_map;
+    p.wide = pl.wide;
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
     p.post_scale = post_scale != 0;
@@ -1217,7 +1233,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     } while (0)
 #define LYRA_GROUP(F, S, DEPTH_)                                                          \
     do {                                                                                  \
-        const int kw = fused_swiglu ? 2 : kSplitWaves;                                    \
+        const int kw = (fused_swiglu || pl.wide) ? 2 : kSplitWaves;                       \
         const int per_wave = (K / 32 + kw - 1) / kw;                                      \
         const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
         if (K % (kw * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);                 \
