@@ -206,3 +206,34 @@ def test_quantize_on_the_fly_and_dispatch_contract():
     U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, O.bf16_round(w[:, :, :200]), sizes), what="fallback")
     with pytest.raises(ValueError, match="Unsupported bias shape"):
         decode_gemm(U.t_bf16(lhs), U.t_bf16(w), gs, bias=torch.zeros(3, N, device=U.dev()))
+
+
+@pytest.mark.parametrize("M,K,N,kind,block,swiglu", [
+    (100, 1024, 512, "fp8", (256, 256), False),   # two row blocks, scale blocks that change along K
+    (200, 1536, 768, "fp8", (1536, 1), True),     # four row blocks (rows past 192 only partly filled), per-channel scales
+    (37, 512, 256, "bf16", None, False),          # bf16 weights, one slice of 512 rows
+    (64, 4096, 1024, "fp8", (128, 128), False),   # 128-row scale blocks, 8 slices
+    (16, 128, 128, "fp8", (128, 1), False),       # the smallest split shape
+])
+def test_split_k_dense_variants(M, K, N, kind, block, swiglu):
+    """One group with a few MB of weights runs split over K: bias, padding rows (group size < M) and SwiGLU included."""
+    sizes = [M - 3]  # the last three rows lie past the group: zero product + bias
+    c = _case(6, M, 1, K, N, sizes, kind=kind, block=block, bias=True, w_std=0.05)
+    _note(f"gemm split-k M={M} K={K} N={N} kind={kind} block={block} swiglu={swiglu}")
+    from lyra_amd import _lib
+
+    assert _lib.lib.lyra_decode_gemm_splits(M, K, N, block[0] if block else 0) >= 1
+    U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="split-k")
+
+
+@pytest.mark.parametrize("G,M,K,N,swiglu", [(64, 300, 1024, 512, True), (64, 300, 1024, 512, False), (200, 256, 256, 256, False)])
+def test_many_experts_unit_list(G, M, K, N, swiglu):
+    """Many experts, most with a few rows, one with several row blocks, some empty, rows left over at the end."""
+    rng = np.random.default_rng(G + M)
+    sizes = rng.multinomial(M - 150 - 5, np.ones(G - 1) / (G - 1)).astype(np.int32)
+    sizes[::7] = 0
+    sizes = np.concatenate([sizes, [150]]).astype(np.int32)  # the last expert is the heavy one
+    assert sizes.sum() <= M
+    c = _case(8, M, G, K, N, sizes, kind="fp8", block=(K, 1), bias=True, w_std=0.05)
+    _note(f"gemm unit list G={G} M={M} swiglu={swiglu} rows={int(sizes.sum())}")
+    U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list")
