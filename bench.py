@@ -115,6 +115,156 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, launches=100):
     return start.elapsed_time(stop) * 1e-3 / launches  # seconds per launch
 
 
+def _time_launches(launch, stream, warm=5, iters=50):
+    import torch
+
+    for i in range(warm):
+        launch(i)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream.synchronize()
+    start.record(stream)
+    for i in range(iters):
+        launch(i)
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / iters
+
+
+def zipf_group_sizes(rng, tokens, n_routed, k_routed, n_shared):
+    """Rows per expert when every token picks `k_routed` distinct routed experts with p_i ~ i^-1.1 and all shared ones."""
+    import numpy as np
+
+    p = 1.0 / np.arange(1, n_routed + 1) ** 1.1
+    p /= p.sum()
+    ids = np.stack([rng.choice(n_routed, size=k_routed, replace=False, p=p) for _ in range(tokens)])
+    if n_shared:
+        ids = np.concatenate([ids, np.broadcast_to(np.arange(n_routed, n_routed + n_shared), (tokens, n_shared))], 1)
+    return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
+
+
+def kernel_table(dev):
+    """Stand-alone timings of the two operators through the C ABI at the shapes of the named model variants: HIP events
+    over back-to-back launches, once rotating over enough distinct caches / weight sets that every launch streams from
+    HBM ("cold") and once re-using one set ("hot", which the 256 MB last-level cache may serve in part)."""
+    import numpy as np
+    import torch
+
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    stream = torch.cuda.current_stream(dev)
+    rows = []
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1000)
+
+    def attention(label, B, N, K, H, S, sw, fp8, lengths=None):
+        es = 1 if fp8 else 2
+        per = 2 * B * K * S * (H * es + (4 if fp8 else 0))
+        nbuf = max(2, min(8, int(1.2e9 // per) + 1))
+        caches = []
+        for _ in range(nbuf):
+            if fp8:
+                kv = [torch.randint(0, 0x78, (B, K, S, H), generator=gen, device=dev, dtype=torch.uint8) for _ in range(2)]
+                sc = [torch.rand(B, K, S, generator=gen, device=dev) * 0.004 + 0.006 for _ in range(2)]
+            else:
+                kv = [torch.randn(B, K, S, H, generator=gen, device=dev, dtype=torch.bfloat16) for _ in range(2)]
+                sc = [None, None]
+            caches.append((kv, sc))
+        q = torch.randn(B, N, H, generator=gen, device=dev, dtype=torch.bfloat16)
+        out = torch.empty_like(q)
+        sinks = torch.randn(N, generator=gen, device=dev)
+        if lengths is None:
+            pos = torch.full((1,), S - 1, dtype=torch.int32, device=dev)
+            stride, visible = 0, B * (min(sw, S) if sw else S)
+        else:
+            pos = torch.from_numpy(lengths.astype(np.int32) - 1).to(dev)
+            stride, visible = 1, int(np.minimum(lengths, sw).sum() if sw else lengths.sum())
+        need = L.lyra_decode_attention_workspace(B, N, K, S, H, sw)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
+
+        def launch(i, hot=False):
+            (k, v), (ks, vs) = caches[0 if hot else i % nbuf]
+            rc = L.lyra_decode_attention(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), ks.data_ptr() if fp8 else None, vs.data_ptr() if fp8 else None,
+                sinks.data_ptr(), pos.data_ptr(), stride, None, out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H,
+                H**-0.5, sw, _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_BF16, stream.cuda_stream)
+            _lib.check(rc, "lyra_decode_attention")
+
+        nbytes = 2 * K * visible * (H * es + (4 if fp8 else 0))
+        cold = _time_launches(launch, stream)
+        hot = _time_launches(lambda i: launch(i, True), stream)
+        rows.append({"operator": "decode_attention", "case": label, "bytes": nbytes, "cold_us": cold * 1e6, "hot_us": hot * 1e6})
+        del caches
+
+    def gemm(label, M, G, K, N, sizes, swiglu, block, fp8=True, out_f32=False):
+        es = 1 if fp8 else 2
+        nbuf = max(2, min(6, int(600e6 // (G * K * N * es)) + 1))
+        if fp8:
+            weights = [torch.randint(0, 0x78, (G, K, N), generator=gen, device=dev, dtype=torch.uint8) for _ in range(nbuf)]
+            bk, bn = block
+            scale = torch.rand(G, K // bk, N // bn, generator=gen, device=dev) * 0.001 + 0.0005
+        else:
+            weights = [torch.randn(G, K, N, generator=gen, device=dev, dtype=torch.bfloat16) for _ in range(nbuf)]
+            bk = bn = 0
+            scale = None
+        lhs = torch.randn(M, K, generator=gen, device=dev, dtype=torch.bfloat16)
+        gs = torch.from_numpy(np.asarray(sizes, np.int32)).to(dev)
+        NO = N // 2 if swiglu else N
+        out = torch.empty(M, NO, device=dev, dtype=torch.float32 if out_f32 else torch.bfloat16)
+        need = L.lyra_decode_gemm_workspace(M, G, K, N, int(swiglu))
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
+        touched = int((np.asarray(sizes) > 0).sum())
+        nbytes = touched * K * N * es + (touched * (K // bk) * (N // bn) * 4 if fp8 else 0) + M * K * 2 + M * NO * out.element_size()
+
+        def launch(i, hot=False):
+            rc = L.lyra_decode_gemm(
+                lhs.data_ptr(), weights[0 if hot else i % nbuf].data_ptr(), scale.data_ptr() if fp8 else None, bk, bn,
+                gs.data_ptr(), None, out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N,
+                _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(swiglu),
+                1.702, 7.0, stream.cuda_stream)
+            _lib.check(rc, "lyra_decode_gemm")
+
+        cold = _time_launches(launch, stream)
+        hot = _time_launches(lambda i: launch(i, True), stream)
+        rows.append({"operator": "decode_gemm", "case": label, "bytes": nbytes, "rows": M, "touched_experts": touched,
+                     "cold_us": cold * 1e6, "hot_us": hot * 1e6})
+        del weights
+
+    rng = np.random.default_rng(1003)
+    attention("lyra-small B=1 ctx 512 bf16 global", 1, 16, 4, 128, 512, 0, False)
+    attention("lyra-small B=8 ctx 4096 fp8 global", 8, 16, 4, 128, 4096, 0, True)
+    attention("lyra-small B=64 ctx 4096 fp8 global (headline)", 64, 16, 4, 128, 4096, 0, True)
+    attention("lyra-small B=64 ctx 4096 fp8 sliding 128", 64, 16, 4, 128, 4096, 128, True)
+    attention("lyra-small B=64 ctx 4096 bf16 global", 64, 16, 4, 128, 4096, 0, False)
+    attention("lyra-medium B=64 ctx 4096 fp8 global", 64, 32, 8, 128, 4096, 0, True)
+    attention("lyra-max B=128 ctx 4096 fp8 global", 128, 32, 8, 128, 4096, 0, True)
+    lengths = np.random.default_rng(1004).integers(256, 4097, size=64)
+    attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged 256..4096 global", 64, 64, 8, 64, 4096, 0, True, lengths)
+    attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged sliding 128", 64, 64, 8, 64, 4096, 128, True, lengths)
+    for T in (1, 16, 64):
+        s = zipf_group_sizes(rng, T, 31, 3, 1)
+        gemm(f"lyra-medium expert up+SwiGLU T={T} (32x4096x8192 fp8)", int(s.sum()), 32, 4096, 8192, s, True, (4096, 1))
+        gemm(f"lyra-medium expert down T={T} (32x4096x4096 fp8)", int(s.sum()), 32, 4096, 4096, s, False, (4096, 1))
+    s = zipf_group_sizes(rng, 64, 31, 3, 1)
+    gemm("lyra-medium expert up+SwiGLU T=64, scale blocks (256,256)", int(s.sum()), 32, 4096, 8192, s, True, (256, 256))
+    s = zipf_group_sizes(rng, 128, 63, 3, 1)
+    gemm("lyra-max expert up+SwiGLU B=128 (64x4096x8192 fp8)", int(s.sum()), 64, 4096, 8192, s, True, (4096, 1))
+    gemm("lyra-max expert down B=128 (64x4096x4096 fp8)", int(s.sum()), 64, 4096, 4096, s, False, (4096, 1))
+    for B in (8, 64):
+        s = zipf_group_sizes(rng, B, 15, 3, 1)
+        gemm(f"lyra-small expert up+SwiGLU B={B} (16x2048x4096 fp8)", int(s.sum()), 16, 2048, 4096, s, True, (2048, 1))
+        gemm(f"lyra-small expert down B={B} (16x2048x2048 fp8)", int(s.sum()), 16, 2048, 2048, s, False, (2048, 1))
+    for name, K, N, sw in (("q/k/v", 2048, 3072, False), ("out", 2048, 2048, False), ("dense up+SwiGLU", 2048, 6144, True),
+                           ("dense down", 3072, 2048, False)):
+        gemm(f"lyra-small {name} projection B=64 ({K}x{N} fp8)", 64, 1, K, N, [64], sw, (K, 1))
+    gemm("lyra-medium dense up+SwiGLU B=64 (4096x12288 fp8)", 64, 1, 4096, 12288, [64], True, (4096, 1))
+    gemm("lyra-small LM head B=64 (2048x204800 bf16, f32 logits)", 64, 1, 2048, 204800, [64], False, None, fp8=False, out_f32=True)
+    for r in rows:
+        r["cold_GBs"] = r["bytes"] / r["cold_us"] / 1e3
+        r["cold_frac_of_peak"] = r["cold_GBs"] / HBM_PEAK_GBS
+    return rows
+
+
 def traffic_probe(device, mib=256, repeats=4):
     """A plain streaming kernel of known HBM traffic (reads `mib` MiB, writes `mib` MiB per launch), launched a few
     times so that a hardware-counter run of this script can scale FETCH_SIZE / WRITE_SIZE against it."""
@@ -169,6 +319,8 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--cpu-sample", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernels", action="store_true",
+                    help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a copy-like kernel of known size (reference point for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -179,6 +331,13 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.kernels:
+        rows = kernel_table(dev)
+        for r in rows:
+            print(f"| {r['operator']} | {r['case']} | {r['bytes'] / 1e6:.1f} | {r['cold_us']:.1f} | {r['cold_GBs'] / 1e3:.2f} | "
+                  f"{100 * r['cold_frac_of_peak']:.1f} | {r['hot_us']:.1f} |", file=sys.stderr)
+        print(json.dumps({"metric": "operator launch time at model shapes", "unit": "us", "peak_GBs": HBM_PEAK_GBS, "kernels": rows}))
+        return
     cfg, weights, cache = build_model(args.batch, args.ctx, dev)
     elapsed = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
     tokens_per_s = args.batch * args.steps / elapsed

@@ -27,16 +27,19 @@ struct GemmParams {
     const int32_t* group_sizes;
     const float* bias;
     void* out;
-    float* part;  // [ksplit, M, N] float32 partial products when ksplit > 1
+    float* part;  // [ksplit, M, N] float32 partial products when ksplit > 1; grouped: two tile slots per workgroup
+    int* arrivals;  // grouped: arrival counters of split units (zero between launches)
     int M, G, K, N;
     int bk, bn, KB, NB;
     int bn_shift;  // log2(bn): scale columns are power-of-two wide
+    int bk_shift;  // log2(bk) when bk is a power of two, else -1
     int scale_mode;  // 0 none, 1 one scale per lane and k-block (bn % 8 == 0), 2 per column (bk == K)
     int out_f32, swiglu;
     float beta, limit;
     int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
     int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
+    int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
     const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
     float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
@@ -44,6 +47,21 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// Index of the scale block (along K) that weight row k lies in.
+__device__ __forceinline__ int scale_block_of(const GemmParams& p, int k) {
+    k = min(k, p.K - 1);
+    return p.bk_shift >= 0 ? k >> p.bk_shift : k / p.bk;
+}
+
+// Scale of one lane's 8 columns for one K step, fetched like the step's weights (a buffer load in the same in-order
+// stream, so waiting for it never waits for younger loads; a plain pointer load here would drain everything in flight).
+// lane_off: byte offset of the lane's scale column within the group's scale table, or kNoLoad.
+__device__ __forceinline__ float load_step_scale(const GemmParams& p, const __amdgpu_buffer_rsrc_t& rsrc, bool live, int lane_off,
+                                                 int k) {
+    const int soff = __builtin_amdgcn_readfirstlane(live ? scale_block_of(p, k) * p.NB * 4 : 0);
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, live ? lane_off : kNoLoad, soff, 0));
+}
 
 // Residual epilogue of a projection (lyra/model.py:371-374, 631-636): the product is a bf16 array, it is scaled in
 // bf16, then added to the bf16 residual stream.
@@ -426,6 +444,9 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
 
     RawW<FP8> w[DEPTH];
     u32x4 a[DEPTH];
+    [[maybe_unused]] float step_sc[DEPTH];  // STEP_SCALES: the scale of each step in flight travels with its weights
+    const __amdgpu_buffer_rsrc_t scrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(STEP_SCALES ? p.scale : nullptr), 0, STEP_SCALES ? (uint32_t)p.KB * (uint32_t)p.NB * 4u : 0u, 0x00020000);
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
         const bool live = d < n_my;
@@ -438,6 +459,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
         const int kk = (wave + kSmallWaves * d) << 5;
 #pragma unroll
         for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
+        if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, live, (ncol >> p.bn_shift) * 4, kk);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -498,6 +520,8 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
             Pack8 bop[8], av;
 #pragma unroll
             for (int i = 0; i < 4; ++i) av.u[i] = a_ok ? a[d][i] : 0u;
+            [[maybe_unused]] float sc = 1.f;
+            if constexpr (STEP_SCALES) sc = step_sc[d];
             if constexpr (!ONE_ROUND) {
                 __builtin_amdgcn_sched_barrier(0);
                 a[d] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff : kNoLoad,
@@ -512,8 +536,8 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            if constexpr (STEP_SCALES && !ONE_ROUND) step_sc[d] = load_step_scale(p, scrsrc, more, (ncol >> p.bn_shift) * 4, kk_next);
             if constexpr (STEP_SCALES) {
-                const float sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
 #pragma unroll
                 for (int c = 0; c < 8; ++c) {
                     const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
@@ -593,7 +617,10 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
 constexpr int kSplitWaves = 4;
 constexpr int kSplitPitch = 132;  // floats per row of a partial tile in LDS (128 + padding against bank conflicts)
 
-template <bool FP8, int DEPTH, bool STEP_SCALES>
+// STEP_SCALES: 0 scales constant along K (applied to the finished tile); 1 scale blocks shorter than K, every wavefront's
+// rows within one block (its scale applied to its finished tile); 2 one scale per 32-row step.  With 1 and 2 a wavefront
+// takes DEPTH consecutive steps instead of every 4th.
+template <bool FP8, int DEPTH, int STEP_SCALES>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
@@ -603,7 +630,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int ncol = span * 128 + 8 * x;
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
     const int steps = (k1 - k0) >> 5;
-    const int n_my = (steps - wave + kSplitWaves - 1) / kSplitWaves;  // steps wave, wave + 4, ... of the slice (<= DEPTH)
+    // steps wave, wave + 4, ... of the slice (<= DEPTH), or steps wave * DEPTH ... when scales change along K
+    const int n_my = STEP_SCALES ? max(0, min(DEPTH, steps - wave * DEPTH)) : (steps - wave + kSplitWaves - 1) / kSplitWaves;
+    auto step_row = [&](int d) { return k0 + ((STEP_SCALES ? wave * DEPTH + d : wave + kSplitWaves * d) << 5); };
 
     const int row_bytes = p.N * ES;
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -625,7 +654,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
         const bool live = d < n_my;
-        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+        const int kk = step_row(d);
         const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
@@ -633,7 +662,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
         const bool live = d < n_my;
-        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+        const int kk = step_row(d);
 #pragma unroll
         for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
     }
@@ -642,10 +671,16 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
     for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
     const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (ncol >> p.bn_shift) : nullptr;
-    if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
-        const float sc = *sc_lane;
+    [[maybe_unused]] float step_sc[DEPTH];
+    if (FP8 && p.scale_mode == 1 && STEP_SCALES != 2) {
+        const float sc = sc_lane[(size_t)(STEP_SCALES ? scale_block_of(p, step_row(0)) : 0) * p.NB];
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = sc;
+    } else if (FP8 && STEP_SCALES == 2) {
+        const __amdgpu_buffer_rsrc_t scrsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(p.scale), 0, (uint32_t)p.KB * (uint32_t)p.NB * 4u, 0x00020000);
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) step_sc[d] = load_step_scale(p, scrsrc, d < n_my, (ncol >> p.bn_shift) * 4, step_row(d));
     } else if (FP8 && p.scale_mode == 2) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(ncol + c) >> p.bn_shift];
@@ -661,12 +696,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        const int kk = k0 + ((wave + kSplitWaves * d) << 5);
+        const int kk = step_row(d);
         Pack8 bop[8];
 #pragma unroll
         for (int pr = 0; pr < 4; ++pr) convert_pair<FP8>(w[d], pr, bop);
         float sc = 1.f;
-        if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+        if constexpr (STEP_SCALES == 2) sc = step_sc[d];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
             if (mt < n_mt) {
@@ -674,7 +709,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
                 const bool a_ok = row0 + mt * 16 + x < cnt;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) av.u[i] = a_ok ? a[d][mt][i] : 0u;
-                if constexpr (STEP_SCALES) {
+                if constexpr (STEP_SCALES == 2) {
 #pragma unroll
                     for (int c = 0; c < 8; ++c) {
                         const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
@@ -753,88 +788,56 @@ __device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[
 // A unit is up to 64 rows of one expert times one 128-column span over the whole K extent (256-1024 KB of weights).
 // Every workgroup first builds the same unit list in LDS from group_sizes (experts without rows contribute nothing, so
 // their weights are never read; the last groups - shared experts, which carry the most rows - come first) and then takes
-// units blockIdx.x, blockIdx.x + gridDim.x, ...  Within a unit its 4 wavefronts interleave over K in steps of 32 rows
-// with DEPTH steps of weights and activations in flight each; their partial tiles are summed through LDS in a fixed
-// order and bias / SwiGLU / residual follow.  The first operands of the next unit are requested before the current
-// unit's tile is summed and written, so a compute unit keeps streaming across unit boundaries.  No float32 partials
-// in global memory, no second pass, results independent of the grid size.  With SwiGLU a span is 128 gate columns
-// (wavefronts 0, 1, interleaved over K) plus the matching 128 linear columns (wavefronts 2, 3), so every load covers whole
-// 128-byte lines of a weight row; 64 + 64 columns per wavefront would fetch twice as many lines per byte.
-// ROUNDS passes over the DEPTH register sets are unrolled per trip of the K loop: in straight-line code every wait counts
-// exactly the loads issued after the one it needs, whereas the wait at the head of a loop drains nearly everything in
-// flight, so the longer the straight-line stretch the better.
+// units blockIdx.x, blockIdx.x + gridDim.x, ...: at any time the workgroups stream neighbouring column spans of the same
+// weight rows.  Within a unit its 4 wavefronts interleave over K in steps of 32 rows with DEPTH steps of weights and
+// activations in flight each; their partial tiles are summed through LDS in a fixed order and bias / SwiGLU / residual
+// follow.  The first operands of the next unit are requested before the current unit's tile is summed and written, so a
+// compute unit keeps streaming across unit boundaries.
+// The units left over after the last full round of gridDim.x (all of them when there are fewer) would keep only some of
+// the compute units busy - and a compute unit ingests ~30 GB/s whatever the others do - so each of them is cut into S
+// slices along K, S as large as keeps tail * S <= gridDim.x, taken slice by slice in the same order.  A slice's tile goes to
+// a float32 slot in the workspace (device-wide visible stores) and bumps the unit's arrival counter; the workgroup that
+// arrives last adds the S slots in K order - so the result does not depend on who that is - and finishes the tile.
+// Nobody waits for anybody, and results do not depend on timing.
+// With SwiGLU a span is 128 gate columns (wavefronts 0, 1, interleaved over K) plus the matching 128 linear columns
+// (wavefronts 2, 3), so every load covers whole 128-byte lines of a weight row; 64 + 64 columns per wavefront would fetch
+// twice as many lines per byte.  ROUNDS passes over the DEPTH register sets are unrolled per trip of the K loop: in
+// straight-line code every wait counts exactly the loads issued after the one it needs, whereas the wait at the head of a
+// loop drains nearly everything in flight.
 constexpr int kGroupTiles = 4;      // 16-row tiles a unit accumulates (64 rows)
 constexpr int kMaxStreamGroups = 256;
-constexpr int kMaxRowBlocks = 512;  // units / spans the LDS table holds
+constexpr int kMaxRowBlocks = 512;  // row blocks the LDS table holds
+constexpr int kGroupMaxWgs = 256;   // shares (workgroups) of a launch; also the number of arrival counters in use
+constexpr size_t kGemmCounterBytes = 65536;  // start of a matmul workspace: arrival counters, zero between launches
 
-struct StreamUnit {
-    int g, row0, rows;  // group, first row (in the sorted lhs), rows in this block (0: no unit)
-};
+// Exclusive prefix sum of one int per thread over the 256 threads of a workgroup (sm4: 4 ints of LDS, free on entry).
+__device__ __forceinline__ int wg_scan_exclusive(int v, int* sm4, int lane, int wave, int& total) {
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int u = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += u;
+    }
+    if (lane == 63) sm4[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int wv = 0; wv < wave; ++wv) base += sm4[wv];
+    total = sm4[0] + sm4[1] + sm4[2] + sm4[3];
+    return base + incl - v;
+}
 
-template <bool FP8, bool STEP_SCALES, int ROUNDS>
+template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int DEPTH = FP8 ? 4 : 2;
     constexpr int MTM = kGroupTiles;
+    constexpr int TRIP = ROUNDS * DEPTH;  // steps of one wavefront per trip
     extern __shared__ float sm_part[];  // [kSplitWaves][16 * MTM][kSplitPitch]
     __shared__ int sm_blk[kMaxRowBlocks][3];  // (group, first row, rows) of every row block, heavy groups first
-    __shared__ int sm_scan[8];
+    __shared__ int sm_scan[12];
+    __shared__ int sm_last;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
-
-    // ---- unit list: thread t looks at group G-1-t ----
-    const int t = threadIdx.x;
-    int my_cnt = 0, my_before = 0;  // rows of "my" group and rows of all groups before it (in lhs order)
-    {
-        // rows before group g = sum of sizes of groups < g: an inclusive scan over groups in natural order
-        const int gnat = t;  // natural order for the scan
-        int v = gnat < p.G ? p.group_sizes[gnat] : 0;
-        int incl = v;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int u = __shfl_up(incl, o, kWave);
-            if (lane >= o) incl += u;
-        }
-        if (lane == 63) sm_scan[wave] = incl;
-        __syncthreads();
-        int base = 0;
-        for (int wv = 0; wv < wave; ++wv) base += sm_scan[wv];
-        const int before = base + incl - v;
-        // hand (before, size) of natural group gnat to the thread that owns it in heavy-first order: thread G-1-gnat
-        __syncthreads();
-        int* tmp = (int*)sm_part;  // scratch before the tiles are used
-        if (gnat < p.G) {
-            tmp[2 * (p.G - 1 - gnat)] = min(before, p.M);
-            tmp[2 * (p.G - 1 - gnat) + 1] = max(0, min(v, p.M - min(before, p.M)));
-        }
-        __syncthreads();
-        if (t < p.G) {
-            my_before = tmp[2 * t];
-            my_cnt = tmp[2 * t + 1];
-        }
-    }
-    const int my_blocks = (my_cnt + 16 * MTM - 1) / (16 * MTM);
-    int blk_incl = my_blocks;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int u = __shfl_up(blk_incl, o, kWave);
-        if (lane >= o) blk_incl += u;
-    }
-    __syncthreads();
-    if (lane == 63) sm_scan[4 + wave] = blk_incl;
-    __syncthreads();
-    int blk_base = 0;
-    for (int wv = 0; wv < wave; ++wv) blk_base += sm_scan[4 + wv];
-    const int n_blocks = min(kMaxRowBlocks, sm_scan[4] + sm_scan[5] + sm_scan[6] + sm_scan[7]);
-    for (int i = 0; i < my_blocks; ++i) {
-        const int j = blk_base + blk_incl - my_blocks + i;
-        if (j < kMaxRowBlocks) {
-            sm_blk[j][0] = p.G - 1 - t;
-            sm_blk[j][1] = my_before + i * 16 * MTM;
-            sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
-        }
-    }
-    __syncthreads();
 
     // wide: a unit is two sets of 128 columns, each taken by a pair of wavefronts that interleave over K (gate and linear
     // columns with SwiGLU, else two adjacent spans); otherwise one set of 128 columns and all 4 wavefronts interleave
@@ -843,33 +846,94 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     const int kw = wide ? 2 : kSplitWaves;
     const int wslot = wide ? (wave & 1) : wave, half = wide ? (wave >> 1) : 0;
     const int half_stride = p.swiglu ? (p.N >> 1) : 128, span_cols = p.swiglu || !wide ? 128 : 256;
-    const int n_units = n_blocks * spans;
+    const int tile_cols = wide ? 256 : 128;  // floats per row of a workspace slot
     const int NO = p.swiglu ? p.N >> 1 : p.N;
     const int q = threadIdx.x & 31;
     const int row_bytes = p.N * ES;
     const int steps = p.K >> 5;
-    const int n_my = (steps - wslot + kw - 1) / kw;
+    const int n_my = (steps - wslot + kw - 1) / kw;                      // steps of this wavefront in a whole unit
+    const int trips = ((steps + kw - 1) / kw + TRIP - 1) / TRIP;        // trips of a whole unit (same for every wavefront)
+
+    // ---- unit list: thread t looks at group G-1-t ----
+    const int t = threadIdx.x;
+    int my_cnt = 0, my_before = 0;  // rows of "my" group and rows of all groups before it (in lhs order)
+    int total_rows;
+    {
+        const int v = t < p.G ? p.group_sizes[t] : 0;
+        const int before = wg_scan_exclusive(v, sm_scan, lane, wave, total_rows);
+        // hand (before, size) of natural group t to the thread that owns it in heavy-first order: thread G-1-t
+        int* tmp = (int*)sm_part;  // scratch before the tiles are used
+        if (t < p.G) {
+            tmp[2 * (p.G - 1 - t)] = min(before, p.M);
+            tmp[2 * (p.G - 1 - t) + 1] = max(0, min(v, p.M - min(before, p.M)));
+        }
+        __syncthreads();
+        if (t < p.G) {
+            my_before = tmp[2 * t];
+            my_cnt = tmp[2 * t + 1];
+        }
+    }
+    const int my_blocks = (my_cnt + 16 * MTM - 1) / (16 * MTM);
+    int n_blocks_all;
+    const int blk_base = wg_scan_exclusive(my_blocks, sm_scan + 4, lane, wave, n_blocks_all);
+    const int n_blocks = min(kMaxRowBlocks, n_blocks_all);  // (the host keeps n_blocks_all <= kMaxRowBlocks)
+    for (int i = 0; i < my_blocks; ++i) {
+        const int j = blk_base + i;
+        if (j < kMaxRowBlocks) {
+            sm_blk[j][0] = p.G - 1 - t;
+            sm_blk[j][1] = my_before + i * 16 * MTM;
+            sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
+        }
+    }
+    __syncthreads();
+    const int n_units = __builtin_amdgcn_readfirstlane(n_blocks * spans);  // (same in every lane: tell the compiler)
+    const int nwg = gridDim.x;
+    // whole units in full rounds of nwg; when there is not even one full round, the units are cut into `slices` K slices each
+    // (a power of two that divides trips).  After a full round slicing the rest was measured to cost as much as it saves:
+    // the few workgroups of a last partial round stream faster, having the memory system to themselves.
+    const int n_whole = n_units / nwg * nwg, tail = n_units - n_whole;
+    int slices = 1;
+    while (SLICED && tail > 0 && n_whole == 0 && 2 * slices * tail <= nwg && trips % (2 * slices) == 0 && 2 * slices <= p.max_slices) slices *= 2;
+    const int trips_per_slice = trips / slices;
+    const int n_work = n_whole + tail * slices;  // work items: unit v for v < n_whole, else slice (v - n_whole) / tail of a tail unit
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
 
-    // state of the unit whose operands are in flight / being consumed
-    int u = blockIdx.x;
+    // state of the work item whose operands are in flight / being consumed
+    int v = blockIdx.x;
+    int seg_u = 0, seg_r0 = 0, seg_r1 = 0;  // its unit and trips [r0, r1) of it
     int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
     __amdgpu_buffer_rsrc_t wrsrc;
     u32x4 a[DEPTH][MTM];
     RawW<FP8> w[DEPTH];
+    [[maybe_unused]] float step_sc[DEPTH];  // STEP_SCALES: the scale of each step in flight travels with its weights
+    [[maybe_unused]] int sc_voff = kNoLoad;
+    const __amdgpu_buffer_rsrc_t scrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(FP8 ? p.scale : nullptr), 0, FP8 ? (uint32_t)p.G * (uint32_t)p.KB * (uint32_t)p.NB * 4u : 0u, 0x00020000);
 
-    // Looks unit `uu` up and requests its first DEPTH steps (a unit past the end requests nothing).
-    auto open_unit = [&](int uu) {
-        const bool valid = uu < n_units;
-        const int blk = valid ? uu / spans : 0;
-        span = valid ? uu - blk * spans : 0;
-        g = valid ? sm_blk[blk][0] : 0;
-        row0 = valid ? sm_blk[blk][1] : 0;
-        rows = valid ? sm_blk[blk][2] : 0;
+    // Looks work item vv up and requests its first DEPTH steps (an item past the end requests nothing).
+    auto open_segment = [&](int vv) {
+        const bool valid = vv < n_work;
+        if constexpr (SLICED) {
+            const int ti = vv - n_whole;  // >= 0: slice ti / tail of tail unit ti % tail
+            const int sl = (valid && ti >= 0) ? ti / tail : 0;
+            seg_u = __builtin_amdgcn_readfirstlane(!valid ? 0 : (ti >= 0 ? n_whole + (ti - sl * tail) : vv));
+            seg_r0 = __builtin_amdgcn_readfirstlane((valid && ti >= 0) ? sl * trips_per_slice : 0);
+            seg_r1 = __builtin_amdgcn_readfirstlane(!valid ? 0 : (ti >= 0 ? seg_r0 + trips_per_slice : trips));
+        } else {
+            seg_u = valid ? vv : 0;
+            seg_r0 = 0;
+            seg_r1 = valid ? trips : 0;
+        }
+        const int blk = seg_u / spans;
+        span = seg_u - blk * spans;
+        g = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][0] : 0);
+        row0 = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][1] : 0);
+        rows = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][2] : 0);
         ncol = half * half_stride + span * span_cols + 8 * x;
         wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
                                                   (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
         wvoff = valid ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
+        if constexpr (STEP_SCALES) sc_voff = valid ? (g * p.KB * p.NB + (ncol >> p.bn_shift)) * 4 : kNoLoad;
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) {
             const int r = mt * 16 + x;
@@ -879,63 +943,69 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         }
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
-            const bool live = d < n_my;
-            const int kk = (wslot + kw * d) << 5;
+            const int idx = seg_r0 * TRIP + d;
+            const bool live = valid && idx < n_my;
+            const int kk = (wslot + kw * idx) << 5;
             const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
 #pragma unroll
             for (int mt = 0; mt < MTM; ++mt)
                 a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
+            if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, live, sc_voff, kk);
         }
     };
 
-    open_unit(u);
-    while (u < n_units) {
+    // Bias / SwiGLU / residual and the store of 4 (wide: 4 + 4) finished columns of one output row.
+    auto finish_row = [&](int fg, int frow, int fspan, float (&vg)[4], float (&vl)[4]) {
+        const int oc = fspan * span_cols + 4 * q;
+        if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
+            float zero[4] = {0.f, 0.f, 0.f, 0.f};
+            group_epilogue(p, vg, zero, fg, frow, oc, NO);
+            group_epilogue(p, vl, zero, fg, frow, oc + 128, NO);
+        } else {
+            group_epilogue(p, vg, vl, fg, frow, oc, NO);
+        }
+    };
+    // workspace slots: [tail unit][K slice][64 rows][tile_cols] float32, at most kGroupMaxWgs of them
+    const __amdgpu_buffer_rsrc_t slot_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        p.part, 0, (uint32_t)(kGroupMaxWgs * 16 * MTM) * (uint32_t)tile_cols * 4u, 0x00020000);
+
+    open_segment(v);
+    while (v < n_work) {
+        const int cur_u = seg_u, r0 = seg_r0, r1 = seg_r1;
         const int cur_g = g, cur_row0 = row0, cur_rows = rows, cur_span = span, cur_ncol = ncol;
         const int n_mt = (cur_rows + 15) >> 4;
         const __amdgpu_buffer_rsrc_t cur_wrsrc = wrsrc;
         const int cur_wvoff = wvoff;
+        [[maybe_unused]] const int cur_sc_voff = sc_voff;
         int cur_avoff[MTM];
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) cur_avoff[mt] = avoff[mt];
-        // column scales: requested behind the first operands, needed only when the tile is written out
-        const float* sc_lane =
-            (FP8 && p.scale_mode == 1) ? p.scale + (size_t)cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift) : nullptr;
-        float colscale[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
-        if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
-            const float sc = *sc_lane;
-#pragma unroll
-            for (int c = 0; c < 8; ++c) colscale[c] = sc;
-        } else if (FP8 && p.scale_mode == 2) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(size_t)cur_g * p.NB + ((cur_ncol + c) >> p.bn_shift)];
-        }
         f32x4 acc[MTM][8];
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt)
 #pragma unroll
             for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        // every pass issues the same loads (past the end they fetch nothing) and multiplies zeros there
-        const int n_rounds = (n_my + DEPTH - 1) / DEPTH;  // a multiple of ROUNDS (the host checks)
-        for (int round0 = 0; round0 < n_rounds; round0 += ROUNDS) {
+        // every pass issues the same loads (past the end of the segment they fetch nothing) and multiplies zeros there
+        const int idx_end = min(n_my, r1 * TRIP);
+        for (int trip = r0; trip < r1; ++trip) {
 #pragma unroll
             for (int ur = 0; ur < ROUNDS; ++ur) {
-                const int base = (round0 + ur) * DEPTH;
 #pragma unroll
                 for (int d = 0; d < DEPTH; ++d) {
-                    const int idx = base + d;
+                    const int idx = (trip * ROUNDS + ur) * DEPTH + d;
                     const int kk = (wslot + kw * idx) << 5;
                     const int kk_next = kk + ((kw * DEPTH) << 5);
-                    const bool more = idx + DEPTH < n_my;
+                    const bool more = idx + DEPTH < idx_end;
                     Pack8 bop[8], av[MTM];
 #pragma unroll
                     for (int mt = 0; mt < MTM; ++mt)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) av[mt].u[i] = a[d][mt][i];
+                    float sc = 1.f;
+                    if constexpr (STEP_SCALES) sc = step_sc[d];
                     __builtin_amdgcn_sched_barrier(0);
                     const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
 #pragma unroll
@@ -948,8 +1018,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         load_w_pair_if<FP8>(more, w[d], pr, cur_wrsrc, cur_wvoff, kk_next, row_bytes);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    float sc = 1.f;
-                    if constexpr (STEP_SCALES) sc = sc_lane[(size_t)(min(kk, p.K - 1) / p.bk) * p.NB];
+                    if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, more, cur_sc_voff, kk_next);
 #pragma unroll
                     for (int mt = 0; mt < MTM; ++mt) {
                         if (mt < n_mt) {
@@ -972,9 +1041,25 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             }
         }
 
-        // the next unit's first operands fly while this unit's tile is summed and written
-        u += gridDim.x;
-        open_unit(u);
+        // Scales that are constant along K are applied to the finished tile.  They are requested here, ahead of the next
+        // item's operands (loads return in order), and arrive while those are being requested.
+        float colscale[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            colscale[c] = 1.f;
+            if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
+                const int off = (cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift)) * 4;
+                if (c == 0) colscale[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));
+                else colscale[c] = colscale[0];
+            } else if (FP8 && p.scale_mode == 2) {
+                const int off = (cur_g * p.NB + ((cur_ncol + c) >> p.bn_shift)) * 4;
+                colscale[c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // the next item's first operands fly while this tile is summed and written
+        v += nwg;
+        open_segment(v);
 
         float* mine = sm_part + wave * (16 * MTM * kSplitPitch);
 #pragma unroll
@@ -991,13 +1076,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             }
         }
         __syncthreads();
-        const int oc = cur_span * span_cols + 4 * q;
         constexpr int TS = 16 * MTM * kSplitPitch;  // floats per wavefront tile
-        for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
+        // Sum of the wavefront tiles for 4 columns of row r: vg (and vl, the second set of 128 columns of a wide unit).
+        auto tile_row = [&](int r, float (&vg)[4], float (&vl)[4]) {
             const float* src = sm_part + r * kSplitPitch + 4 * q;
             const f32x4 t0 = *(const f32x4*)src, t1 = *(const f32x4*)(src + TS), t2 = *(const f32x4*)(src + 2 * TS),
                         t3 = *(const f32x4*)(src + 3 * TS);
-            float vg[4], vl[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (wide) {
@@ -1008,20 +1092,76 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                     vl[c] = 0.f;
                 }
             }
-            if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
-                float zero[4] = {0.f, 0.f, 0.f, 0.f};
-                group_epilogue(p, vg, zero, cur_g, cur_row0 + r, oc, NO);
-                group_epilogue(p, vl, zero, cur_g, cur_row0 + r, oc + 128, NO);
-            } else {
-                group_epilogue(p, vg, vl, cur_g, cur_row0 + r, oc, NO);
+        };
+        bool finish = !SLICED || (r0 == 0 && r1 == trips);  // the whole unit was summed here
+        if (SLICED && !finish) {
+            // a K slice of a unit: publish the tile, count the arrival; whoever arrives last adds all slices in K order
+            const int ui = cur_u - n_whole;                          // tail unit
+            const int my_slot = ui * slices + r0 / trips_per_slice;  // slots of a unit are consecutive, in K order
+            for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
+                float vg[4], vl[4];
+                tile_row(r, vg, vl);
+                const int off = ((my_slot * (16 * MTM) + r) * tile_cols + 4 * q) * 4;
+                store_agent_b128(slot_rsrc, off, f32x4{vg[0], vg[1], vg[2], vg[3]});
+                if (wide) store_agent_b128(slot_rsrc, off + 512, f32x4{vl[0], vl[1], vl[2], vl[3]});
+            }
+            wait_all_memory();  // this lane's part has reached device-wide visibility
+            __syncthreads();    // ... and so has everybody else's in this workgroup, before the arrival is counted
+            if (threadIdx.x == 0) {
+                const int seen = add_agent(&p.arrivals[ui], 1);
+                sm_last = seen == slices - 1;
+                if (sm_last) store_agent(&p.arrivals[ui], 0);  // leave the counter ready for the next launch
+            }
+            __syncthreads();
+            finish = sm_last;
+            if (finish) {
+                // the sums replace this thread's part of the wavefront tiles (tile 0, and tile 2 for the second set of
+                // columns; the others become zero), so that one epilogue serves both cases
+                f32x4 vg[8], vl[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) vg[j] = vl[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int c = 0; c < slices; ++c) {
+                    const int base = (ui * slices + c) * (16 * MTM);
+                    f32x4 tg[8], tl[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int r = (threadIdx.x >> 5) + 8 * j;
+                        const int off = r < cur_rows ? ((base + r) * tile_cols + 4 * q) * 4 : kNoLoad;
+                        tg[j] = load_agent_b128(slot_rsrc, off);
+                        tl[j] = load_agent_b128(slot_rsrc, wide ? off + 512 : kNoLoad);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        vg[j] += tg[j];
+                        vl[j] += tl[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int r = (threadIdx.x >> 5) + 8 * j;
+                    if (r < cur_rows) {
+                        float* dst = sm_part + r * kSplitPitch + 4 * q;
+                        *(f32x4*)dst = vg[j];
+                        *(f32x4*)(dst + TS) = f32x4{0.f, 0.f, 0.f, 0.f};
+                        *(f32x4*)(dst + 2 * TS) = vl[j];
+                        *(f32x4*)(dst + 3 * TS) = f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+            }
+        }
+        if (finish) {
+            for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
+                float vg[4], vl[4];
+                tile_row(r, vg, vl);
+                finish_row(cur_g, cur_row0 + r, cur_span, vg, vl);
             }
         }
         __syncthreads();  // the tiles are free for the next unit
     }
-    wait_all_memory();  // (requests of a unit past the end return nothing, but must not outlive the wavefront's registers)
+    wait_all_memory();  // (requests of an item past the end return nothing, but must not outlive the wavefront's registers)
 
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
-    const int total = sm_scan[0] + sm_scan[1] + sm_scan[2] + sm_scan[3];
+    const int total = total_rows;
     const int pad_rows = p.M - min(total, p.M);
     const int pad_spans = p.swiglu ? spans : p.N / 128;
     for (int i = blockIdx.x; i < pad_rows * pad_spans; i += gridDim.x) {
@@ -1120,7 +1260,8 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
     const dim3 grid(pl.spans, pl.ksplit, pl.row_par), block(kSplitWaves * 64);
     const size_t lds = (size_t)kSplitWaves * 64 * kSplitPitch * sizeof(float);
     const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4
-    const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+    // scales that change along K: free when every wavefront's rows (32 * depth) lie within one scale block
+    const int step_scales = !(fp8 && p.scale_mode == 1 && p.bk < p.K) ? 0 : (p.bk % (32 * std::max(1, std::min(depth, 4))) == 0 ? 1 : 2);
 #define LYRA_SPLITK(F, D, S)                                                                                          \
     do {                                                                                                              \
         static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S>,          \
@@ -1135,9 +1276,10 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
         else if (depth == 3) LYRA_SPLITK(F, 3, S); \
         else LYRA_SPLITK(F, 4, S);            \
     } while (0)
-    if (step_scales) LYRA_SPLITK_D(true, true);
-    else if (fp8) LYRA_SPLITK_D(true, false);
-    else LYRA_SPLITK_D(false, false);
+    if (step_scales == 1) LYRA_SPLITK_D(true, 1);
+    else if (step_scales == 2) LYRA_SPLITK_D(true, 2);
+    else if (fp8) LYRA_SPLITK_D(true, 0);
+    else LYRA_SPLITK_D(false, 0);
 #undef LYRA_SPLITK_D
 #undef LYRA_SPLITK
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
@@ -1149,8 +1291,10 @@ extern "C" size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fus
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return 0;
     // the split factor may depend on the scale block; size for the largest split the plan can choose
     const lyra::GemmPlan pl = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu);
-    if (pl.ksplit == 1 && !pl.split_k) return 256;
-    return ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+    if (pl.grouped)  // one tile slot of 64 rows x 256 columns per workgroup, behind the counters
+        return lyra::kGemmCounterBytes + (size_t)lyra::kGroupMaxWgs * 16 * lyra::kGroupTiles * 256 * sizeof(float);
+    if (pl.ksplit == 1 && !pl.split_k) return lyra::kGemmCounterBytes;
+    return lyra::kGemmCounterBytes + ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
 }
 
 extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
@@ -1181,11 +1325,13 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.bk = p.bn = 1;
     p.KB = p.NB = 1;
     p.bn_shift = 0;
+    p.bk_shift = 0;
     if (fp8) {
         if (bk <= 0 || bn <= 0 || K % bk || N % bn) return LYRA_E_BADARG;
         if (bn & (bn - 1)) return LYRA_E_UNSUPPORTED;  // scale columns must be a power of two wide
         p.bk = bk; p.bn = bn; p.KB = K / bk; p.NB = N / bn;
         p.bn_shift = __builtin_ctz((unsigned)bn);
+        p.bk_shift = (bk & (bk - 1)) ? -1 : __builtin_ctz((unsigned)bk);
         if (bn % 8 == 0 && (bk % 32 == 0 || bk == K)) p.scale_mode = 1;
         else if (bk == K) p.scale_mode = 2;
         else return LYRA_E_UNSUPPORTED;
@@ -1208,28 +1354,44 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.kpart = pl.kpart;
     p.row_map = lhs_row_map;
     p.wide = pl.wide;
+    static const int max_slices_env = [] {
+        const char* e = getenv("LYRA_GEMM_MAX_SLICES");  // tuning override, read once
+        return e ? atoi(e) : 64;
+    }();
+    p.max_slices = max_slices_env;
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
     p.post_scale = post_scale != 0;
-    if (pl.ksplit > 1 || pl.split_k) {
-        const size_t need = ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+    p.arrivals = nullptr;
+    if (pl.ksplit > 1 || pl.split_k || pl.grouped) {
+        // the first kGemmCounterBytes belong to the grouped kernel's arrival counters, whichever kernel runs
+        const size_t need = lyra_decode_gemm_workspace(M, G, K, N, fused_swiglu);
         if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
-        p.part = (float*)workspace;
+        p.arrivals = (int*)workspace;
+        p.part = (float*)((char*)workspace + kGemmCounterBytes);
     }
 
     hipStream_t st = (hipStream_t)stream;
     if (pl.grouped) {
         // one workgroup per compute unit (more would only queue behind the LDS tiles), fewer when there is less work
         const long most_units = (long)pl.spans * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
-        const dim3 ggrid((unsigned)std::max(1L, std::min(256L, most_units))), gblock(kSplitWaves * 64);
+        const int gkw = (fused_swiglu || pl.wide) ? 2 : kSplitWaves;
+        const long trips_least = std::max(1, ((K / 32 + gkw - 1) / gkw + 7) / 8);  // trips per unit (at least)
+        const dim3 ggrid((unsigned)std::max(1L, std::min((long)kGroupMaxWgs, most_units * trips_least))), gblock(kSplitWaves * 64);
         const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
         const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
-#define LYRA_GROUP_R(F, S, R)                                                                                         \
+#define LYRA_GROUP_RS(F, S, R, C)                                                                                     \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R>,           \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C>,        \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R>), ggrid, gblock, glds, st, p);                          \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C>), ggrid, gblock, glds, st, p);                       \
+    } while (0)
+    // fewer units than workgroups whatever the group sizes: the variant that cuts units into K slices
+#define LYRA_GROUP_R(F, S, R)                                               \
+    do {                                                                    \
+        if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
+        else LYRA_GROUP_RS(F, S, R, false);                                 \
     } while (0)
 #define LYRA_GROUP(F, S, DEPTH_)                                                          \
     do {                                                                                  \
@@ -1244,6 +1406,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         else LYRA_GROUP(false, false, 2);
 #undef LYRA_GROUP
 #undef LYRA_GROUP_R
+#undef LYRA_GROUP_RS
         return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
     }
     if (pl.split_k) {
@@ -1323,6 +1486,7 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
         if (bn & (bn - 1)) return LYRA_E_UNSUPPORTED;
         p.bk = bk; p.bn = bn; p.KB = K / bk; p.NB = N / bn;
         p.bn_shift = __builtin_ctz((unsigned)bn);
+        p.bk_shift = (bk & (bk - 1)) ? -1 : __builtin_ctz((unsigned)bk);
         if (bn % 8 == 0 && (bk % 32 == 0 || bk == K)) p.scale_mode = 1;
         else if (bk == K) p.scale_mode = 2;
         else return LYRA_E_UNSUPPORTED;

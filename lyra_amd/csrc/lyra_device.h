@@ -124,6 +124,20 @@ __device__ __forceinline__ void store_agent(int* p, int v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void wait_all_memory() { __builtin_amdgcn_s_waitcnt(0); }
+// 16-byte forms of store_agent / load_agent through a buffer descriptor (cache-policy bit 4 = sc1: agent scope on gfx950).
+__device__ __forceinline__ void store_agent_b128(__amdgpu_buffer_rsrc_t rsrc, int voff, f32x4 v) {
+    u32x4 d;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) d[i] = __float_as_uint(v[i]);
+    __builtin_amdgcn_raw_buffer_store_b128(d, rsrc, voff, 0, 16);
+}
+__device__ __forceinline__ f32x4 load_agent_b128(__amdgpu_buffer_rsrc_t rsrc, int voff) {
+    const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 16);
+    f32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(d[i]);
+    return v;
+}
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll

@@ -76,7 +76,7 @@ def test_workspace_sizes_are_host_arithmetic():
     assert L.lyra_argmax_workspace(64, 201088) % 256 == 0 and L.lyra_argmax_workspace(0, 5) == 0
     assert L.lyra_decode_attention_workspace(0, 16, 4, 512, 128, 0) == 0
     moe = L.lyra_decode_gemm_workspace(256, 16, 2048, 4096, 1)
-    assert moe % 256 == 0 and moe >= 256
+    assert moe == 65536 + 256 * 64 * 256 * 4  # arrival counters + one 64-row x 256-column float32 tile slot per workgroup
     splits = L.lyra_decode_gemm_splits(64, 2048, 3072, 2048)
-    assert splits >= 2 and L.lyra_decode_gemm_workspace(64, 1, 2048, 3072, 0) == splits * 64 * 3072 * 4  # K slices of a dense projection
+    assert splits >= 2 and L.lyra_decode_gemm_workspace(64, 1, 2048, 3072, 0) == 65536 + splits * 64 * 3072 * 4  # counters + K slices
     assert L.lyra_decode_gemm_splits(64, 2048, 100, 2048) == 0
