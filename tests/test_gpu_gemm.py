@@ -237,3 +237,22 @@ def test_many_experts_unit_list(G, M, K, N, swiglu):
     c = _case(8, M, G, K, N, sizes, kind="fp8", block=(K, 1), bias=True, w_std=0.05)
     _note(f"gemm unit list G={G} M={M} swiglu={swiglu} rows={int(sizes.sum())}")
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list")
+
+
+@pytest.mark.parametrize("kind,block,swiglu", [
+    ("fp8", (2048, 1), True), ("fp8", (2048, 1), False), ("fp8", (256, 256), True), ("bf16", None, False),
+])
+def test_few_units_are_cut_into_k_slices(kind, block, swiglu):
+    """Fewer (row block, column span) units than compute units: every unit is cut along K, the slices meet in the
+    workspace and the last workgroup to arrive sums them in K order.  Run three times on one workspace: the arrival
+    counters must be back at zero after every launch, and the result must not depend on which workgroup came last."""
+    G, M, K, N = 8, 6, 2048, 1024
+    sizes = np.array([1, 0, 2, 0, 0, 1, 0, 2], np.int32)
+    c = _case(9, M, G, K, N, sizes, kind=kind, block=block, bias=True, w_std=0.05)
+    _note(f"gemm k-slices kind={kind} block={block} swiglu={swiglu}")
+    want = _want(c, swiglu, big=True)
+    first = _run(c, swiglu)
+    U.assert_close(first, want, what="k slices")
+    for _ in range(2):
+        again = _run(c, swiglu)
+        assert np.array_equal(again, first), "the sum over K slices depends on arrival order or on stale counters"
