@@ -784,6 +784,39 @@ __device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[
     }
 }
 
+__device__ __forceinline__ f32x4 load_f32x4(__amdgpu_buffer_rsrc_t rsrc, int voff) {
+    const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0);
+    return f32x4{__uint_as_float(d[0]), __uint_as_float(d[1]), __uint_as_float(d[2]), __uint_as_float(d[3])};
+}
+// 4 consecutive bf16 values as float32
+__device__ __forceinline__ f32x4 load_bf16x4(__amdgpu_buffer_rsrc_t rsrc, int voff) {
+    const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, 0, 0);
+    return f32x4{__uint_as_float(d[0] << 16), __uint_as_float(d[0] & 0xFFFF0000u), __uint_as_float(d[1] << 16),
+                 __uint_as_float(d[1] & 0xFFFF0000u)};
+}
+
+// Finishes 4 consecutive output columns of one row of a unit, all operands in registers: v the accumulated columns (gate
+// columns with SwiGLU, then l the matching linear columns), their biases (zeros when there are none), res the 4 residual
+// values.  The same arithmetic, in the same order, as group_epilogue.
+__device__ __forceinline__ void finish4(const GemmParams& p, f32x4 v, f32x4 l, f32x4 bias_v, f32x4 bias_l, f32x4 res, size_t oidx) {
+    float o[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float a = v[c] + bias_v[c];
+        if (p.swiglu) a = swiglu_one(a, l[c] + bias_l[c], p.beta, p.limit);
+        if (p.post_scale) a = round_bf16(round_bf16(a) * p.out_scale) + res[c];
+        o[c] = a;
+    }
+    if (p.out_f32) {
+        *(f32x4*)((float*)p.out + oidx) = f32x4{o[0], o[1], o[2], o[3]};
+    } else {
+        u32x2 d;
+        d[0] = pack_bf16(o[0], o[1]);
+        d[1] = pack_bf16(o[2], o[3]);
+        *(u32x2*)((uint16_t*)p.out + oidx) = d;
+    }
+}
+
 // ---- several groups (MoE experts), a handful of rows each: workgroups walk a list of (row block, column span) units -----
 // A unit is up to 64 rows of one expert times one 128-column span over the whole K extent (256-1024 KB of weights).
 // Every workgroup first builds the same unit list in LDS from group_sizes (experts without rows contribute nothing, so
@@ -967,6 +1000,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             group_epilogue(p, vg, vl, fg, frow, oc, NO);
         }
     };
+    // bias [G, N] float32 and residual [M, NO] bf16 through descriptors, so that an absent operand reads as zeros
+    const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(p.bias), 0, p.bias ? (uint32_t)p.G * (uint32_t)p.N * 4u : 0u, 0x00020000);
+    const __amdgpu_buffer_rsrc_t res_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.residual), 0, p.residual ? (uint32_t)p.M * (uint32_t)NO * 2u : 0u, 0x00020000);
     // workspace slots: [tail unit][K slice][64 rows][tile_cols] float32, at most kGroupMaxWgs of them
     const __amdgpu_buffer_rsrc_t slot_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         p.part, 0, (uint32_t)(kGroupMaxWgs * 16 * MTM) * (uint32_t)tile_cols * 4u, 0x00020000);
@@ -1150,10 +1188,35 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             }
         }
         if (finish) {
-            for (int r = threadIdx.x >> 5; r < cur_rows; r += 8) {
-                float vg[4], vl[4];
-                tile_row(r, vg, vl);
-                finish_row(cur_g, cur_row0 + r, cur_span, vg, vl);
+            // biases of this thread's columns once per unit; residual values per row; every load unconditional (a null
+            // operand is read with an offset outside its descriptor and yields zeros), rows two at a time
+            const int oc = cur_span * span_cols + 4 * q;
+            const int oc2 = p.swiglu ? NO + oc : oc + 128;  // second set of columns of a wide unit: linear columns, or the next span
+            const f32x4 bias_v = load_f32x4(bias_rsrc, p.bias ? (cur_g * p.N + oc) * 4 : kNoLoad);
+            const f32x4 bias_l = load_f32x4(bias_rsrc, (p.bias && wide) ? (cur_g * p.N + oc2) * 4 : kNoLoad);
+            const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int r = threadIdx.x >> 5; r < cur_rows; r += 16) {
+                const int rb = min(r + 8, 16 * MTM - 1);  // second row of the pair (clamped: read, not written, when past the end)
+                const bool two = r + 8 < cur_rows;
+                float ag[4], al[4], bg[4], bl[4];
+                tile_row(r, ag, al);
+                tile_row(rb, bg, bl);
+                const size_t oa = (size_t)(cur_row0 + r) * NO + oc, ob = (size_t)(cur_row0 + rb) * NO + oc;
+                f32x4 ra = load_bf16x4(res_rsrc, p.residual ? (int)(oa * 2) : kNoLoad);
+                f32x4 rb4 = load_bf16x4(res_rsrc, (p.residual && two) ? (int)(ob * 2) : kNoLoad);
+                if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
+                    const f32x4 ra2 = load_bf16x4(res_rsrc, p.residual ? (int)((oa + 128) * 2) : kNoLoad);
+                    const f32x4 rb2 = load_bf16x4(res_rsrc, (p.residual && two) ? (int)((ob + 128) * 2) : kNoLoad);
+                    finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
+                    finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
+                    if (two) {
+                        finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
+                        finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
+                    }
+                } else {
+                    finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, oa);
+                    if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, ob);
+                }
             }
         }
         __syncthreads();  // the tiles are free for the next unit
