@@ -91,7 +91,9 @@ int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t s
  *   fused_swiglu  out[:, j] = (clip(t[:, N/2+j], +-limit) + 1) * g * sigmoid(beta*g),
  *               g = min(t[:, j], limit)  (lyra/kernels/common.py:98-114); out is then [M,N/2]
  *   out         [M,N] or [M,N/2], out_dtype (bf16 or float32)
- *   workspace   at least lyra_decode_gemm_workspace(...) bytes, 256-byte aligned
+ *   workspace   at least lyra_decode_gemm_workspace(...) bytes, 256-byte aligned.  Its first 64 KiB hold arrival
+ *               counters (units cut into K slices meet there): zero the buffer once after allocating it
+ *               (lyra_workspace_init); every call leaves the counters at zero.  Float32 partial products follow.
  * Supported: K % 32 == 0, N % 128 == 0 (N % 256 == 0 with fused_swiglu), G <= 8191; fp8 blocks with bn a
  * power of two, and either (bn % 8 == 0 and (bk % 32 == 0 or bk == K)) or bk == K.
  */
