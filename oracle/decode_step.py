@@ -35,8 +35,10 @@ def _gemm(lhs, w, sizes, *, swiglu=False, beta=1.702, limit=7.0, use_c=False, ou
     return y
 
 
-def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False):
+def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins=None):
     """tokens [B] int; weights/cache: dicts of NumPy arrays mirroring lyra_amd.model; pos: int.
+    router_margins: optional list; receives one float32 [B] array per MoE layer, the gap between the last router logit
+    that is selected and the first that is not (top-k is discontinuous: a row with a tiny gap is not a parity case).
 
     cache["k"][l], cache["v"][l]: float32 [B,K,S,H] (bf16 cache) or (qval uint8, scale f32 [B,K,S,1]); updated in
     place.  Returns float32 logits [B, padded_vocab] with -inf beyond vocab_size.
@@ -90,6 +92,10 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False):
             logits = xn.astype(np.float32) @ m["router"]
             if m["router_bias"] is not None:
                 logits = logits + m["router_bias"]
+            if router_margins is not None:
+                srt = np.sort(logits, axis=-1)[:, ::-1]
+                kr = cfg.n_active_routed_experts
+                router_margins.append((srt[:, kr - 1] - srt[:, kr]).astype(np.float32) if kr < srt.shape[1] else np.full(B, np.inf, np.float32))
             scores, active_map, groups = O.route_tokens(logits, cfg.n_active_routed_experts, cfg.n_routed_experts, cfg.n_shared_experts)
             topk = cfg.n_active_experts
             perm, dest = O.bpermute(active_map, groups, cfg.n_experts)
