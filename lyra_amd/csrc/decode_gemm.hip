@@ -1026,6 +1026,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 #pragma unroll
             for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+        [[maybe_unused]] int cur_blk = -1;     // STEP_SCALES: scale block the accumulators are expressed in, and its scale
+        [[maybe_unused]] float s_cur = 1.f;
         // every pass issues the same loads (past the end of the segment they fetch nothing) and multiplies zeros there
         const int idx_end = min(n_my, r1 * TRIP);
         for (int trip = r0; trip < r1; ++trip) {
@@ -1057,22 +1059,35 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, more, cur_sc_voff, kk_next);
+                    if constexpr (STEP_SCALES) {
+                        // The accumulators are kept in units of the current scale block's scale; when the block changes
+                        // they are converted (one multiply each), so the products themselves need no scaling.  A zero
+                        // scale counts as 1e-30: its block then contributes nothing that float32 can see.
+                        const int blk = scale_block_of(p, kk);
+                        if (blk != cur_blk && kk < p.K) {  // same for the whole wavefront; steps past the end change nothing
+                            cur_blk = blk;
+                            const float s_new = fabsf(sc) < 1e-30f ? 1e-30f : sc;
+                            const float ratio = s_cur * __builtin_amdgcn_rcpf(s_new);
+                            s_cur = s_new;
+#pragma unroll
+                            for (int mt = 0; mt < MTM; ++mt) {
+                                if (mt < n_mt) {
+#pragma unroll
+                                    for (int c = 0; c < 8; ++c) {
+                                        acc[mt][c][0] *= ratio;
+                                        acc[mt][c][1] *= ratio;
+                                        acc[mt][c][2] *= ratio;
+                                        acc[mt][c][3] *= ratio;
+                                    }
+                                }
+                            }
+                        }
+                    }
 #pragma unroll
                     for (int mt = 0; mt < MTM; ++mt) {
                         if (mt < n_mt) {
-                            if constexpr (STEP_SCALES) {
 #pragma unroll
-                                for (int c = 0; c < 8; ++c) {
-                                    const f32x4 tt = mfma_16x16x32(av[mt].v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
-                                    acc[mt][c][0] += tt[0] * sc;
-                                    acc[mt][c][1] += tt[1] * sc;
-                                    acc[mt][c][2] += tt[2] * sc;
-                                    acc[mt][c][3] += tt[3] * sc;
-                                }
-                            } else {
-#pragma unroll
-                                for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
-                            }
+                            for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
                         }
                     }
                 }
@@ -1084,7 +1099,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         float colscale[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            colscale[c] = 1.f;
+            colscale[c] = STEP_SCALES ? s_cur : 1.f;
             if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
                 const int off = (cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift)) * 4;
                 if (c == 0) colscale[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));
