@@ -30,13 +30,13 @@ def attention_algorithmic_bytes(batch, kv_heads, visible, head_dim, fp8=True):
     return 2 * batch * kv_heads * visible * per_row
 
 
-def build_model(batch, ctx, device):
+def build_model(batch, ctx, device, variant="lyra-small"):
     import torch
 
     from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights
     from lyra_amd.nn.quant import QArray
 
-    cfg = apply_inference_overrides(MODEL_VARIANTS["lyra-small"], fp8=True, fp8_attn=True, per_channel=True)
+    cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True, fp8_attn=True, per_channel=True)
     weights = init_weights(cfg, device)
     cache = init_cache(cfg, batch, ctx, device)
     g = torch.Generator(device=device)
@@ -319,6 +319,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--cpu-sample", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--model", default="lyra-small", help="model variant of the decode step (the headline figure is lyra-small)")
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -338,7 +339,7 @@ def main():
                   f"{100 * r['cold_frac_of_peak']:.1f} | {r['hot_us']:.1f} |", file=sys.stderr)
         print(json.dumps({"metric": "operator launch time at model shapes", "unit": "us", "peak_GBs": HBM_PEAK_GBS, "kernels": rows}))
         return
-    cfg, weights, cache = build_model(args.batch, args.ctx, dev)
+    cfg, weights, cache = build_model(args.batch, args.ctx, dev, args.model)
     elapsed = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
     tokens_per_s = args.batch * args.steps / elapsed
 
@@ -365,7 +366,8 @@ def main():
         "dtype": "fp8_e4m3fn weights and KV cache, bf16 activations, f32 accumulate",
         "data": "synthetic (random-init weights N(0,0.02), random KV history)",
         "config": {
-            "workload": f"full lyra-small decode step (16 layers, 16Q/4KV heads, H=128, 15+1 experts, LM head 204800), "
+            "workload": f"full {args.model} decode step ({cfg.n_layers} layers, {cfg.n_attn_heads}Q/{cfg.n_kv_heads}KV heads, "
+                        f"H={cfg.head_dim}, {cfg.n_routed_experts}+{cfg.n_shared_experts} experts, LM head {cfg.padded_vocab_size}), "
                         f"B={args.batch}, ctx {args.ctx}, FP8 KV cache, FP8 per-output-channel weights, greedy sampling",
             "batch": args.batch,
             "ctx": args.ctx,

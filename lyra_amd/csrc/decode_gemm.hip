@@ -620,7 +620,9 @@ constexpr int kSplitPitch = 132;  // floats per row of a partial tile in LDS (12
 // STEP_SCALES: 0 scales constant along K (applied to the finished tile); 1 scale blocks shorter than K, every wavefront's
 // rows within one block (its scale applied to its finished tile); 2 one scale per 32-row step.  With 1 and 2 a wavefront
 // takes DEPTH consecutive steps instead of every 4th.
-template <bool FP8, int DEPTH, int STEP_SCALES>
+// LOOP: slices longer than 4 * DEPTH steps (larger matrices, cut less finely so that one round of workgroups covers them):
+// the DEPTH register sets are refilled as they are used, wavefronts interleave, STEP_SCALES is 0 or 2.
+template <bool FP8, int DEPTH, int STEP_SCALES, bool LOOP>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
@@ -631,8 +633,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
     const int steps = (k1 - k0) >> 5;
     // steps wave, wave + 4, ... of the slice (<= DEPTH), or steps wave * DEPTH ... when scales change along K
-    const int n_my = STEP_SCALES ? max(0, min(DEPTH, steps - wave * DEPTH)) : (steps - wave + kSplitWaves - 1) / kSplitWaves;
-    auto step_row = [&](int d) { return k0 + ((STEP_SCALES ? wave * DEPTH + d : wave + kSplitWaves * d) << 5); };
+    const int n_my = (STEP_SCALES && !LOOP) ? max(0, min(DEPTH, steps - wave * DEPTH)) : (steps - wave + kSplitWaves - 1) / kSplitWaves;
+    auto step_row = [&](int d) { return k0 + (((STEP_SCALES && !LOOP) ? wave * DEPTH + d : wave + kSplitWaves * d) << 5); };
 
     const int row_bytes = p.N * ES;
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -672,15 +674,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     for (int c = 0; c < 8; ++c) colscale[c] = 1.f;
     const float* sc_lane = (FP8 && p.scale_mode == 1) ? p.scale + (ncol >> p.bn_shift) : nullptr;
     [[maybe_unused]] float step_sc[DEPTH];
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t scrsrc2 = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(FP8 ? p.scale : nullptr), 0, FP8 ? (uint32_t)p.KB * (uint32_t)p.NB * 4u : 0u, 0x00020000);
     if (FP8 && p.scale_mode == 1 && STEP_SCALES != 2) {
         const float sc = sc_lane[(size_t)(STEP_SCALES ? scale_block_of(p, step_row(0)) : 0) * p.NB];
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = sc;
     } else if (FP8 && STEP_SCALES == 2) {
-        const __amdgpu_buffer_rsrc_t scrsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(p.scale), 0, (uint32_t)p.KB * (uint32_t)p.NB * 4u, 0x00020000);
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) step_sc[d] = load_step_scale(p, scrsrc, d < n_my, (ncol >> p.bn_shift) * 4, step_row(d));
+        for (int d = 0; d < DEPTH; ++d) step_sc[d] = load_step_scale(p, scrsrc2, d < n_my, (ncol >> p.bn_shift) * 4, step_row(d));
     } else if (FP8 && p.scale_mode == 2) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = p.scale[(ncol + c) >> p.bn_shift];
@@ -694,37 +696,60 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    for (int base = 0; base < (LOOP ? n_my : 1); base += DEPTH) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-        const int kk = step_row(d);
-        Pack8 bop[8];
+        for (int d = 0; d < DEPTH; ++d) {
+            const int idx = base + d;
+            Pack8 bop[8], av[4];
 #pragma unroll
-        for (int pr = 0; pr < 4; ++pr) convert_pair<FP8>(w[d], pr, bop);
-        float sc = 1.f;
-        if constexpr (STEP_SCALES == 2) sc = step_sc[d];
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            if (mt < n_mt) {
-                Pack8 av;
+            for (int mt = 0; mt < 4; ++mt) {
                 const bool a_ok = row0 + mt * 16 + x < cnt;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) av.u[i] = a_ok ? a[d][mt][i] : 0u;
-                if constexpr (STEP_SCALES == 2) {
+                for (int i = 0; i < 4; ++i) av[mt].u[i] = a_ok ? a[d][mt][i] : 0u;
+            }
+            float sc = 1.f;
+            if constexpr (STEP_SCALES == 2) sc = step_sc[d];
+            if constexpr (LOOP) {
+                // refill this register set with the step DEPTH further on (past the end: nothing is fetched)
+                const bool more = idx + DEPTH < n_my;
+                const int kk_next = step_row(idx + DEPTH);
+                __builtin_amdgcn_sched_barrier(0);
+                const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
 #pragma unroll
-                    for (int c = 0; c < 8; ++c) {
-                        const f32x4 t = mfma_16x16x32(av.v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
-                        acc[mt][c][0] += t[0] * sc;
-                        acc[mt][c][1] += t[1] * sc;
-                        acc[mt][c][2] += t[2] * sc;
-                        acc[mt][c][3] += t[3] * sc;
+                for (int mt = 0; mt < 4; ++mt)
+                    a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff[mt] : kNoLoad, soff, 0);
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    convert_pair<FP8>(w[d], pr, bop);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_w_pair_if<FP8>(more, w[d], pr, wrsrc, wvoff, kk_next, row_bytes);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (STEP_SCALES == 2) step_sc[d] = load_step_scale(p, scrsrc2, more, (ncol >> p.bn_shift) * 4, kk_next);
+            } else {
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) convert_pair<FP8>(w[d], pr, bop);
+            }
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                if (mt < n_mt) {
+                    if constexpr (STEP_SCALES == 2) {
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) {
+                            const f32x4 t = mfma_16x16x32(av[mt].v, bop[c].v, f32x4{0.f, 0.f, 0.f, 0.f});
+                            acc[mt][c][0] += t[0] * sc;
+                            acc[mt][c][1] += t[1] * sc;
+                            acc[mt][c][2] += t[2] * sc;
+                            acc[mt][c][3] += t[3] * sc;
+                        }
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
                     }
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av.v, bop[c].v, acc[mt][c]);
                 }
             }
+            if constexpr (!LOOP) __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
     }
 
     float* mine = sm_part + wave * (64 * kSplitPitch);
@@ -1290,7 +1315,7 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
         pl.split_k = false;
         return pl;
     }
-    pl.split_k = G == 1 && weight_bytes <= 48e6 && M <= 256 && K % 128 == 0 && !no_split_k;
+    pl.split_k = G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && !no_split_k;
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
         pl.mt = 4;
@@ -1300,7 +1325,8 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
         if (bk > 0 && bk < K) unit = std::max(unit, (bk + 127) / 128 * 128);
         const long want = std::max(1L, 256L / ((long)pl.spans * pl.row_par));
         int kpart = (int)((K + want - 1) / want);
-        kpart = std::min(512, (kpart + unit - 1) / unit * unit);
+        // up to 512 rows per slice everything is requested at once; longer slices (larger matrices) refill 4 register sets
+        kpart = std::min(2048, (kpart + unit - 1) / unit * unit);
         if (unit > 512 || (bk > 0 && bk < K && kpart % bk)) pl.split_k = false;  // scale blocks that do not tile a slice
         pl.kpart = kpart;
         pl.ksplit = (K + kpart - 1) / kpart;
@@ -1337,15 +1363,24 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
 static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st) {
     const dim3 grid(pl.spans, pl.ksplit, pl.row_par), block(kSplitWaves * 64);
     const size_t lds = (size_t)kSplitWaves * 64 * kSplitPitch * sizeof(float);
-    const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4
+    const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4 steps per wavefront, or more: the looping variant
+    const bool loop = depth > 4;
     // scales that change along K: free when every wavefront's rows (32 * depth) lie within one scale block
-    const int step_scales = !(fp8 && p.scale_mode == 1 && p.bk < p.K) ? 0 : (p.bk % (32 * std::max(1, std::min(depth, 4))) == 0 ? 1 : 2);
+    const int step_scales =
+        !(fp8 && p.scale_mode == 1 && p.bk < p.K) ? 0 : ((!loop && p.bk % (32 * std::max(1, std::min(depth, 4))) == 0) ? 1 : 2);
 #define LYRA_SPLITK(F, D, S)                                                                                          \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S>,          \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S, false>,   \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S>), grid, block, lds, st, p);                            \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S, false>), grid, block, lds, st, p);                     \
+    } while (0)
+#define LYRA_SPLITK_LOOP(F, S)                                                                                        \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, (F ? 4 : 2), S, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, (F ? 4 : 2), S, true>), grid, block, lds, st, p);            \
     } while (0)
 #define LYRA_SPLITK_D(F, S)                   \
     do {                                      \
@@ -1354,11 +1389,16 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
         else if (depth == 3) LYRA_SPLITK(F, 3, S); \
         else LYRA_SPLITK(F, 4, S);            \
     } while (0)
-    if (step_scales == 1) LYRA_SPLITK_D(true, 1);
+    if (loop) {
+        if (step_scales == 2) LYRA_SPLITK_LOOP(true, 2);
+        else if (fp8) LYRA_SPLITK_LOOP(true, 0);
+        else LYRA_SPLITK_LOOP(false, 0);
+    } else if (step_scales == 1) LYRA_SPLITK_D(true, 1);
     else if (step_scales == 2) LYRA_SPLITK_D(true, 2);
     else if (fp8) LYRA_SPLITK_D(true, 0);
     else LYRA_SPLITK_D(false, 0);
 #undef LYRA_SPLITK_D
+#undef LYRA_SPLITK_LOOP
 #undef LYRA_SPLITK
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }

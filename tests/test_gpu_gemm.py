@@ -256,3 +256,17 @@ def test_few_units_are_cut_into_k_slices(kind, block, swiglu):
     for _ in range(2):
         again = _run(c, swiglu)
         assert np.array_equal(again, first), "the sum over K slices depends on arrival order or on stale counters"
+
+
+@pytest.mark.parametrize("M,K,N,kind,block,swiglu", [
+    (64, 4096, 6144, "fp8", (4096, 1), False),   # a q/k/v projection of the 4096-wide variants: slices of 896 rows
+    (40, 6144, 4096, "fp8", (6144, 1), False),   # their down projection: 8 slices of 768 rows
+    (64, 4096, 4096, "fp8", (256, 256), True),   # scale blocks along K in slices of 1024 rows
+    (16, 4096, 2048, "bf16", None, False),       # bf16 weights, two register sets refilled
+])
+def test_long_k_slices_of_larger_projections(M, K, N, kind, block, swiglu):
+    """One group with tens of MB of weights: K is cut only as far as needed for one round of workgroups, so a slice is
+    longer than what is requested up front and the register sets are refilled in a loop."""
+    c = _case(10, M, 1, K, N, [M - 1], kind=kind, block=block, bias=True, w_std=0.03)
+    _note(f"gemm long k slices M={M} K={K} N={N} kind={kind} block={block} swiglu={swiglu}")
+    U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="long k slices")
