@@ -348,8 +348,8 @@ def main():
     achieved = attn_bytes / t_attn / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "decode_attention_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
+    if os.path.exists(tpath) and (args.model, args.batch, args.ctx) == ("lyra-small", 64, 4096):
+        with open(tpath) as f:  # counters were collected for the headline launch only
             traffic = json.load(f).get("hbm_bytes_per_launch")
 
     result = {
