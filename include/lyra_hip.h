@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 5
+#define LYRA_ABI_VERSION 6
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -197,6 +197,18 @@ int lyra_moe_combine(const void* rows, const float* scores, const int32_t* dest,
 int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols, int ld,
                 lyra_stream_t stream);
 size_t lyra_argmax_workspace(int rows, int cols);
+
+/*
+ * Temperature / top-k sampling (lyra/generate.py:46-53 with temperature > 0): per row, the k largest of
+ * x[r, 0:cols] / temperature (ties go to the lower index, as lax.top_k), softmax over them, and the inverse CDF at
+ * uniforms[r] in [0, 1) taken in that order: out[r] = index of the drawn column.  The reference draws with
+ * jax.random.categorical from its own key stream; the distribution is the same, the caller supplies the randomness.
+ * 1 <= k <= 8; x float32 [rows, ld], ld % 4 == 0, 16-byte aligned; workspace as for lyra_argmax (zero on first use).
+ */
+int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
+                     int cols, int ld, int k, float temperature, lyra_stream_t stream);
+size_t lyra_sample_topk_workspace(int rows, int cols, int k);
+
 
 /*
  * Self-check of the matrix-core register layouts and FP8 conversions the kernels rely on.

@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _c = ctypes
 SIGNATURES = {
@@ -52,6 +52,8 @@ SIGNATURES = {
     ),
     "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p]),
     "lyra_argmax_workspace": (_c.c_size_t, [_c.c_int] * 2),
+    "lyra_sample_topk": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p]),
+    "lyra_sample_topk_workspace": (_c.c_size_t, [_c.c_int] * 3),
     "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
 }
 

@@ -432,6 +432,164 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
     if (threadIdx.x == 0) p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
 }
 
+// ---- temperature / top-k sampling ---------------------------------------------------------------------------------
+// lyra/generate.py:46-53 with temperature > 0: logits / temperature, keep the k largest (lax.top_k: ties go to the lower
+// index), draw from their softmax.  The draw is the inverse CDF at a uniform number the caller supplies per row (the
+// reference draws with jax.random.categorical from its own key stream; the distribution is the same).
+// Grid (chunks, rows) as for the argmax: every workgroup reduces its chunk to its k best (value, index) pairs, the
+// workgroup that arrives last for the row merges the chunks' candidates, forms the softmax and picks the token.
+constexpr int kMaxSampleK = 8;
+
+struct SampleParams {
+    const float* x;
+    const float* uniforms;  // [rows] in [0, 1)
+    int32_t* out;
+    float* part_v;   // [rows, chunks, k]
+    int* part_i;     // [rows, chunks, k]
+    int* arrivals;   // [rows] zero on entry, zero again on exit
+    int rows, cols, ld, chunks, chunk_len, k;
+    float temperature;
+};
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+// Keeps the k best pairs seen so far in (tv, ti), best first.
+__device__ __forceinline__ void topk_insert(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], int k, float v, int i) {
+    if (!better(v, i, tv[k - 1], ti[k - 1])) return;
+#pragma unroll
+    for (int j = kMaxSampleK - 1; j >= 0; --j) {
+        if (j >= k) continue;
+        const bool here = better(v, i, tv[j], ti[j]);
+        const bool above = j > 0 && better(v, i, tv[j > 0 ? j - 1 : 0], ti[j > 0 ? j - 1 : 0]);
+        if (here && above) {  // the pair goes further up: move the entry above down into this slot
+            tv[j] = tv[j - 1];
+            ti[j] = ti[j - 1];
+        } else if (here) {
+            tv[j] = v;
+            ti[j] = i;
+        }
+    }
+}
+
+// The k best pairs over all threads of a workgroup of `nthreads` (64 or 256) threads, each holding its own k best,
+// best first: k rounds of "best head wins, its owner moves on".  Result in sm_tv / sm_ti (valid after the call).
+__device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], int k, int nthreads, float* sm_wv,
+                                           int* sm_wi, float* sm_tv, int* sm_ti) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = nthreads >> 6;
+    int head = 0;
+    for (int r = 0; r < k; ++r) {
+        float hv = -INFINITY;
+        int hi = 0x7FFFFFFF;
+#pragma unroll
+        for (int j = 0; j < kMaxSampleK; ++j)
+            if (j == head && j < k) {
+                hv = tv[j];
+                hi = ti[j];
+            }
+        float bv = hv;
+        int bi = hi;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, kWave);
+            const int oi = __shfl_xor(bi, o, kWave);
+            if (better(ov, oi, bv, bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (lane == 0) {
+            sm_wv[wave] = bv;
+            sm_wi[wave] = bi;
+        }
+        __syncthreads();
+        for (int w = 0; w < waves; ++w)
+            if (better(sm_wv[w], sm_wi[w], bv, bi)) {
+                bv = sm_wv[w];
+                bi = sm_wi[w];
+            }
+        if (hi == bi && bi != 0x7FFFFFFF) ++head;  // indices are unique: exactly one thread owns the winner
+        if (threadIdx.x == 0) {
+            sm_tv[r] = bv;
+            sm_ti[r] = bi;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
+    __shared__ float sm_wv[4], sm_tv[kMaxSampleK];
+    __shared__ int sm_wi[4], sm_ti[kMaxSampleK];
+    __shared__ int sm_last;
+    const int c = blockIdx.x, row = blockIdx.y, k = p.k;
+    const float* xr = p.x + (size_t)row * p.ld;
+    const int lo = c * p.chunk_len, hi = min(lo + p.chunk_len, p.cols);
+    float tv[kMaxSampleK];
+    int ti[kMaxSampleK];
+#pragma unroll
+    for (int j = 0; j < kMaxSampleK; ++j) {
+        tv[j] = -INFINITY;
+        ti[j] = 0x7FFFFFFF;
+    }
+    for (int i = lo + threadIdx.x * 4; i < hi; i += 1024) {  // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads
+        if (i + 4 <= hi) {
+            const f32x4 v = *(const f32x4*)(xr + i);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) topk_insert(tv, ti, k, v[q], i + q);
+        } else {
+            for (int q = 0; i + q < hi; ++q) topk_insert(tv, ti, k, xr[i + q], i + q);
+        }
+    }
+    topk_merge(tv, ti, k, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    if (threadIdx.x < k) {
+        store_agent(&p.part_v[((size_t)row * p.chunks + c) * k + threadIdx.x], sm_tv[threadIdx.x]);
+        store_agent(&p.part_i[((size_t)row * p.chunks + c) * k + threadIdx.x], sm_ti[threadIdx.x]);
+    }
+    wait_all_memory();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int seen = add_agent(&p.arrivals[row], 1);
+        sm_last = seen == p.chunks - 1;
+        if (sm_last) store_agent(&p.arrivals[row], 0);
+    }
+    __syncthreads();
+    if (!sm_last) return;
+    // merge the candidates of all chunks (every thread takes some, then the same k rounds)
+#pragma unroll
+    for (int j = 0; j < kMaxSampleK; ++j) {
+        tv[j] = -INFINITY;
+        ti[j] = 0x7FFFFFFF;
+    }
+    for (int q = threadIdx.x; q < p.chunks * k; q += 256) {
+        const float v = load_agent(&p.part_v[(size_t)row * p.chunks * k + q]);
+        const int i = __hip_atomic_load(&p.part_i[(size_t)row * p.chunks * k + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (i != 0x7FFFFFFF) topk_insert(tv, ti, k, v, i);
+    }
+    topk_merge(tv, ti, k, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    if (threadIdx.x == 0) {
+        // softmax of logits / temperature over the candidates (best first), inverse CDF at the row's uniform number
+        float e[kMaxSampleK], total = 0.f;
+        const float top = sm_tv[0] / p.temperature;
+        int n = 0;
+        for (int j = 0; j < k; ++j) {
+            if (sm_ti[j] == 0x7FFFFFFF) break;
+            e[j] = expf(sm_tv[j] / p.temperature - top);
+            total += e[j];
+            n = j + 1;
+        }
+        const float target = p.uniforms[row] * total;
+        float run = 0.f;
+        int pick = n > 0 ? sm_ti[n - 1] : 0;
+        for (int j = 0; j < n; ++j) {
+            run += e[j];
+            if (target < run) {
+                pick = sm_ti[j];
+                break;
+            }
+        }
+        p.out[row] = pick;
+    }
+}
+
 }  // namespace lyra
 
 extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
@@ -548,5 +706,36 @@ extern "C" int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t
     p.part_v = (float*)((char*)workspace + counters);
     p.part_i = (int*)(p.part_v + (size_t)rows * argmax_chunks(rows, cols));
     hipLaunchKernelGGL(argmax_kernel, dim3(p.chunks, rows), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" size_t lyra_sample_topk_workspace(int rows, int cols, int k) {
+    if (rows <= 0 || cols <= 0 || k <= 0) return 0;
+    return lyra::kArgmaxCounterBytes + ((size_t)rows * lyra::argmax_chunks(rows, cols) * k * 8 + 255) / 256 * 256;
+}
+
+extern "C" int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
+                                int cols, int ld, int k, float temperature, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!x || !uniforms || !out || rows <= 0 || cols <= 0 || ld < cols || k <= 0 || !(temperature > 0.f)) return LYRA_E_BADARG;
+    if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535 || k > kMaxSampleK) return LYRA_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < lyra_sample_topk_workspace(rows, cols, k) || ((uintptr_t)workspace % 256))
+        return LYRA_E_WORKSPACE;
+    SampleParams p;
+    p.x = x;
+    p.uniforms = uniforms;
+    p.out = out;
+    p.rows = rows;
+    p.cols = cols;
+    p.ld = ld;
+    p.k = std::min(k, cols);
+    p.temperature = temperature;
+    p.chunks = argmax_chunks(rows, cols);
+    p.chunk_len = ((cols + p.chunks - 1) / p.chunks + 3) / 4 * 4;
+    p.chunks = (cols + p.chunk_len - 1) / p.chunk_len;
+    p.arrivals = (int*)workspace;
+    p.part_v = (float*)((char*)workspace + kArgmaxCounterBytes);
+    p.part_i = (int*)(p.part_v + (size_t)rows * argmax_chunks(rows, cols) * k);
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(p.chunks, rows), dim3(256), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }

@@ -17,6 +17,13 @@ def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Genera
 
             return argmax(logits, min(cfg.vocab_size, logits.shape[-1]))
         return torch.argmax(logits, dim=-1).to(torch.int32)
+    if (logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla"
+            and 0 < cfg.sample_topk <= 8):
+        # the draw is the inverse CDF over the k candidates at one uniform number per row
+        from lyra_amd.kernels.decode_fused import sample_topk
+
+        u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=generator)
+        return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]))
     logits = logits.to(torch.float32) / cfg.sample_temperature
     if 0 < cfg.sample_topk < logits.shape[-1]:
         top = torch.topk(logits, cfg.sample_topk, dim=-1)
@@ -40,8 +47,11 @@ class GraphedDecoder:
     replayed.  Token ids are read from / written to fixed device buffers.
     """
 
-    def __init__(self, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, batch: int, warmup: int = 2):
-        self.cfg, self.model, self.cache = cfg, model, cache
+    def __init__(self, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, batch: int, warmup: int = 2,
+                 greedy: bool = True):
+        # greedy=False: temperature / top-k sampling as configured, the uniform numbers drawn inside the graph from the
+        # device's default generator (its state advances with every replay)
+        self.cfg, self.model, self.cache, self.greedy = cfg, model, cache, greedy
         dev = model.emb.device
         self.tokens = torch.zeros(batch, dtype=torch.int64, device=dev)
         self.next_tokens = torch.zeros(batch, dtype=torch.int32, device=dev)
@@ -62,9 +72,9 @@ class GraphedDecoder:
     def _step(self):
         logits, _ = model_apply(self.tokens, self.model, self.cache, self.cfg)
         self.logits = logits
-        self.next_tokens.copy_(sample_token(logits, replace(self.cfg, sample_temperature=0.0)))
+        self.next_tokens.copy_(sample_token(logits, replace(self.cfg, sample_temperature=0.0) if self.greedy else self.cfg))
 
     def step(self) -> torch.Tensor:
-        """Run one decode step on ``self.tokens``; returns the greedy next tokens (device, int32)."""
+        """Run one decode step on ``self.tokens``; returns the next tokens (device, int32): greedy, or sampled."""
         self.graph.replay()
         return self.next_tokens

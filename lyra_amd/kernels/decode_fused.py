@@ -224,3 +224,20 @@ def argmax(logits: torch.Tensor, cols: int | None = None) -> torch.Tensor:
     rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, stream)
     _lib.check(rc, "lyra_argmax")
     return out
+
+
+def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperature: float, cols: int | None = None) -> torch.Tensor:
+    """Temperature / top-k token choice (lyra/generate.py:46-53 at temperature > 0) for every row of float32 ``logits``
+    [rows, ld] over its first ``cols`` columns: softmax of the k largest ``logits / temperature`` (ties to the lower
+    index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows]."""
+    rows, ld = logits.shape
+    cols = ld if cols is None else cols
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    assert uniforms.dtype == torch.float32 and uniforms.shape == (rows,) and uniforms.is_contiguous()
+    out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    stream = _stream(logits.device)
+    ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_sample_topk_workspace(rows, cols, k))
+    rc = _L.lyra_sample_topk(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,
+                             float(temperature), stream)
+    _lib.check(rc, "lyra_sample_topk")
+    return out

@@ -27,6 +27,11 @@ formulas; the checks live in tests/test_oracle_*.py):
 * SwiGLU ........................... scalar closed forms
 * routing / bpermute ............... stable argsort + bincount; the input
                                      vector of reference tests/test_combine.py:13
+* sample_topk ....................... closed forms: k = 1 is the argmax, u -> 0 / u -> 1 pick the first / k-th
+                                     candidate, ties to the lower index, frequencies over a grid of u against
+                                     ``torch.softmax`` of the k largest logits / temperature
+* ``jax.random.categorical``'s key stream (lyra/generate.py:53): PARITY UNPINNED - the draw is restated as the
+  inverse CDF at a caller-supplied uniform number (same distribution, different randomness)
 * exact XLA bf16 rounding points and summation order inside einsum:
   PARITY UNPINNED (needs the reference runtime, which cannot be imported
   here); irrelevant to acceptance because tolerances are against fp32.
@@ -518,3 +523,29 @@ def combine(rows: np.ndarray, scores: np.ndarray, unpermute_map: np.ndarray) -> 
     F, k = scores.shape
     t = np.asarray(rows, dtype=np.float32)[unpermute_map].reshape(F, k, -1)
     return np.einsum("fkc,fk->fc", t, np.asarray(scores, dtype=np.float32), dtype=np.float32)
+
+
+def sample_topk(logits: np.ndarray, uniforms: np.ndarray, k: int, temperature: float) -> np.ndarray:
+    """lyra/generate.py:46-53 with temperature > 0, one row of ``logits`` [rows, V] per draw: logits / temperature,
+    keep the k largest (lax.top_k: descending, ties to the lower index), categorical draw over their softmax.
+
+    The reference draws with jax.random.categorical from its key stream; that stream cannot be reproduced here, so the
+    draw is restated as the inverse CDF at ``uniforms`` [rows] in [0, 1), taken over the candidates in top_k order: the
+    same distribution, a different (caller-supplied) source of randomness.  Returns int32 [rows].
+    """
+    x = np.asarray(logits, dtype=np.float32) / np.float32(temperature)
+    rows, V = x.shape
+    k = min(int(k), V)
+    out = np.zeros(rows, np.int32)
+    for r in range(rows):
+        order = np.lexsort((np.arange(V), -x[r]))[:k]  # value descending, then index ascending
+        e = np.exp(x[r, order] - x[r, order[0]], dtype=np.float32)
+        target = np.float32(uniforms[r]) * np.float32(e.sum(dtype=np.float32))
+        run, pick = np.float32(0.0), order[-1]
+        for j in range(k):
+            run = np.float32(run + e[j])
+            if target < run:
+                pick = order[j]
+                break
+        out[r] = pick
+    return out

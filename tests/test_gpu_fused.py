@@ -315,3 +315,59 @@ def test_unsummed_projection_consumers_equal_summed_path(fp8, B, C, N, K, H):
     x2 = F.gemm(t, w_out, one, residual=x, out_scale=0.1767766952966369)
     h2, y2 = F.rmsnorm_proj(x2, scale, 1e-5, router, None)
     assert torch.equal(x1, x2) and torch.equal(h1, h2) and torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("rows,cols,ld,k,temperature", [(64, 201088, 204800, 4, 0.8), (3, 1000, 1024, 8, 1.5), (130, 5000, 5000, 1, 0.3),
+                                                        (1, 201088, 204800, 4, 0.8), (5, 7, 8, 4, 1.0)])
+def test_sample_topk_matches_oracle(rows, cols, ld, k, temperature):
+    """lyra/generate.py:46-53 with temperature > 0: the drawn column must be the oracle's for the same uniform numbers
+    (rows whose uniform number lies within 1e-5 of a CDF boundary are not compared: expf differs in the last bit).  Ties
+    between logits are planted, the padding beyond `cols` holds larger values that must be ignored, and the call is
+    repeated on the same workspace."""
+    from lyra_amd.kernels import decode_fused as F
+
+    rng = np.random.default_rng(rows * 7 + k)
+    x = rng.standard_normal((rows, ld)).astype(np.float32)
+    x[:, cols:] = 50.0
+    if cols > 40:
+        x[0, 11] = x[0, 37] = 9.0  # a tie for first place: index 11 first
+    u = rng.random(rows).astype(np.float32)
+    u[0] = 0.0
+    xt, ut = torch.from_numpy(x).to(U.dev()), torch.from_numpy(u).to(U.dev())
+    want = O.sample_topk(x[:, :cols], u, k, temperature)
+    kk = min(k, cols)
+    order = np.argsort(-x[:, :cols], axis=1, kind="stable")[:, :kk]
+    top = np.take_along_axis(x[:, :cols], order, 1) / np.float32(temperature)
+    cdf = np.cumsum(np.exp(top - top[:, :1]), axis=1)
+    cdf = cdf / cdf[:, -1:]
+    safe = np.abs(cdf - u[:, None]).min(axis=1) > 1e-5
+    assert safe.mean() > 0.9
+    for _ in range(2):
+        got = U.to_np(F.sample_topk(xt, ut, k, temperature, cols))
+        assert (got < cols).all() and (got >= 0).all()
+        assert (got[safe] == want[safe]).all(), np.flatnonzero(got != want)
+    if cols > 40:
+        assert got[0] == 11
+
+
+def test_sample_token_draws_from_the_topk_softmax():
+    """sample_token on the device path: over many draws the tokens of one row are distributed as the softmax of its 4
+    largest logits / temperature, and nothing outside the top 4 is ever drawn."""
+    from dataclasses import replace
+
+    from lyra_amd.generate import sample_token
+    from lyra_amd.model import MODEL_VARIANTS
+
+    cfg = replace(MODEL_VARIANTS["dev"], sample_topk=4, sample_temperature=0.8, implementation="pallas")
+    rng = np.random.default_rng(3)
+    row = rng.standard_normal(cfg.padded_vocab_size).astype(np.float32)
+    row[cfg.vocab_size:] = -np.inf
+    logits = torch.from_numpy(np.repeat(row[None], 4096, 0)).to(U.dev())
+    gen = torch.Generator(device=U.dev())
+    gen.manual_seed(11)
+    picks = np.concatenate([U.to_np(sample_token(logits, cfg, gen)) for _ in range(8)])
+    top = np.argsort(-row[: cfg.vocab_size], kind="stable")[:4]
+    assert set(picks.tolist()) <= set(top.tolist())
+    want = torch.softmax(torch.from_numpy(row[top] / np.float32(0.8)), 0).numpy()
+    got = np.array([(picks == t).mean() for t in top])
+    np.testing.assert_allclose(got, want, atol=0.015)  # 32768 draws: ~4 standard errors

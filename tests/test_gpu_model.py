@@ -163,3 +163,28 @@ def test_lyra_small_full_width_decode_steps_match_oracle():
         assert err.mean() < 0.03
         assert (g[clear].argmax(-1) == t[clear].argmax(-1)).mean() >= 0.5  # greedy tokens mostly agree (near-ties aside)
     assert int(cache.pos.item()) == start + steps
+
+
+def test_graphed_decoder_samples_inside_the_graph():
+    """Temperature / top-k sampling recorded into the HIP graph: every replay draws fresh uniform numbers, every drawn
+    token is one of the row's 4 largest logits, and replays on identical inputs do not all draw the same tokens."""
+    from lyra_amd.generate import GraphedDecoder
+    from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights
+
+    cfg = apply_inference_overrides(replace(MODEL_VARIANTS["dev"], implementation="pallas", sample_topk=4, sample_temperature=0.8),
+                                    fp8=True, fp8_attn=True, per_channel=True)
+    dev = U.dev()
+    w = init_weights(cfg, dev, seed=3)
+    cache = init_cache(cfg, 8, 256, dev)
+    cache.pos.fill_(9)
+    dec = GraphedDecoder(w, cache, cfg, batch=8, greedy=False)
+    dec.tokens.copy_(torch.arange(8, device=dev) + 3)
+    draws = []
+    for _ in range(12):
+        cache.pos.fill_(9)
+        nxt = dec.step()
+        torch.cuda.synchronize()
+        top4 = torch.topk(dec.logits[:, : cfg.vocab_size], 4, dim=-1).indices
+        assert (nxt.long()[:, None] == top4).any(-1).all()
+        draws.append(U.to_np(nxt).copy())
+    assert len({d.tobytes() for d in draws}) > 1

@@ -173,3 +173,26 @@ def test_rms_norm_and_rotate_against_torch():
     z = (x[0, :32] + 1j * x[0, 32:]) * np.exp(1j * np.arange(5, 6) * (1.0 / 150000.0 ** (np.arange(0, 64, 2) / 64)))
     np.testing.assert_allclose(r[0, :32], z.real, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(r[0, 32:], z.imag, rtol=1e-4, atol=1e-5)
+
+
+def test_sample_topk_closed_forms():
+    """lyra/generate.py:46-53 restated with a caller-supplied uniform number: k = 1 is the argmax whatever the number;
+    u -> 0 picks the largest logit, u -> 1 the k-th largest; ties go to the lower index; and over a fine grid of uniform
+    numbers the picks are distributed as the softmax of the k largest logits / temperature."""
+    rng = np.random.default_rng(4)
+    logits = rng.standard_normal((6, 50)).astype(np.float32)
+    logits[2, 7] = logits[2, 30] = logits[2].max() + 1.0  # a tie for first place
+    u = rng.random(6).astype(np.float32)
+    assert (O.sample_topk(logits, u, 1, 0.7) == np.array([np.flatnonzero(r == r.max())[0] for r in logits])).all()
+    order = np.argsort(-logits, axis=1, kind="stable")
+    assert (O.sample_topk(logits, np.zeros(6, np.float32), 4, 0.8) == order[:, 0]).all()
+    assert (O.sample_topk(logits, np.full(6, 0.999999, np.float32), 4, 0.8) == order[:, 3]).all()
+    assert O.sample_topk(logits[2:3], np.zeros(1, np.float32), 4, 0.8)[0] == 7  # the lower index of the tied pair
+    row = logits[:1]
+    grid = ((np.arange(20000) + 0.5) / 20000).astype(np.float32)
+    picks = O.sample_topk(np.repeat(row, grid.size, 0), grid, 4, 0.8)
+    top = order[0, :4]
+    want = torch.softmax(torch.from_numpy(row[0, top] / np.float32(0.8)), 0).numpy()
+    got = np.array([(picks == t).mean() for t in top])
+    assert set(picks.tolist()) <= set(top.tolist())
+    np.testing.assert_allclose(got, want, atol=2e-4)
