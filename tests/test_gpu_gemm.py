@@ -270,3 +270,16 @@ def test_long_k_slices_of_larger_projections(M, K, N, kind, block, swiglu):
     c = _case(10, M, 1, K, N, [M - 1], kind=kind, block=block, bias=True, w_std=0.03)
     _note(f"gemm long k slices M={M} K={K} N={N} kind={kind} block={block} swiglu={swiglu}")
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="long k slices")
+
+
+@pytest.mark.parametrize("block,swiglu", [((256, 256), True), ((128, 128), False), ((512, 256), False), ((64, 128), True)])
+def test_many_experts_with_scale_blocks_along_k(block, swiglu):
+    """Scale blocks shorter than K in the unit-list kernel: the accumulators are re-expressed whenever a wavefront's next
+    step lies in another block (every 1, 2 or 4 steps depending on block height and on how the wavefronts interleave)."""
+    G, M, K, N = 40, 300, 1024, 512
+    rng = np.random.default_rng(17)
+    sizes = rng.multinomial(M - 70, np.ones(G - 1) / (G - 1)).astype(np.int32)
+    sizes = np.concatenate([sizes, [70]]).astype(np.int32)
+    c = _case(12, M, G, K, N, sizes, kind="fp8", block=block, bias=True, w_std=0.05)
+    _note(f"gemm unit list with k scale blocks block={block} swiglu={swiglu}")
+    U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list, k scale blocks")
