@@ -283,3 +283,23 @@ def test_many_experts_with_scale_blocks_along_k(block, swiglu):
     c = _case(12, M, G, K, N, sizes, kind="fp8", block=block, bias=True, w_std=0.05)
     _note(f"gemm unit list with k scale blocks block={block} swiglu={swiglu}")
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list, k scale blocks")
+
+
+@pytest.mark.parametrize("G,M", [(1, 20), (6, 20)])
+def test_zero_and_extreme_block_scales(G, M):
+    """Scales a quantiser never produces but a caller may pass: exactly zero (the block must contribute nothing), and
+    neighbouring blocks 1e8 apart.  K-split (one group) and unit-list (several groups) kernels."""
+    K, N = 1024, 256
+    sizes = [M] if G == 1 else [3, 0, 7, 2, 5, 3]
+    c = _case(21, M, G, K, N, sizes, kind="fp8", block=(256, 128), bias=True, w_std=0.05)
+    q, s = c["w"]
+    s = s.copy()
+    s[:, 1, :] = 0.0          # second K block of every expert: zero scale
+    s[:, 2, 0] *= 1e4         # third block, first column block: large
+    s[:, 3, 0] *= 1e-4        # fourth: tiny
+    c["w"] = (q, s)
+    _note(f"gemm zero / extreme scales G={G}")
+    want = _want(c, False, big=True)
+    got = _run(c, False)
+    assert np.isfinite(got).all()
+    U.assert_close(got, want, atol=2e-2 * max(1.0, float(np.abs(want).max()) / 50), what="zero / extreme scales")
