@@ -1321,7 +1321,9 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
         pl.mt = 4;
         pl.row_par = (M + 63) / 64;
         pl.spans = (N + 127) / 128;
-        int unit = 128;
+        // slices of at least 256 rows: 128-row slices fill more compute units but double the float32 slices the consumer
+        // has to sum (2048 x 2048 out projection: 16 -> 8 slices shortened the decode step by 1.2 %)
+        int unit = (K % 256 == 0 && K >= 512) ? 256 : 128;
         if (bk > 0 && bk < K) unit = std::max(unit, (bk + 127) / 128 * 128);
         const long want = std::max(1L, 256L / ((long)pl.spans * pl.row_par));
         int kpart = (int)((K + want - 1) / want);
