@@ -59,7 +59,7 @@ def test_small_shapes_match_oracle(fp8, H, N, K, sw):
 
 
 def test_config1_lyra_small_bf16_global_with_gate():
-    """BASELINE config 1 at the variants.py shape (16Q/4KV/H=128) and at its literal 32Q/4KV/H=64."""
+    """Benchmark configuration 1 (single-sequence attention) at the variants.py shape (16Q/4KV/H=128) and at its literal 32Q/4KV/H=64."""
     for (N, K, H) in ((16, 4, 128), (32, 4, 64)):
         case = U.attention_case(1001, 1, N, K, 512, H, fp8=False)
         rng = np.random.default_rng(7)
@@ -168,7 +168,7 @@ def test_split_count_does_not_change_the_result():
 
 
 def test_config4_gpt_oss_shape_ragged_fp8_full_size():
-    """BASELINE config 4: B=64, 64Q/8KV, H=64, S=4096, L_b ~ U{256..4096}, FP8 cache; global and window 128."""
+    """Benchmark configuration 4 (gpt-oss attention shape, ragged batch): B=64, 64Q/8KV, H=64, S=4096, L_b ~ U{256..4096}, FP8 cache; global and window 128."""
     B, N, K, S, H = 64, 64, 8, 4096, 64
     case = U.attention_case(1004, B, N, K, S, H, fp8=True)
     rng = np.random.default_rng(1004)

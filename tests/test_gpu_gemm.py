@@ -135,7 +135,7 @@ def _zipf_routing(rng, T, n_routed, k, n_shared):
 
 @pytest.mark.parametrize("T", [1, 16, 64])
 def test_config3_moe_medium_shape_zipf_routing(T):
-    """BASELINE config 3: width 4096, 31 routed + 1 shared expert, FP8 per-channel scales, top-(3+1) Zipf(1.1)."""
+    """Benchmark configuration 3 (MoE matmul at lyra-medium widths): width 4096, 31 routed + 1 shared expert, FP8 per-channel scales, top-(3+1) Zipf(1.1)."""
     C, Hd, E = 4096, 4096, 32
     rng = np.random.default_rng(1003 + T)
     sizes = _zipf_routing(rng, T, 31, 3, 1)
