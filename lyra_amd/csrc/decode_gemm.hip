@@ -15,6 +15,7 @@
 //   D[16 rows, 16 cols] += X[16 rows x 32 k] . W[32 k x 16 cols]   for each of the 8 column phases.
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "lyra_device.h"
 
@@ -74,7 +75,7 @@ __device__ __forceinline__ float residual_epilogue(const GemmParams& p, float t,
 __device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, float limit) {
     glu = fminf(glu, limit);
     lin = fminf(fmaxf(lin, -limit), limit);
-    const float sig = 1.0f / (1.0f + fast_exp2(-beta * kLog2e * glu));
+    const float sig = __builtin_amdgcn_rcpf(1.0f + fast_exp2(-beta * kLog2e * glu));  // (1 ulp; the division sequence is 10 instructions)
     return (lin + 1.0f) * (glu * sig);
 }
 
@@ -1235,29 +1236,42 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             const f32x4 bias_v = load_f32x4(bias_rsrc, p.bias ? (cur_g * p.N + oc) * 4 : kNoLoad);
             const f32x4 bias_l = load_f32x4(bias_rsrc, (p.bias && wide) ? (cur_g * p.N + oc2) * 4 : kNoLoad);
             const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
-            for (int r = threadIdx.x >> 5; r < cur_rows; r += 16) {
-                const int rb = min(r + 8, 16 * MTM - 1);  // second row of the pair (clamped: read, not written, when past the end)
-                const bool two = r + 8 < cur_rows;
-                float ag[4], al[4], bg[4], bl[4];
-                tile_row(r, ag, al);
-                tile_row(rb, bg, bl);
-                const size_t oa = (size_t)(cur_row0 + r) * NO + oc, ob = (size_t)(cur_row0 + rb) * NO + oc;
-                f32x4 ra = load_bf16x4(res_rsrc, p.residual ? (int)(oa * 2) : kNoLoad);
-                f32x4 rb4 = load_bf16x4(res_rsrc, (p.residual && two) ? (int)(ob * 2) : kNoLoad);
-                if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
-                    const f32x4 ra2 = load_bf16x4(res_rsrc, p.residual ? (int)((oa + 128) * 2) : kNoLoad);
-                    const f32x4 rb2 = load_bf16x4(res_rsrc, (p.residual && two) ? (int)((ob + 128) * 2) : kNoLoad);
-                    finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
-                    finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
-                    if (two) {
-                        finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
-                        finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
+            // Two copies of the row loop: without a residual there is no load in it, so nothing in it waits for memory -
+            // a load in the loop makes every pass wait for the stores of the pass before (stores and loads share the
+            // counter the compiler waits on), which cost ~1 us per pass.
+            auto run_rows = [&](auto with_residual) {
+                constexpr bool kRes = decltype(with_residual)::value;
+                for (int r = threadIdx.x >> 5; r < cur_rows; r += 16) {
+                    const int rb = min(r + 8, 16 * MTM - 1);  // second row of the pair (clamped: read, not written, when past the end)
+                    const bool two = r + 8 < cur_rows;
+                    float ag[4], al[4], bg[4], bl[4];
+                    tile_row(r, ag, al);
+                    tile_row(rb, bg, bl);
+                    const size_t oa = (size_t)(cur_row0 + r) * NO + oc, ob = (size_t)(cur_row0 + rb) * NO + oc;
+                    f32x4 ra = zero4, rb4 = zero4, ra2 = zero4, rb2 = zero4;
+                    if constexpr (kRes) {
+                        ra = load_bf16x4(res_rsrc, (int)(oa * 2));
+                        rb4 = load_bf16x4(res_rsrc, two ? (int)(ob * 2) : kNoLoad);
+                        if (wide && !p.swiglu) {
+                            ra2 = load_bf16x4(res_rsrc, (int)((oa + 128) * 2));
+                            rb2 = load_bf16x4(res_rsrc, two ? (int)((ob + 128) * 2) : kNoLoad);
+                        }
                     }
-                } else {
-                    finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, oa);
-                    if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, ob);
+                    if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
+                        finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
+                        finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
+                        if (two) {
+                            finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
+                            finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
+                        }
+                    } else {
+                        finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, oa);
+                        if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, ob);
+                    }
                 }
-            }
+            };
+            if (p.residual) run_rows(std::true_type{});
+            else run_rows(std::false_type{});
         }
         __syncthreads();  // the tiles are free for the next unit
     }
