@@ -346,6 +346,9 @@ void decode_attention_kernel(AttnParams p) {
     const u32x4 q_raw = __builtin_amdgcn_raw_buffer_load_b128(qrsrc, (q_row * H + q_piece * 8) * 2, 0, 0);
     const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(p.sinks + kh * G, (uint32_t)(G * 4));
     const float sink_raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(srsrc, x * 4, 0, 0));
+    // ... and the output gates of these heads (an absent gate reads as zeros and is replaced by 1 below)
+    const __amdgpu_buffer_rsrc_t grsrc = make_rsrc(p.gate ? p.gate + (size_t)b * p.N + kh * G : nullptr, p.gate ? (uint32_t)(G * 2) : 0u);
+    const uint16_t gate_raw = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(grsrc, x * 2, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 
     // First tile of this wavefront: requested next.  Without a sliding window the chunk starts at a
@@ -449,6 +452,12 @@ void decode_attention_kernel(AttnParams p) {
     float* sm_o = smem;                             // [waves][G][HP]
     float* sm_m = smem + WAVES * G * HP;            // [waves][16]
     float* sm_l = sm_m + WAVES * 16;                // [waves][16]
+    float* sm_sink = sm_l + WAVES * 16;             // [16] sink logit (base 2) and output gate of every head: the final
+    float* sm_gate = sm_sink + 16;                  // [16] loop below then reads no global memory between its stores
+    if (wave == 0 && kb == 0 && x < G) {
+        sm_sink[x] = sink2;
+        sm_gate[x] = p.gate ? bf16_bits_to_f32(gate_raw) : 1.f;
+    }
     if (x < G) {
         float* dst = sm_o + ((size_t)wave * G + x) * HP;
 #pragma unroll
@@ -477,10 +486,8 @@ void decode_attention_kernel(AttnParams p) {
         }
         const int n = kh * G + g;
         if (final_out) {
-            const float sk = p.sinks[n] * kLog2e;
-            const float den = l + fast_exp2(sk - mm);  // mm >= sink by construction
-            const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
-            store_out(p, ((size_t)b * p.N + n) * H + col, o / den, gate);
+            const float den = l + fast_exp2(sm_sink[g] - mm);  // mm >= sink by construction
+            store_out(p, ((size_t)b * p.N + n) * H + col, o / den, sm_gate[g]);
         } else {
             const size_t item = ((size_t)b * p.K + kh) * p.n_chunks + c_idx;
             store_agent(p.part_o + (item * G + g) * H + col, o);
@@ -695,7 +702,7 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
 
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(pl.n_chunks, K, B), block(pl.waves * 64);
-    const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16) * sizeof(float);
+    const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16 + 32) * sizeof(float);
     const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
     const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
     const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
