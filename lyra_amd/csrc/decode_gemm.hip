@@ -1015,17 +1015,6 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         }
     };
 
-    // Bias / SwiGLU / residual and the store of 4 (wide: 4 + 4) finished columns of one output row.
-    auto finish_row = [&](int fg, int frow, int fspan, float (&vg)[4], float (&vl)[4]) {
-        const int oc = fspan * span_cols + 4 * q;
-        if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
-            float zero[4] = {0.f, 0.f, 0.f, 0.f};
-            group_epilogue(p, vg, zero, fg, frow, oc, NO);
-            group_epilogue(p, vl, zero, fg, frow, oc + 128, NO);
-        } else {
-            group_epilogue(p, vg, vl, fg, frow, oc, NO);
-        }
-    };
     // bias [G, N] float32 and residual [M, NO] bf16 through descriptors, so that an absent operand reads as zeros
     const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(p.bias), 0, p.bias ? (uint32_t)p.G * (uint32_t)p.N * 4u : 0u, 0x00020000);
