@@ -8,29 +8,37 @@ import torch
 from lyra_amd.model import ModelCache, ModelConfig, ModelWeights, model_apply
 
 
-def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Generator | None = None) -> torch.Tensor:
+def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Generator | None = None,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
     """lyra/generate.py:46-53 applied to each row of ``logits`` [B, V]: greedy when temperature <= 0, else
     temperature scaling, top-k masking (lowest index wins ties, like lax.top_k) and a categorical draw."""
     if cfg.sample_temperature <= 0:
         if logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla":
             from lyra_amd.kernels.decode_fused import argmax
 
-            return argmax(logits, min(cfg.vocab_size, logits.shape[-1]))
-        return torch.argmax(logits, dim=-1).to(torch.int32)
+            return argmax(logits, min(cfg.vocab_size, logits.shape[-1]), out)
+        return _into(out, torch.argmax(logits, dim=-1).to(torch.int32))
     if (logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla"
             and 0 < cfg.sample_topk <= 8):
         # the draw is the inverse CDF over the k candidates at one uniform number per row
         from lyra_amd.kernels.decode_fused import sample_topk
 
         u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=generator)
-        return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]))
+        return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]), out)
     logits = logits.to(torch.float32) / cfg.sample_temperature
     if 0 < cfg.sample_topk < logits.shape[-1]:
         top = torch.topk(logits, cfg.sample_topk, dim=-1)
         masked = torch.full_like(logits, torch.finfo(torch.float32).min)
         logits = masked.scatter(-1, top.indices, top.values)
     probs = torch.softmax(logits, dim=-1)
-    return torch.multinomial(probs, 1, generator=generator)[:, 0].to(torch.int32)
+    return _into(out, torch.multinomial(probs, 1, generator=generator)[:, 0].to(torch.int32))
+
+
+def _into(out: torch.Tensor | None, value: torch.Tensor) -> torch.Tensor:
+    if out is None:
+        return value
+    out.copy_(value)
+    return out
 
 
 def generate(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig,
@@ -72,7 +80,7 @@ class GraphedDecoder:
     def _step(self):
         logits, _ = model_apply(self.tokens, self.model, self.cache, self.cfg)
         self.logits = logits
-        self.next_tokens.copy_(sample_token(logits, replace(self.cfg, sample_temperature=0.0) if self.greedy else self.cfg))
+        sample_token(logits, replace(self.cfg, sample_temperature=0.0) if self.greedy else self.cfg, out=self.next_tokens)
 
     def step(self) -> torch.Tensor:
         """Run one decode step on ``self.tokens``; returns the next tokens (device, int32): greedy, or sampled."""

@@ -148,7 +148,8 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
 
 def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,
          residual: torch.Tensor | None = None, out_scale: float | None = None, fused_swiglu: bool = False,
-         swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False) -> torch.Tensor:
+         swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False,
+         bias: torch.Tensor | None = None) -> torch.Tensor:
     """lyra_decode_gemm_ex: the decode grouped matmul with an optional row gather on the input and an optional
     ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray."""
     dev = lhs.device
@@ -170,10 +171,12 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
         assert residual.dtype == torch.bfloat16 and residual.is_contiguous() and tuple(residual.shape) == (M, NO)
     if row_map is not None:
         assert row_map.dtype == torch.int32 and row_map.numel() >= M
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == G * N
     stream = _stream(dev)
     need = _L.lyra_decode_gemm_workspace(M, G, K, N, int(fused_swiglu))
     ws = _lib.workspace("gemm", dev, stream, need)
-    rc = _L.lyra_decode_gemm_ex(lhs.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), None,
+    rc = _L.lyra_decode_gemm_ex(lhs.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
                                 _ptr(residual), 1.0 if out_scale is None else float(out_scale), int(out_scale is not None),
                                 out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
                                 _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
@@ -212,13 +215,15 @@ def moe_combine(rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, x:
     return out
 
 
-def argmax(logits: torch.Tensor, cols: int | None = None) -> torch.Tensor:
+def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
     """Greedy token choice (lyra/generate.py:46-53 at temperature 0): first index of each row's maximum over the first
     ``cols`` columns of float32 ``logits`` [rows, ld]; returns int32 [rows]."""
     rows, ld = logits.shape
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
-    out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_argmax_workspace(rows, cols))
     rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, stream)
@@ -226,7 +231,8 @@ def argmax(logits: torch.Tensor, cols: int | None = None) -> torch.Tensor:
     return out
 
 
-def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperature: float, cols: int | None = None) -> torch.Tensor:
+def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperature: float, cols: int | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
     """Temperature / top-k token choice (lyra/generate.py:46-53 at temperature > 0) for every row of float32 ``logits``
     [rows, ld] over its first ``cols`` columns: softmax of the k largest ``logits / temperature`` (ties to the lower
     index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows]."""
@@ -234,7 +240,9 @@ def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperatur
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
     assert uniforms.dtype == torch.float32 and uniforms.shape == (rows,) and uniforms.is_contiguous()
-    out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_sample_topk_workspace(rows, cols, k))
     rc = _L.lyra_sample_topk(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,

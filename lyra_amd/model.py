@@ -201,6 +201,9 @@ class ModelWeights:
     unemb_t: torch.Tensor     # [1, C, V_padded] bf16: LM head weight laid out for the decode matmul
     norm_scale: torch.Tensor  # [C] f32
     layers: list[LayerWeights] = field(default_factory=list)
+    # [1, V_padded] f32: 0 for real tokens, -inf for the padding of the vocabulary.  Passed to the LM-head matmul as its
+    # bias, it makes `logits[:, vocab_size:] = -inf` (lyra/model.py:789) part of that launch.
+    vocab_mask: torch.Tensor | None = None
 
 
 def _maybe_quantize(w: torch.Tensor, cfg: ModelConfig, enabled: bool):
@@ -253,7 +256,9 @@ def init_weights(cfg: ModelConfig, device, seed: int | None = None) -> ModelWeig
         layers.append(LayerWeights(attn=attn, mlp=mlp))
     emb = rnd(cfg.padded_vocab_size, C)
     unemb = emb if cfg.tie_embeddings else rnd(cfg.padded_vocab_size, C)
-    return ModelWeights(emb=emb, unemb_t=unemb.t().contiguous()[None], norm_scale=ones(C), layers=layers)
+    vocab_mask = torch.zeros(1, cfg.padded_vocab_size, dtype=torch.float32, device=device)
+    vocab_mask[:, cfg.vocab_size :] = float("-inf")
+    return ModelWeights(emb=emb, unemb_t=unemb.t().contiguous()[None], norm_scale=ones(C), layers=layers, vocab_mask=vocab_mask)
 
 
 # ---- KV cache ----------------------------------------------------------------------------------------
@@ -477,8 +482,9 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
         h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
         h = moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
     h = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)[0]
-    logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True)
-    logits[:, cfg.vocab_size :] = float("-inf")
+    logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
+    if model.vocab_mask is None:
+        logits[:, cfg.vocab_size :] = float("-inf")
     cache.pos += 1
     return logits, cache
 
