@@ -149,7 +149,8 @@ int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const float* rhs
 int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C,
                       int n, int mode, float eps, lyra_stream_t stream);
 /* Same, but the row to normalise is first formed from unsummed projection slices (lyra/model.py:371-374, 631-636):
- * x_out = bf16(residual + bf16(bf16(sum_s partials[s]) * out_scale)), partials [splits, B, C] float32; x is ignored. */
+ * x_out = bf16(residual + bf16(bf16(sum_s partials[s]) * out_scale)), partials [splits, B, C] float32; x is ignored.
+ * x_out and h must not overlap the inputs (several workgroups read a row while one of them writes its outputs). */
 int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale, void* x_out,
                           const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C, int n,
                           int mode, float eps, lyra_stream_t stream);

@@ -49,7 +49,10 @@ constexpr int kNormThreads = 1024;
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjParams p) {
     extern __shared__ float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
     float* sm_red = sm_h + p.C;
-    const int b = blockIdx.x;
+    // blockIdx.y: which share of the projection outputs this workgroup computes.  The shares of a row each normalise the
+    // row again (cheap: the input comes from L2) so that the projection matrix, which every row needs in full, is pulled
+    // through 4 compute units per row instead of one; share 0 writes the row's other outputs.
+    const int b = blockIdx.x, share = blockIdx.y, shares = gridDim.y;
     const uint16_t* xr = p.x + (size_t)b * p.C;
     float ss = 0.f;
     for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // C % 4 == 0
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
             const float r2 = __uint_as_float(r[1] << 16), r3 = __uint_as_float(r[1] & 0xFFFF0000u);
             d[0] = pack_bf16(r0 + bf16r(bf16r(t[0]) * p.out_scale), r1 + bf16r(bf16r(t[1]) * p.out_scale));
             d[1] = pack_bf16(r2 + bf16r(bf16r(t[2]) * p.out_scale), r3 + bf16r(bf16r(t[3]) * p.out_scale));
-            *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
+            if (share == 0) *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
         } else {
             d = *(const u32x2*)(xr + c);
         }
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
         u32x2 d;
         d[0] = pack_bf16(v[0], v[1]);
         d[1] = pack_bf16(v[2], v[3]);
-        *(u32x2*)(p.h + (size_t)b * p.C + c) = d;
+        if (share == 0) *(u32x2*)(p.h + (size_t)b * p.C + c) = d;
         sm_h[c] = __uint_as_float(d[0] << 16);
         sm_h[c + 1] = __uint_as_float(d[0] & 0xFFFF0000u);
         sm_h[c + 2] = __uint_as_float(d[1] << 16);
@@ -104,7 +107,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     if (!p.proj_t) return;
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int j = wave; j < p.n; j += kNormThreads / 64) {
+    const int per_share = (p.n + shares - 1) / shares, j_end = min(p.n, (share + 1) * per_share);
+    for (int j = share * per_share + wave; j < j_end; j += kNormThreads / 64) {
         // one output per wavefront at a time; its weight row is requested 8 x 16 bytes per lane at once (offsets past
         // the row read as zeros), so a row of up to 2048 columns costs one memory round trip
         const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.proj_t) + (size_t)j * p.C, 0,
@@ -609,7 +613,8 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out};
     const size_t lds = ((size_t)C + 16) * sizeof(float);
-    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B), dim3(kNormThreads), lds, (hipStream_t)stream, p);
+    const int shares = (proj_t && n >= 8 && B <= 256) ? 4 : 1;
+    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 
