@@ -3,6 +3,7 @@
 // per layer instead of hundreds of elementwise ones.  All arithmetic follows the reference's dtype flow: bf16
 // activations, float32 maths inside an op, a bf16 rounding wherever the JAX code holds a bf16 array.
 #include <algorithm>
+#include <cstdlib>
 
 #include "lyra_device.h"
 
@@ -613,7 +614,8 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out};
     const size_t lds = ((size_t)C + 16) * sizeof(float);
-    const int shares = (proj_t && n >= 8 && B <= 256) ? 4 : 1;
+    static const int shares_env = [] { const char* e = getenv("LYRA_NORM_SHARES"); return e ? atoi(e) : 4; }();  // tuning override
+    const int shares = (proj_t && n >= 8 && B <= 256) ? std::max(1, std::min(shares_env, n)) : 1;
     hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
