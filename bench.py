@@ -142,7 +142,7 @@ def zipf_group_sizes(rng, tokens, n_routed, k_routed, n_shared):
     return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
 
 
-def kernel_table(dev):
+def kernel_table(dev, only=""):
     """Stand-alone timings of the two operators through the C ABI at the shapes of the named model variants: HIP events
     over back-to-back launches, once rotating over enough distinct caches / weight sets that every launch streams from
     HBM ("cold") and once re-using one set ("hot", which the 256 MB last-level cache may serve in part)."""
@@ -158,6 +158,8 @@ def kernel_table(dev):
     gen.manual_seed(1000)
 
     def attention(label, B, N, K, H, S, sw, fp8, lengths=None):
+        if only not in label:
+            return
         es = 1 if fp8 else 2
         per = 2 * B * K * S * (H * es + (4 if fp8 else 0))
         nbuf = max(2, min(8, int(1.2e9 // per) + 1))
@@ -197,6 +199,8 @@ def kernel_table(dev):
         del caches
 
     def gemm(label, M, G, K, N, sizes, swiglu, block, fp8=True, out_f32=False):
+        if only not in label:
+            return
         es = 1 if fp8 else 2
         nbuf = max(2, min(6, int(600e6 // (G * K * N * es)) + 1))
         if fp8:
@@ -327,6 +331,7 @@ def main():
     ap.add_argument("--model", default="lyra-small", help="model variant of the decode step (the headline figure is lyra-small)")
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
+    ap.add_argument("--only", default="", help="with --kernels: only the cases whose name contains this text")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a copy-like kernel of known size (reference point for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -338,7 +343,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.kernels:
-        rows = kernel_table(dev)
+        rows = kernel_table(dev, args.only)
+        if args.traffic_probe:
+            traffic_probe(dev)
         for r in rows:
             print(f"| {r['operator']} | {r['case']} | {r['bytes'] / 1e6:.1f} | {r['cold_us']:.1f} | {r['cold_GBs'] / 1e3:.2f} | "
                   f"{100 * r['cold_frac_of_peak']:.1f} | {r['hot_us']:.1f} |", file=sys.stderr)
