@@ -53,6 +53,7 @@ def build_model(batch, ctx, device, variant="lyra-small"):
 
 
 def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup):
+    """Wall time of `steps` replays of the captured decode step; also returns the function that runs one more step."""
     import torch
 
     from lyra_amd.generate import GraphedDecoder
@@ -73,12 +74,15 @@ def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert torch.isfinite(dec.logits[:, : cfg.vocab_size]).all(), "non-finite logits"
-    return elapsed
+    return elapsed, one_step
 
 
-def time_dominant_kernel(cfg, weights, cache, batch, ctx, launches=100):
-    """Average duration of the FP8 global-layer decode-attention launch, HIP events on the launch stream, rotating
-    over the caches of the model's global layers so every launch streams from HBM (working set >> 256 MB MALL)."""
+def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13):
+    """Average duration of the FP8 global-layer decode-attention launch through the C ABI, HIP events on the launch
+    stream.  The launches come as they do in the workload: one per global layer of the model (each on that layer's
+    cache, so every launch streams from HBM), timed as a group, with a replay of the whole decode step between groups.
+    (A hundred launches back to back measure something else: at 6 TB/s the device reaches its power limit within
+    milliseconds and the launch time climbs from 44 to 54 us.)"""
     import torch
 
     from lyra_amd import _lib
@@ -95,24 +99,25 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, launches=100):
     ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
 
-    def launch(i):
-        c = layers[i % len(layers)]
+    def launch(c):
         rc = L.lyra_decode_attention(
             q.data_ptr(), c.k.qval.data_ptr(), c.v.qval.data_ptr(), c.k.scale.data_ptr(), c.v.scale.data_ptr(), sinks.data_ptr(),
             pos.data_ptr(), 0, None, out.data_ptr(), ws.data_ptr(), ws.numel(), batch, N, K, ctx, H, H**-0.5, 0,
             _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, stream.cuda_stream)
         _lib.check(rc, "lyra_decode_attention")
 
-    for i in range(10):
-        launch(i)
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pairs = []
+    for r in range(rounds + 2):  # the first two groups warm up
+        one_step()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for c in layers:
+            launch(c)
+        stop.record(stream)
+        if r >= 2:
+            pairs.append((start, stop))
     stream.synchronize()
-    start.record(stream)
-    for i in range(launches):
-        launch(i)
-    stop.record(stream)
-    stop.synchronize()
-    return start.elapsed_time(stop) * 1e-3 / launches  # seconds per launch
+    return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / (len(pairs) * len(layers))  # seconds per launch
 
 
 def _time_launches(launch, stream, warm=5, iters=50):
@@ -352,10 +357,10 @@ def main():
         print(json.dumps({"metric": "operator launch time at model shapes", "unit": "us", "peak_GBs": HBM_PEAK_GBS, "kernels": rows}))
         return
     cfg, weights, cache = build_model(args.batch, args.ctx, dev, args.model)
-    elapsed = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
+    elapsed, one_step = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
     tokens_per_s = args.batch * args.steps / elapsed
 
-    t_attn = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx)
+    t_attn = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step)
     attn_bytes = attention_algorithmic_bytes(args.batch, cfg.n_kv_heads, args.ctx, cfg.head_dim, fp8=True)
     achieved = attn_bytes / t_attn / 1e9
     traffic = None

@@ -115,7 +115,7 @@ __device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int w = 0; w < KW; w += 4) {
-            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, voff + j * 16 * RB + (w / 4) * 64, soff, 0);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.k, voff + j * 16 * RB + (w / 4) * 64, soff, kStream);
             t.k[j][w] = d[0];
             t.k[j][w + 1] = d[1];
             t.k[j][w + 2] = d[2];
@@ -130,8 +130,8 @@ __device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base, bool l
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         if constexpr (VEC4) {
-            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(sl.ks, voff + j * 64, ssoff, 0);
-            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(sl.vs, voff + j * 64, ssoff, 0);
+            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(sl.ks, voff + j * 64, ssoff, kStream);
+            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(sl.vs, voff + j * 64, ssoff, kStream);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 t.ks[4 * j + r] = __uint_as_float(a[r]);
@@ -140,8 +140,8 @@ __device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base, bool l
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                t.ks[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.ks, voff + j * 64 + r * 4, ssoff, 0));
-                t.vs[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.vs, voff + j * 64 + r * 4, ssoff, 0));
+                t.ks[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.ks, voff + j * 64 + r * 4, ssoff, kStream));
+                t.vs[4 * j + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sl.vs, voff + j * 64 + r * 4, ssoff, kStream));
             }
         }
     }
@@ -158,13 +158,13 @@ __device__ __forceinline__ void load_v(RawV<H, FP8>& t, const Slab& sl, int base
     for (int i = 0; i < 8; ++i) {
         const int off = voff + (16 * (i >> 2) + (i & 3)) * RB;
         if constexpr (VW == 1) {
-            t.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(sl.v, off, soff, 0);
+            t.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(sl.v, off, soff, kStream);
         } else if constexpr (VW == 2) {
-            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(sl.v, off, soff, 0);
+            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(sl.v, off, soff, kStream);
             t.v[i][0] = d[0];
             t.v[i][1] = d[1];
         } else {
-            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.v, off, soff, 0);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(sl.v, off, soff, kStream);
             t.v[i][0] = d[0];
             t.v[i][1] = d[1];
             t.v[i][2] = d[2];

@@ -96,11 +96,11 @@ __device__ __forceinline__ void load_w_pair(RawW<FP8>& t, int pair, __amdgpu_buf
         const int i = 2 * pair + h;
         const int soff = __builtin_amdgcn_readfirstlane((kk + i) * row_bytes);
         if constexpr (FP8) {
-            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 0);
+            const u32x2 d = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, kStream);
             t.w[i][0] = d[0];
             t.w[i][1] = d[1];
         } else {
-            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+            const u32x4 d = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, kStream);
             t.w[i][0] = d[0];
             t.w[i][1] = d[1];
             t.w[i][2] = d[2];

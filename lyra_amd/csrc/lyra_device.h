@@ -22,6 +22,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 // A buffer-load lane offset beyond any buffer descriptor used here (all are shorter than 2 GiB; the constant
 // offsets added to it stay far below 4 GiB): such a load returns zeros without touching memory.
 constexpr int kNoLoad = (int)0x80000000u;
+// Cache policy of buffer loads that stream data read once per launch (KV cache, weights): non-temporal.  A plain linear
+// read of 277 MB runs at 7.1 TB/s with it and at 6.3 TB/s without.
+constexpr int kStream = 2;
 
 // D(16x16,f32) += A(16x32,bf16) * B(32x16,bf16).  Lane l supplies row (l & 15) of A and column
 // (l & 15) of B, each as the 8 consecutive k-slots of k-group (l >> 4); both operands use the same
