@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 6
+#define LYRA_ABI_VERSION 7
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -154,6 +154,12 @@ int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* p
 int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale, void* x_out,
                           const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C, int n,
                           int mode, float eps, lyra_stream_t stream);
+/* Same, but the row to normalise is the residual update that ends a MoE layer (lyra/model.py:557-567; what lyra_moe_combine
+ * computes): x_out = bf16(residual + bf16(bf16(sum_k scores[b,k] * rows[dest[b*topk+k]]) * out_scale)), rows [B*topk, C]
+ * bf16 in sorted order, scores [B, topk] float32, dest [B*topk] int32, topk <= 16.  Same aliasing rule. */
+int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, const int32_t* dest, int topk, const void* residual,
+                              float out_scale, void* x_out, const float* scale, void* h, const float* proj_t, const float* bias,
+                              void* y, int B, int C, int n, int mode, float eps, lyra_stream_t stream);
 
 /*
  * lyra_qkv_post: everything between the fused q/k/v projection and the attention kernel (model.py:309-336):

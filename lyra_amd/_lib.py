@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _c = ctypes
 SIGNATURES = {
@@ -45,6 +45,10 @@ SIGNATURES = {
     "lyra_rmsnorm_proj_sum": (
         _c.c_int,
         [_c.c_void_p] * 2 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
+    ),
+    "lyra_rmsnorm_proj_combine": (
+        _c.c_int,
+        [_c.c_void_p] * 3 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
     ),
     "lyra_qkv_post_sum": (
         _c.c_int,

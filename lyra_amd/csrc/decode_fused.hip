@@ -43,10 +43,18 @@ struct NormProjParams {
     const uint16_t* residual;
     float out_scale;
     uint16_t* x_out;
+    // or: the row is the residual update that ends a MoE layer (lyra/model.py:557-567),
+    // bf16(residual + bf16(bf16(sum_k scores[b,k] * rows[dest[b,k]]) * out_scale)), also written to x_out
+    const uint16_t* comb_rows;  // [B * topk, C] expert outputs in sorted order, or null
+    const float* comb_scores;   // [B, topk]
+    const int32_t* comb_dest;   // [B, topk] sorted row of every assignment
+    int comb_topk;              // <= 16
 };
 
 constexpr int kNormThreads = 1024;
 
+// COMBINE: the instantiation whose rows come from a MoE layer's combine step (comb_rows set).
+template <bool COMBINE>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjParams p) {
     extern __shared__ float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
     float* sm_red = sm_h + p.C;
@@ -56,9 +64,37 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     const int b = blockIdx.x, share = blockIdx.y, shares = gridDim.y;
     const uint16_t* xr = p.x + (size_t)b * p.C;
     float ss = 0.f;
+    [[maybe_unused]] int comb_row[16];
+    [[maybe_unused]] float comb_sc[16];
+    if constexpr (COMBINE) {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            comb_row[k] = k < p.comb_topk ? p.comb_dest[b * p.comb_topk + k] : 0;
+            comb_sc[k] = k < p.comb_topk ? p.comb_scores[b * p.comb_topk + k] : 0.f;
+        }
+    }
     for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // C % 4 == 0
         u32x2 d;
-        if (p.partials) {
+        if constexpr (COMBINE) {
+            // the expert outputs of this token in assignment order, as the combine step adds them
+            float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                if (k < p.comb_topk) {
+                    const u32x2 e = *(const u32x2*)(p.comb_rows + (size_t)comb_row[k] * p.C + c);
+                    t[0] += __uint_as_float(e[0] << 16) * comb_sc[k];
+                    t[1] += __uint_as_float(e[0] & 0xFFFF0000u) * comb_sc[k];
+                    t[2] += __uint_as_float(e[1] << 16) * comb_sc[k];
+                    t[3] += __uint_as_float(e[1] & 0xFFFF0000u) * comb_sc[k];
+                }
+            }
+            const u32x2 r = *(const u32x2*)(p.residual + (size_t)b * p.C + c);
+            const float r0 = __uint_as_float(r[0] << 16), r1 = __uint_as_float(r[0] & 0xFFFF0000u);
+            const float r2 = __uint_as_float(r[1] << 16), r3 = __uint_as_float(r[1] & 0xFFFF0000u);
+            d[0] = pack_bf16(r0 + bf16r(bf16r(t[0]) * p.out_scale), r1 + bf16r(bf16r(t[1]) * p.out_scale));
+            d[1] = pack_bf16(r2 + bf16r(bf16r(t[2]) * p.out_scale), r3 + bf16r(bf16r(t[3]) * p.out_scale));
+            if (share == 0) *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
+        } else if (!COMBINE && p.partials) {
             // slices are requested 8 at a time (slices past the last read as zeros) and added in slice order
             const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<float*>(p.partials), 0, (uint32_t)((size_t)p.splits * p.B * p.C * 4), 0x00020000);
@@ -597,6 +633,17 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
 
 }  // namespace lyra
 
+namespace lyra {
+static int launch_rmsnorm_proj(const NormProjParams& p, int B, lyra_stream_t stream) {
+    const size_t lds = ((size_t)p.C + 16) * sizeof(float);
+    static const int shares_env = [] { const char* e = getenv("LYRA_NORM_SHARES"); return e ? atoi(e) : 4; }();  // tuning override
+    const int shares = (p.proj_t && p.n >= 8 && B <= 256) ? std::max(1, std::min(shares_env, p.n)) : 1;
+    if (p.comb_rows) hipLaunchKernelGGL(rmsnorm_proj_kernel<true>, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
+    else hipLaunchKernelGGL(rmsnorm_proj_kernel<false>, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+}  // namespace lyra
+
 extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
                                  int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
     return lyra_rmsnorm_proj_sum(x, nullptr, 0, nullptr, 1.0f, nullptr, scale, h, proj_t, bias, y, B, C, n, mode, eps, stream);
@@ -612,12 +659,22 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
-                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out};
-    const size_t lds = ((size_t)C + 16) * sizeof(float);
-    static const int shares_env = [] { const char* e = getenv("LYRA_NORM_SHARES"); return e ? atoi(e) : 4; }();  // tuning override
-    const int shares = (proj_t && n >= 8 && B <= 256) ? std::max(1, std::min(shares_env, n)) : 1;
-    hipLaunchKernelGGL(rmsnorm_proj_kernel, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
-    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0};
+    return launch_rmsnorm_proj(p, B, stream);
+}
+
+extern "C" int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, const int32_t* dest, int topk, const void* residual,
+                                         float out_scale, void* x_out, const float* scale, void* h, const float* proj_t,
+                                         const float* bias, void* y, int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!rows || !scores || !dest || !residual || !x_out || topk <= 0) return LYRA_E_BADARG;
+    if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
+    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (C % 4 || C > 32768 || topk > 16) return LYRA_E_UNSUPPORTED;
+    NormProjParams p{nullptr, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
+                     nullptr, 0, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out,
+                     (const uint16_t*)rows, scores, dest, topk};
+    return launch_rmsnorm_proj(p, B, stream);
 }
 
 extern "C" int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,

@@ -51,6 +51,17 @@ class Unsummed:
         self.partials, self.residual, self.scale = partials, residual, scale
 
 
+class Uncombined:
+    """The end of a MoE layer before its combine step: expert outputs ``rows`` [T * topk, C] bf16 in sorted order,
+    ``scores`` [T, topk] float32, ``dest`` [T * topk] int32, the residual stream ``residual`` [T, C] bf16 and the residual
+    ``scale``; the kernel that consumes it forms bf16(residual + bf16(bf16(sum_k scores * rows[dest]) * scale))."""
+
+    __slots__ = ("rows", "scores", "dest", "residual", "scale")
+
+    def __init__(self, rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, residual: torch.Tensor, scale: float):
+        self.rows, self.scores, self.dest, self.residual, self.scale = rows, scores, dest, residual, scale
+
+
 def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed | None:
     """lyra_decode_gemm_partials for a one-group projection; None when the shape does not run split over K."""
     M, K = lhs.shape
@@ -78,7 +89,26 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
     float32 logits, or bf16 ``2*sigmoid`` gates when ``gate`` is set (model.py:343-347).  Returns (h, y | None).
 
     ``x`` may be an ``Unsummed`` projection with its residual: the row is then first formed as
-    ``bf16(residual + bf16(bf16(sum of slices) * scale))`` and returned as a third value."""
+    ``bf16(residual + bf16(bf16(sum of slices) * scale))`` and returned as a third value.  Likewise for an ``Uncombined``
+    MoE layer end (the combine step of lyra/model.py:557-567 happens while the row is read)."""
+    if isinstance(x, Uncombined):
+        u = x
+        B, C = u.residual.shape
+        topk = u.scores.shape[1]
+        assert u.residual.dtype == torch.bfloat16 and u.residual.is_contiguous()
+        assert u.rows.dtype == torch.bfloat16 and u.rows.is_contiguous() and tuple(u.rows.shape) == (B * topk, C)
+        x_out = torch.empty_like(u.residual)
+        h = torch.empty_like(u.residual)
+        y, n = None, 0
+        if proj is not None:
+            n = proj.shape[1]
+            y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=h.device)
+            proj = _f32(_transposed(proj))
+        rc = _L.lyra_rmsnorm_proj_combine(u.rows.data_ptr(), _f32(u.scores).data_ptr(), u.dest.data_ptr(), topk, u.residual.data_ptr(),
+                                          float(u.scale), x_out.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj),
+                                          _ptr(bias), _ptr(y), B, C, n, 1 if gate else 2, float(eps), _stream(h.device))
+        _lib.check(rc, "lyra_rmsnorm_proj_combine")
+        return h, y, x_out
     if isinstance(x, Unsummed):
         u = x
         splits, B, C = u.partials.shape

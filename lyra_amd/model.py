@@ -9,6 +9,8 @@ one thing a decode loop cannot afford), everything else is a pure function of it
 """
 from __future__ import annotations
 
+import os
+
 import math
 from dataclasses import dataclass, field, replace
 from functools import lru_cache
@@ -399,6 +401,7 @@ def _one_group(rows: int, device) -> torch.Tensor:
 
 
 _ONE_GROUP: dict = {}
+_SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tuning override: combine in a launch of its own
 
 
 def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
@@ -408,7 +411,7 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     from lyra_amd.kernels import decode_fused as F
 
     H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
-    if isinstance(x, F.Unsummed):
+    if isinstance(x, (F.Unsummed, F.Uncombined)):
         h, gate, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
     else:
         h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
@@ -429,11 +432,12 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
 
 
 def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
-    """moe_apply as norm+router | routing | up matmul (token gather fused) | down matmul | combine+residual."""
+    """moe_apply as norm+router | routing | up matmul (token gather fused) | down matmul; the combine + residual step is
+    handed to the next norm as an ``Uncombined`` value."""
     from lyra_amd.kernels import decode_fused as F
 
     topk = cfg.n_active_experts
-    if isinstance(x, F.Unsummed):
+    if isinstance(x, (F.Unsummed, F.Uncombined)):
         xn, logits, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
     else:
         xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
@@ -442,13 +446,15 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
     t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
                swiglu_limit=cfg.swiglu_limit)
     t = F.gemm(t, w.mlp_down, groups)
+    if topk <= 16 and not _SEPARATE_COMBINE:  # the combine step is left to the norm that follows (the next layer's, or the final one)
+        return F.Uncombined(t, scores, dest, x, cfg.residual_scale)
     return F.moe_combine(t, scores, dest, x, cfg.residual_scale)
 
 
 def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     from lyra_amd.kernels import decode_fused as F
 
-    if isinstance(x, F.Unsummed):
+    if isinstance(x, (F.Unsummed, F.Uncombined)):
         t, _, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     else:
         t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)

@@ -317,6 +317,35 @@ def test_unsummed_projection_consumers_equal_summed_path(fp8, B, C, N, K, H):
     assert torch.equal(x1, x2) and torch.equal(h1, h2) and torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("T,topk,C,n,gate", [(64, 4, 2048, 16, True), (64, 4, 2048, 15, False), (3, 2, 256, 0, False), (17, 16, 4096, 7, False)])
+def test_uncombined_moe_layer_end_equals_combine_then_norm(T, topk, C, n, gate):
+    """Leaving the combine step of a MoE layer to the norm that follows must give bit for bit what combining first gives,
+    and the combined row itself is checked against the oracle."""
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"uncombined T{T} topk{topk} C{C} n{n}")
+    dev = U.dev()
+    rng = np.random.default_rng(T * 31 + topk)
+    rows_np = O.bf16_round(rng.standard_normal((T * topk, C), dtype=np.float32))
+    x_np = O.bf16_round(rng.standard_normal((T, C), dtype=np.float32))
+    scores_np = rng.random((T, topk)).astype(np.float32)
+    dest_np = rng.permutation(T * topk).astype(np.int32)
+    rows, x, scores, dest = U.t_bf16(rows_np), U.t_bf16(x_np), U.t_f32(scores_np), torch.from_numpy(dest_np).to(dev)
+    rs = 0.1767766952966369
+    g = torch.Generator(device=dev)
+    g.manual_seed(T)
+    scale = torch.rand(C, generator=g, device=dev) + 0.5
+    proj = torch.randn(C, n, generator=g, device=dev) * 0.05 if n else None
+    bias = torch.randn(n, generator=g, device=dev) if (n and not gate) else None
+    h1, y1, x1 = F.rmsnorm_proj(F.Uncombined(rows, scores, dest, x, rs), scale, 1e-5, proj, bias, gate=gate)
+    x2 = F.moe_combine(rows, scores, dest, x, rs)
+    h2, y2 = F.rmsnorm_proj(x2, scale, 1e-5, proj, bias, gate=gate)
+    assert torch.equal(x1, x2) and torch.equal(h1, h2)
+    assert (y1 is None and y2 is None) or torch.equal(y1, y2)
+    t = O.bf16_round(O.bf16_round(O.combine(rows_np, scores_np, dest_np)) * np.float32(rs))
+    _bf16_close(U.to_np(x1), x_np + t, "combined row")
+
+
 @pytest.mark.parametrize("rows,cols,ld,k,temperature", [(64, 201088, 204800, 4, 0.8), (3, 1000, 1024, 8, 1.5), (130, 5000, 5000, 1, 0.3),
                                                         (1, 201088, 204800, 4, 0.8), (5, 7, 8, 4, 1.0)])
 def test_sample_topk_matches_oracle(rows, cols, ld, k, temperature):
