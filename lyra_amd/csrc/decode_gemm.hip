@@ -41,6 +41,7 @@ struct GemmParams {
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
     int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
     int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
+    int even_spans;     // plain kernel: spans dealt out evenly over one workgroup per compute unit
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
     const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
     float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
@@ -187,7 +188,7 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
 }
 
 template <bool FP8, int MT>
-__global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 3 : 2)))
+__global__ __launch_bounds__(MT == 1 ? 768 : 512) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 3 : 2)))
 void decode_gemm_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int KC = 512;          // rows of K whose activations are staged in LDS at a time
@@ -196,7 +197,14 @@ void decode_gemm_kernel(GemmParams p) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
     const int g = blockIdx.z / p.row_par, rpar = blockIdx.z - g * p.row_par, ks = blockIdx.y;
-    const int span = blockIdx.x * kGemmWaves + wave;  // which 128-column span this wavefront owns
+    const int nwaves = blockDim.x >> 6;
+    // which 128-column span this wavefront owns: 4 per workgroup, or (p.even_spans, one workgroup per compute unit)
+    // workgroup i of n takes spans [i * total / n, (i + 1) * total / n), so that every compute unit has the same number
+    // of spans to within one - 1600 spans as 400 workgroups of 4 leave 144 compute units with 8 spans and 112 with 4
+    const int total_spans = p.swiglu ? (p.N >> 1) / 64 : p.N / 128;
+    const int first_span = p.even_spans ? (int)((long)blockIdx.x * total_spans / gridDim.x) : (int)blockIdx.x * kGemmWaves;
+    const int end_span = p.even_spans ? (int)((long)(blockIdx.x + 1) * total_spans / gridDim.x) : total_spans;
+    const int span = first_span + wave;
 
     // rows of this group: [off, off + cnt)
     int part_sum = 0;
@@ -214,11 +222,11 @@ void decode_gemm_kernel(GemmParams p) {
     const bool is_lin_lane = p.swiglu && x >= 8;
     if (p.swiglu) {
         const int half = p.N >> 1;
-        span_ok = span * 64 < half;
+        span_ok = span < end_span && span * 64 < half;
         out_col = span * 64 + 8 * (x & 7);
         ncol = is_lin_lane ? half + out_col : out_col;
     } else {
-        span_ok = span * 128 < p.N;
+        span_ok = span < end_span && span * 128 < p.N;
         ncol = out_col = span * 128 + 8 * x;
     }
     if (!span_ok) ncol = out_col = 0;  // idle wavefront of the last workgroup: keeps pace, stores nothing
@@ -266,7 +274,7 @@ void decode_gemm_kernel(GemmParams p) {
             __syncthreads();  // the previous chunk has been consumed by every wavefront
             const int pieces = (kc_end - kc) >> 3;  // <= 64
             if (lane < pieces) {
-                for (int r = wave; r < 16 * n_mt; r += kGemmWaves) {
+                for (int r = wave; r < 16 * n_mt; r += nwaves) {
                     u32x4 d = u32x4{0u, 0u, 0u, 0u};
                     if (r < rows_here) {
                         const int src = p.row_map ? p.row_map[rowbase + r] : rowbase + r;
@@ -1482,6 +1490,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         return e ? atoi(e) : 64;
     }();
     p.max_slices = max_slices_env;
+    p.even_spans = 0;
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
     p.post_scale = post_scale != 0;
@@ -1563,7 +1572,15 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
 #undef LYRA_SMALL
         return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
     }
-    const dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
+    dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
+    // a very wide single projection (the LM head): one workgroup per compute unit with as many wavefronts as its share of spans
+    static const bool no_even = getenv("LYRA_GEMM_NO_EVEN_SPANS") != nullptr;  // tuning override
+    const int per_cu = (pl.spans + kGroupMaxWgs - 1) / kGroupMaxWgs;
+    if (!no_even && G == 1 && pl.ksplit == 1 && pl.row_par == 1 && pl.spans >= 4 * kGroupMaxWgs && per_cu <= (pl.mt == 1 ? 12 : 8)) {
+        p.even_spans = 1;
+        grid = dim3(kGroupMaxWgs, 1, 1);
+        block = dim3(per_cu * 64);
+    }
     const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t);
 #define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p)
     if (fp8) {
