@@ -254,6 +254,9 @@ def kernel_table(dev, only=""):
         s = zipf_group_sizes(rng, T, 31, 3, 1)
         gemm(f"lyra-medium expert up+SwiGLU T={T} (32x4096x8192 fp8)", int(s.sum()), 32, 4096, 8192, s, True, (4096, 1))
         gemm(f"lyra-medium expert down T={T} (32x4096x4096 fp8)", int(s.sum()), 32, 4096, 4096, s, False, (4096, 1))
+    even = np.array([8] * 31 + [64], np.int32)  # evenly routed tokens (what a load-balancing loss aims at) + the shared expert
+    gemm("lyra-medium expert up+SwiGLU T=64, even routing (32x4096x8192 fp8)", int(even.sum()), 32, 4096, 8192, even, True, (4096, 1))
+    gemm("lyra-medium expert down T=64, even routing (32x4096x4096 fp8)", int(even.sum()), 32, 4096, 4096, even, False, (4096, 1))
     s = zipf_group_sizes(rng, 64, 31, 3, 1)
     gemm("lyra-medium expert up+SwiGLU T=64, scale blocks (256,256)", int(s.sum()), 32, 4096, 8192, s, True, (256, 256))
     s = zipf_group_sizes(rng, 128, 63, 3, 1)
