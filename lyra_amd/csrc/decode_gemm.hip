@@ -893,7 +893,9 @@ __device__ __forceinline__ int wg_scan_exclusive(int v, int* sm4, int lane, int 
     return base + incl - v;
 }
 
-template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED>
+// WIDE_DYN: an instantiation for launches without SwiGLU that may have enough units for the wider ones (decided below,
+// once the unit list is known; the other instantiations know their layout from the start).
+template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int DEPTH = FP8 ? 4 : 2;
@@ -907,19 +909,26 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     const int x = lane & 15, kb = lane >> 4;
 
     // wide: a unit is two sets of 128 columns, each taken by a pair of wavefronts that interleave over K (gate and linear
-    // columns with SwiGLU, else two adjacent spans); otherwise one set of 128 columns and all 4 wavefronts interleave
-    const bool wide = p.swiglu || p.wide;
-    const int spans = p.swiglu ? (p.N >> 1) / 128 : (wide ? p.N / 256 : p.N / 128);
-    const int kw = wide ? 2 : kSplitWaves;
-    const int wslot = wide ? (wave & 1) : wave, half = wide ? (wave >> 1) : 0;
-    const int half_stride = p.swiglu ? (p.N >> 1) : 128, span_cols = p.swiglu || !wide ? 128 : 256;
-    const int tile_cols = wide ? 256 : 128;  // floats per row of a workspace slot
+    // columns with SwiGLU, else two adjacent spans: 256 contiguous bytes of every weight row per workgroup instead of 128,
+    // which streams ~14 % faster); otherwise one set of 128 columns and all 4 wavefronts interleave.
     const int NO = p.swiglu ? p.N >> 1 : p.N;
     const int q = threadIdx.x & 31;
     const int row_bytes = p.N * ES;
     const int steps = p.K >> 5;
-    const int n_my = (steps - wslot + kw - 1) / kw;                      // steps of this wavefront in a whole unit
-    const int trips = ((steps + kw - 1) / kw + TRIP - 1) / TRIP;        // trips of a whole unit (same for every wavefront)
+    const int half_stride = p.swiglu ? (p.N >> 1) : 128;
+    bool wide;
+    int spans, kw, wslot, half, span_cols, tile_cols, n_my, trips;
+    auto set_layout = [&](bool w) {
+        wide = w;
+        spans = p.swiglu ? (p.N >> 1) / 128 : (w ? p.N / 256 : p.N / 128);
+        kw = w ? 2 : kSplitWaves;
+        wslot = w ? (wave & 1) : wave, half = w ? (wave >> 1) : 0;
+        span_cols = p.swiglu || !w ? 128 : 256;
+        tile_cols = w ? 256 : 128;                                  // floats per row of a workspace slot
+        n_my = (steps - wslot + kw - 1) / kw;                       // steps of this wavefront in a whole unit
+        trips = ((steps + kw - 1) / kw + TRIP - 1) / TRIP;          // trips of a whole unit (same for every wavefront)
+    };
+    if constexpr (!WIDE_DYN) set_layout(p.swiglu || p.wide);
 
     // ---- unit list: thread t looks at group G-1-t ----
     const int t = threadIdx.x;
@@ -953,8 +962,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         }
     }
     __syncthreads();
-    const int n_units = __builtin_amdgcn_readfirstlane(n_blocks * spans);  // (same in every lane: tell the compiler)
     const int nwg = gridDim.x;
+    // Without SwiGLU the wider units are taken when they still fill 1.75 rounds of workgroups (lyra-max down projection at
+    // batch 128: -8 %); with fewer, their coarser rounds cost more than the access pattern gains.
+    if constexpr (WIDE_DYN) set_layout(p.swiglu || p.wide || 4 * n_blocks * (p.N / 256) >= 7 * nwg);
+    const int n_units = __builtin_amdgcn_readfirstlane(n_blocks * spans);  // (same in every lane: tell the compiler)
     // whole units in full rounds of nwg; when there is not even one full round, the units are cut into `slices` K slices each
     // (a power of two that divides trips).  After a full round slicing the rest was measured to cost as much as it saves:
     // the few workgroups of a last partial round stream faster, having the memory system to themselves.
@@ -1520,9 +1532,21 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C>), ggrid, gblock, glds, st, p);                       \
     } while (0)
     // fewer units than workgroups whatever the group sizes: the variant that cuts units into K slices
+    // without SwiGLU, when the shapes allow 1.75 rounds of 256-column units: the variant that decides on them on the device
+    static const bool no_wide_dyn = getenv("LYRA_GEMM_NO_WIDE_IF_MANY") != nullptr;  // tuning override
+    const bool wide_dyn = !no_wide_dyn && !fused_swiglu && !pl.wide && N % 256 == 0 &&
+                          4 * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M)) * (N / 256) >= 7 * (long)kGroupMaxWgs;
+#define LYRA_GROUP_RSW(F, S, R)                                                                                       \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, false, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, false, true>), ggrid, gblock, glds, st, p);             \
+    } while (0)
 #define LYRA_GROUP_R(F, S, R)                                               \
     do {                                                                    \
         if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
+        else if (wide_dyn) LYRA_GROUP_RSW(F, S, R);                         \
         else LYRA_GROUP_RS(F, S, R, false);                                 \
     } while (0)
 #define LYRA_GROUP(F, S, DEPTH_)                                                          \
@@ -1538,6 +1562,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         else LYRA_GROUP(false, false, 2);
 #undef LYRA_GROUP
 #undef LYRA_GROUP_R
+#undef LYRA_GROUP_RSW
 #undef LYRA_GROUP_RS
         return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
     }

@@ -151,6 +151,20 @@ def test_config3_moe_medium_shape_zipf_routing(T):
     U.assert_close(_run(down, False), _want(down, False, big=True), what="down")
 
 
+@pytest.mark.parametrize("kind,block", [("fp8", (512, 1)), ("fp8", (128, 128)), ("bf16", None)])
+def test_down_projection_with_many_units_takes_256_column_units(kind, block):
+    """Without SwiGLU and with at least 1.75 rounds of 256-column units (here 34 row blocks x 16 = 544 for 256 workgroups)
+    the grouped kernel picks the wider units on the device; the result must not depend on that choice."""
+    G, K, N = 32, 512, 4096
+    rng = np.random.default_rng(77)
+    sizes = rng.integers(1, 9, size=G).astype(np.int32)
+    sizes[3], sizes[31] = 70, 129  # two and three row blocks
+    M = int(sizes.sum())
+    c = _case(21, M, G, K, N, sizes, kind=kind, block=block, bias=True)
+    _note(f"gemm many units {kind} {block} M={M}")
+    U.assert_close(_run(c, False), _want(c, False, big=True), what=f"many units {kind}")
+
+
 def test_reference_default_blocks_256_at_small_moe_shape():
     """lyra-small MoE: 15+1 experts, K=2048, up N=4096 with SwiGLU; QArray block (256,256) (model.py:154-156)."""
     rng = np.random.default_rng(8)
