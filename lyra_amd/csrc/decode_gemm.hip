@@ -1330,7 +1330,7 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     if (pl.grouped) {
         pl.mt = 4;
         pl.row_par = 1;
-        static const bool want_wide = getenv("LYRA_GEMM_WIDE") != nullptr;  // tuning override: measured no faster, off
+        static const bool want_wide = getenv("LYRA_GEMM_WIDE") != nullptr;  // tuning override: 256-column units whatever their number
         pl.wide = !fused_swiglu && N % 256 == 0 && want_wide;
         pl.spans = (fused_swiglu || pl.wide) ? N / 256 : N / 128;
         pl.ksplit = 1;

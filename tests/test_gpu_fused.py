@@ -188,7 +188,8 @@ def test_moe_combine(T, topk, C):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("M,G,K,N,swiglu", [(64, 1, 2048, 2048, False), (256, 16, 2048, 4096, True), (48, 8, 1024, 2048, False)])
+@pytest.mark.parametrize("M,G,K,N,swiglu", [(64, 1, 2048, 2048, False), (256, 16, 2048, 4096, True), (48, 8, 1024, 2048, False),
+                                              (320, 40, 512, 4096, False)])  # the last: enough units for the 256-column ones
 def test_gemm_row_map_and_residual_epilogue(fp8, M, G, K, N, swiglu):
     """The fused variants must equal the plain kernel composed with the torch ops they replace, bit for bit."""
     from lyra_amd.kernels import decode_fused as F
