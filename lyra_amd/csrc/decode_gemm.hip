@@ -42,6 +42,7 @@ struct GemmParams {
     int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
     int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
     int even_spans;     // plain kernel: spans dealt out evenly over one workgroup per compute unit
+    int row_block;      // K-split kernel: rows per workgroup (64 or 32)
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
     const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
     float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
@@ -637,7 +638,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
-    const int span = blockIdx.x, ks = blockIdx.y, row0 = blockIdx.z * 64;
+    const int span = blockIdx.x, ks = blockIdx.y, row0 = blockIdx.z * p.row_block;
     const int ncol = span * 128 + 8 * x;
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
     const int steps = (k1 - k0) >> 5;
@@ -654,10 +655,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
         const int arow = row0 + mt * 16 + x;
-        const int asrc = arow < p.M ? (p.row_map ? p.row_map[arow] : arow) : 0;
-        avoff[mt] = arow < p.M ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
+        const bool mine = arow < p.M && mt * 16 < p.row_block;
+        const int asrc = mine ? (p.row_map ? p.row_map[arow] : arow) : 0;
+        avoff[mt] = mine ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
     }
-    const int n_mt = min(4, (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
+    const int n_mt = min(p.row_block >> 4, (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
 
     // all operands are requested before anything is waited for, in the order they are consumed
     u32x4 a[DEPTH][4];
@@ -1302,6 +1304,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 struct GemmPlan {
     int mt;       // 16-row tiles held in registers per pass
     int row_par;  // row blocks of one group spread over this many workgroups
+    int row_block = 64;  // K-split kernel: rows per block
     int spans;    // 128-column spans (64+64 with SwiGLU)
     int ksplit, kpart;
     bool one_pass;  // single group with a few MB of weights, swiglu tile layout: decode_gemm_small_kernel
@@ -1342,8 +1345,22 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
         pl.mt = 4;
-        pl.row_par = (M + 63) / 64;
         pl.spans = (N + 127) / 128;
+        // Row blocks of 64, 32 or 16 rows: as many blocks as still leave K slices of 512 rows for ~256 workgroups.  These
+        // launches are bound by what one workgroup has to pull in and by the float32 slices their consumer sums, not by their
+        // bytes: smaller blocks shrink a workgroup's activation slice and partial tile, and more row blocks mean fewer K
+        // slices (2048-wide variant at 64 rows: q/k/v 8 -> 4 slices with 32-row blocks, output projection 8 -> 4 with 16-row
+        // blocks; decode step -3 %).  Matrices with enough spans and slices to fill the device keep 64-row blocks: smaller
+        // ones would read the weights again for nothing (4096-wide variant: +4 % when forced).
+        static const int row_block_env = [] {
+            const char* e = getenv("LYRA_GEMM_ROW_BLOCK");  // tuning override, read once: 16, 32 or 64 for every K-split launch
+            return e ? atoi(e) : 0;
+        }();
+        const long blocks_wanted = std::max(1L, 256L / ((long)pl.spans * ((K + 511) / 512)));
+        pl.row_block = 64;
+        while (pl.row_block > 16 && (M + pl.row_block / 2 - 1) / (pl.row_block / 2) <= blocks_wanted) pl.row_block /= 2;
+        if (row_block_env == 16 || row_block_env == 32 || row_block_env == 64) pl.row_block = row_block_env;
+        pl.row_par = (M + pl.row_block - 1) / pl.row_block;
         // slices of at least 256 rows: 128-row slices fill more compute units but double the float32 slices the consumer
         // has to sum (2048 x 2048 out projection: 16 -> 8 slices shortened the decode step by 1.2 %)
         int unit = (K % 256 == 0 && K >= 512) ? 256 : 128;
@@ -1494,6 +1511,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.limit = swiglu_limit;
     p.ksplit = pl.ksplit;
     p.row_par = pl.row_par;
+    p.row_block = pl.row_block;
     p.kpart = pl.kpart;
     p.row_map = lhs_row_map;
     p.wide = pl.wide;
@@ -1668,5 +1686,6 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     p.ksplit = pl.ksplit;
     p.kpart = pl.kpart;
     p.row_par = pl.row_par;
+    p.row_block = pl.row_block;
     return launch_split_k(p, pl, fp8, (hipStream_t)stream);
 }
