@@ -250,6 +250,10 @@ def kernel_table(dev, only=""):
     lengths = np.random.default_rng(1004).integers(256, 4097, size=64)
     attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged 256..4096 global", 64, 64, 8, 64, 4096, 0, True, lengths)
     attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged sliding 128", 64, 64, 8, 64, 4096, 128, True, lengths)
+    attention("gpt-oss shape B=64 64Q/8KV H=64 ctx 4096 fp8 global", 64, 64, 8, 64, 4096, 0, True)
+    attention("lyra-medium B=64 fp8 ragged 256..4096 global", 64, 32, 8, 128, 4096, 0, True, lengths)
+    attention("lyra-medium B=64 ctx 4096 fp8 global, one position per row", 64, 32, 8, 128, 4096, 0, True, np.full(64, 4096))
+    attention("lyra-max B=128 ctx 4096 fp8 global, one position per row", 128, 32, 8, 128, 4096, 0, True, np.full(128, 4096))
     for T in (1, 16, 64):
         s = zipf_group_sizes(rng, T, 31, 3, 1)
         gemm(f"lyra-medium expert up+SwiGLU T={T} (32x4096x8192 fp8)", int(s.sum()), 32, 4096, 8192, s, True, (4096, 1))

@@ -49,6 +49,7 @@ struct AttnParams {
 };
 
 constexpr int kTile = 32;
+constexpr int kMaxRankedRows = 256;  // batch rows the whole-row kernel can rank by length (one per thread)
 constexpr int kMergeStageFloats = 3 * 1024 + 16;  // LDS floats used when the last workgroup merges chunks
 
 // Visible key range of one batch row; bit-exact restatement of the mask
@@ -577,6 +578,197 @@ void decode_attention_kernel(AttnParams p) {
     }
 }
 
+// ---- whole rows, longest first ------------------------------------------------------------------
+// For launches with more (batch row, kv head) pairs than compute units and no sliding window.  One workgroup per compute
+// unit stays resident and works through several pairs, each from its first key to its last (no chunks, no merge across
+// workgroups).  With one position per batch row the rows are ranked by length first (descending, ties by row index) and
+// dealt out in serpentine order - workgroup w takes entries w, 2W-1-w, 2W+w, 4W-1-w, ... of the ranked list of pairs - so
+// every workgroup gets long and short rows in turn and all finish together; handed out in launch order instead, two long
+// rows that land on the same compute unit set the time of the launch (gpt-oss shape, lengths 256...4096: 39 us, of which
+// only 24 us are the average unit's share).  The first tile of the next pair is requested before the current pair's
+// wavefronts are merged, so a compute unit keeps streaming across pairs.
+template <int H, bool FP8>
+struct PairState {
+    Slab sl;
+    int b, kh, pos;
+    u32x4 q_raw;
+    float sink_raw;
+    uint16_t gate_raw;
+};
+
+template <int H, bool FP8, bool VEC4>
+__device__ __forceinline__ void request_pair(const AttnParams& p, int pair, bool live_pair, const int* sm_pos, const int* sm_order,
+                                             int tid, int lane, int wave, PairState<H, FP8>& st, RawK<H, FP8>& rk, RawS& rs,
+                                             RawV<H, FP8>& rv) {
+    constexpr int ES = FP8 ? 1 : 2;
+    const int x = lane & 15, kb = lane >> 4;
+    const int G = p.G;
+    const int row_rank = pair / p.K;
+    st.kh = pair - row_rank * p.K;
+    st.b = __builtin_amdgcn_readfirstlane(sm_order[row_rank]);
+    st.pos = __builtin_amdgcn_readfirstlane(sm_pos[st.b]);
+    const size_t head_row = ((size_t)st.b * p.K + st.kh) * p.S;
+    st.sl.k = make_rsrc(p.k + head_row * (H * ES), (uint32_t)p.S * (H * ES));
+    st.sl.v = make_rsrc(p.v + head_row * (H * ES), (uint32_t)p.S * (H * ES));
+    st.sl.ks = make_rsrc(FP8 ? p.ks + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
+    st.sl.vs = make_rsrc(FP8 ? p.vs + head_row : nullptr, FP8 ? (uint32_t)p.S * 4u : 0u);
+    st.sl.voff_k = x * (H * ES) + kb * 16;
+    st.sl.voff_v = 4 * kb * (H * ES) + x * (H * ES / 16);
+    st.sl.voff_s = 16 * kb;
+    // q, sinks and gates first (loads return in order), then this wavefront's first tile
+    const __amdgpu_buffer_rsrc_t qrsrc = make_rsrc(p.q + ((size_t)st.b * p.N + st.kh * G) * H, (uint32_t)(G * H * 2));
+    const int q_row = tid / (H / 8), q_piece = tid % (H / 8);
+    st.q_raw = __builtin_amdgcn_raw_buffer_load_b128(qrsrc, (q_row * H + q_piece * 8) * 2, 0, 0);
+    const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(p.sinks + st.kh * G, (uint32_t)(G * 4));
+    st.sink_raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(srsrc, x * 4, 0, 0));
+    const __amdgpu_buffer_rsrc_t grsrc =
+        make_rsrc(p.gate ? p.gate + (size_t)st.b * p.N + st.kh * G : nullptr, p.gate ? (uint32_t)(G * 2) : 0u);
+    st.gate_raw = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(grsrc, x * 2, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    const bool live = live_pair && wave * kTile <= min(st.pos, p.S - 1);
+    load_k<H, FP8>(rk, st.sl, wave * kTile, live);
+    if constexpr (FP8) load_s<VEC4>(rs, st.sl, wave * kTile, live);
+    load_v<H, FP8>(rv, st.sl, wave * kTile, live);
+}
+
+template <int H, bool FP8, bool VEC4, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4)))  // one workgroup per compute unit
+void decode_attention_rows_kernel(AttnParams p) {
+    constexpr int CB = H / 16;
+    constexpr int HP = H + 4;  // LDS row pitch of the merge buffer in floats
+    constexpr int QP = H + 8;  // LDS row pitch of q in bf16 elements
+    extern __shared__ float smem[];
+    __shared__ int sm_pos[kMaxRankedRows];
+    __shared__ int sm_order[kMaxRankedRows];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int x = lane & 15, kb = lane >> 4;
+    const int G = p.G;
+    const int n_pairs = p.B * p.K;
+    const int n_wg = gridDim.x;  // <= n_pairs
+
+    // rank the rows: thread t places row t
+    int mine = 0;
+    if (tid < p.B) {
+        mine = p.position[(size_t)tid * p.pos_stride];
+        sm_pos[tid] = mine;
+    }
+    __syncthreads();
+    if (tid < p.B) {
+        int rank = tid;
+        if (p.pos_stride != 0) {
+            rank = 0;
+            for (int j = 0; j < p.B; ++j) {
+                const int other = sm_pos[j];
+                rank += (other > mine) || (other == mine && j < tid);
+            }
+        }
+        sm_order[rank] = tid;
+    }
+    __syncthreads();
+
+    PairState<H, FP8> st;
+    RawK<H, FP8> rk;
+    RawS rs;
+    RawV<H, FP8> rv;
+    int round = 0;
+    request_pair<H, FP8, VEC4>(p, (int)blockIdx.x, true, sm_pos, sm_order, tid, lane, wave, st, rk, rs, rv);
+
+    uint16_t* sm_q = (uint16_t*)smem;
+    static_assert(WAVES * 64 >= 16 * (H / 8), "one q piece per thread");
+    const int q_row = tid / (H / 8), q_piece = tid % (H / 8);
+    for (;;) {
+        const Range rg = visible_range(st.pos, 0, p.S);
+        const int n_tiles = (rg.hi + kTile) / kTile;  // 0 when the position is negative: only the sink is attended
+        *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = st.q_raw;
+
+        Acc<H> acc;
+        const float sink2 = x < G ? st.sink_raw * kLog2e : 0.f;
+        acc.m = fmaxf(sink2, -1e30f);
+        acc.lsum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CB; ++c) acc.o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+
+        // same software pipeline as decode_attention_kernel: tiles wave, wave + WAVES, ... of the row
+        for (int tile = wave; tile < n_tiles; tile += WAVES) {
+            const int base = tile * kTile;
+            const int next = base + WAVES * kTile;
+            const bool more = tile + WAVES < n_tiles;
+            const bool full = base + kTile - 1 <= rg.hi;
+            f32x4 s[2];
+            tile_logits<H, FP8>(rk, sm_q, lane, s);
+            __builtin_amdgcn_sched_barrier(0);
+            load_k<H, FP8>(rk, st.sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+            uint32_t vis = 0;
+            bf16x8 pop;
+            if (full) pop = tile_softmax<H, FP8, false>(s, rs, base, 0, rg.hi, p.scale_log2, lane, acc, vis);
+            else pop = tile_softmax<H, FP8, true>(s, rs, base, 0, rg.hi, p.scale_log2, lane, acc, vis);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (FP8) load_s<VEC4>(rs, st.sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+            if (full) tile_values<H, FP8, false>(rv, pop, vis, acc);
+            else tile_values<H, FP8, true>(rv, pop, vis, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            load_v<H, FP8>(rv, st.sl, next, more);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        acc.lsum = group4_sum(acc.lsum);
+
+        // what the merge needs of the finished pair, then the requests of the next one (none after the last: the loads
+        // are still issued, with lane offsets that touch no memory, so both paths have the same loads in flight)
+        const int done_b = st.b, done_kh = st.kh;
+        const float done_gate = p.gate ? bf16_bits_to_f32(st.gate_raw) : 1.f;
+        ++round;
+        const int next_pair = round * n_wg + ((round & 1) ? n_wg - 1 - (int)blockIdx.x : (int)blockIdx.x);
+        const bool has_next = next_pair < n_pairs;
+        request_pair<H, FP8, VEC4>(p, has_next ? next_pair : 0, has_next, sm_pos, sm_order, tid, lane, wave, st, rk, rs, rv);
+
+        // ---- merge the wavefronts through LDS (as in decode_attention_kernel) ----
+        __syncthreads();  // everyone is done reading q
+        float* sm_o = smem;                   // [waves][G][HP]
+        float* sm_m = smem + WAVES * G * HP;  // [waves][16]
+        float* sm_l = sm_m + WAVES * 16;      // [waves][16]
+        float* sm_sink = sm_l + WAVES * 16;   // [16]
+        float* sm_gate = sm_sink + 16;        // [16]
+        if (wave == 0 && kb == 0 && x < G) {
+            sm_sink[x] = sink2;
+            sm_gate[x] = done_gate;
+        }
+        if (x < G) {
+            float* dst = sm_o + ((size_t)wave * G + x) * HP;
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dst[(4 * kb + r) * CB + c] = acc.o[c][r];
+            if (kb == 0) {
+                sm_m[wave * 16 + x] = acc.m;
+                sm_l[wave * 16 + x] = acc.lsum;
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < G * H; idx += WAVES * 64) {
+            const int g = idx / H, col = idx - g * H;
+            float mm = sm_m[g];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) mm = fmaxf(mm, sm_m[w * 16 + g]);
+            float o = 0.f, l = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const float f = fast_exp2(sm_m[w * 16 + g] - mm);
+                o += sm_o[((size_t)w * G + g) * HP + col] * f;
+                l += sm_l[w * 16 + g] * f;
+            }
+            const float den = l + fast_exp2(sm_sink[g] - mm);  // mm >= sink by construction
+            store_out(p, ((size_t)done_b * p.N + done_kh * G + g) * H + col, o / den, sm_gate[g]);
+        }
+        if (!has_next) break;
+        __syncthreads();  // the merge buffer has been read: q of the next pair may replace it
+    }
+}
+
 // ---- host side ---------------------------------------------------------------------------------
 struct AttnPlan {
     int chunk, n_chunks, waves;
@@ -706,6 +898,48 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
     const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
     const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
+    // Whole-row launch: more (row, kv head) pairs than compute units, no window.  LYRA_ATTN_ROWS=0 switches it off,
+    // =1 takes it only for one position per row (rows of different lengths), =2 also for a shared position;
+    // LYRA_ATTN_ROWS_WAVES (4 or 8) overrides the wavefront count.
+    static const char* rows_env = getenv("LYRA_ATTN_ROWS");
+    static const long rows_mode = rows_env ? atol(rows_env) : 1;
+    static const long rows_waves_env = env_long("LYRA_ATTN_ROWS_WAVES");
+    const bool rows = rows_mode > 0 && (position_stride == 1 || rows_mode > 1) && sliding_window == 0 && pl.n_chunks == 1 &&
+                      (long)B * K > 256 && B <= kMaxRankedRows;
+    if (rows) {
+        const int waves = (rows_waves_env == 4 || rows_waves_env == 8) ? (int)rows_waves_env : (H == 64 ? 8 : 4);
+        const size_t lds_need = std::max(((size_t)waves * G * (H + 4) + 2 * waves * 16 + 32) * sizeof(float),
+                                         (size_t)(waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t));
+        // more than half of a compute unit's 160 KB: one workgroup per unit
+        const size_t lds_r = std::max(lds_need, (size_t)81 * 1024);
+        const dim3 grid_r(256), block_r(waves * 64);
+#define LYRA_LAUNCH_ATTN_R(HH, F, V, W)                                                                        \
+    do {                                                                                                      \
+        auto kern = decode_attention_rows_kernel<HH, F, V, W>;                                                \
+        static const hipError_t attr =                                                                        \
+            hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                         \
+        hipLaunchKernelGGL(kern, grid_r, block_r, lds_r, st, p);                                              \
+    } while (0)
+#define LYRA_LAUNCH_ATTN_RW(HH, F, V)                    \
+    do {                                                 \
+        if (waves == 4) LYRA_LAUNCH_ATTN_R(HH, F, V, 4); \
+        else LYRA_LAUNCH_ATTN_R(HH, F, V, 8);            \
+    } while (0)
+        if (H == 128) {
+            if (!fp8) LYRA_LAUNCH_ATTN_RW(128, false, false);
+            else if (vec4) LYRA_LAUNCH_ATTN_RW(128, true, true);
+            else LYRA_LAUNCH_ATTN_RW(128, true, false);
+        } else {
+            if (!fp8) LYRA_LAUNCH_ATTN_RW(64, false, false);
+            else if (vec4) LYRA_LAUNCH_ATTN_RW(64, true, true);
+            else LYRA_LAUNCH_ATTN_RW(64, true, false);
+        }
+#undef LYRA_LAUNCH_ATTN_RW
+#undef LYRA_LAUNCH_ATTN_R
+        if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
+        return LYRA_OK;
+    }
 #define LYRA_LAUNCH_ATTN_W(HH, F, V, W)                                                                        \
     do {                                                                                                      \
         if (sliding_window == 0) hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, W, true, 1>), grid, block, lds, st, p); \

@@ -186,6 +186,27 @@ def test_config4_gpt_oss_shape_ragged_fp8_full_size():
     np.testing.assert_array_equal(got2, got1 * 2.0)
 
 
+@pytest.mark.parametrize("fp8,H,N,K,B", [(True, 64, 16, 8, 37), (False, 128, 8, 4, 70), (True, 128, 4, 2, 200), (True, 64, 2, 1, 256)])
+def test_ragged_rows_longest_first_launch(fp8, H, N, K, B):
+    """More (batch row, kv head) pairs than compute units with one position per row: the kernel hands rows out longest
+    first.  Equal lengths (rank ties), a row that sees only the sink (position -1), full rows, and the output gate."""
+    S = 384
+    case = U.attention_case(4000 + B, B, N, K, S, H, fp8=fp8)
+    rng = np.random.default_rng(B)
+    pos = rng.integers(0, S, B).astype(np.int32)
+    pos[: B // 4] = pos[B // 2 : B // 2 + B // 4]  # many ties
+    pos[1], pos[B - 1], pos[B // 3] = -1, S - 1, S - 1
+    gate = O.bf16_round((2.0 / (1.0 + np.exp(-rng.standard_normal((B, N))))).astype(np.float32))
+    _note(f"attn sorted fp8={fp8} H={H} N={N} K={K} B={B}")
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, pos)
+    got = _run(case, H**-0.5, 0, pos)
+    U.assert_close(got, want, what="ragged")
+    assert np.all(got[1] == 0)
+    got_g = _run(case, H**-0.5, 0, pos, gate=gate)
+    want_g = want * gate[:, :, None, None]
+    U.assert_close(got_g, want_g, what="ragged + gate")
+
+
 def test_headline_shape_b64_ctx4096_fp8():
     """B=64, ctx 4096, FP8 cache at the lyra-small shape (16Q/4KV/H=128), all rows full."""
     B, N, K, S, H = 64, 16, 4, 4096, 128
