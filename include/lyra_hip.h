@@ -49,7 +49,10 @@ const char* lyra_strerror(int code);
  *   sinks    [N] float32 learned sink logits (a virtual key with value 0)
  *   position int32; element b*position_stride is the index of the newest token of row b; keys
  *            0..position are visible (minus the window).  position_stride 0 = one scalar for the
- *            whole batch (the reference's only mode), 1 = ragged batch.
+ *            whole batch (the reference's only mode), 1 = ragged batch.  A ragged batch without a window and
+ *            with more than 256 (row, kv head) pairs (B <= 256) is worked through longest rows first by
+ *            resident workgroups; results do not depend on which launch is taken beyond float32
+ *            summation order.
  *   gate     [B,N] bf16 or NULL; out = bf16(bf16(attn) * gate)  (lyra/model.py:343-347)
  *   out      [B,N,H] out_dtype (bf16 or float32)
  *   sliding_window  0 = global layer; w > 0 = only keys j with position-w < j <= position
