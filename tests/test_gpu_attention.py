@@ -223,6 +223,25 @@ def test_headline_shape_b64_ctx4096_fp8():
     assert np.abs(got_p - got).max() <= 1e-2
 
 
+def test_config5_lyra_max_shape_b128_ctx4096_fp8():
+    """Benchmark configuration 5, the attention of one lyra-max layer: B=128, 32Q/8KV, H=128, ctx 4096, FP8 cache, global
+    and window 128; then the same batch with one position per row (the whole-row launch) against the shared position."""
+    B, N, K, S, H = 128, 32, 8, 4096, 128
+    case = U.attention_case(1005, B, N, K, S, H, fp8=True)
+    (kq, ks), (vq, vs) = case["k"], case["v"]
+    pos = np.full(B, S - 1, np.int32)
+    got0 = None
+    for sw in (0, 128):
+        _note(f"attn cfg5 sw={sw}")
+        want = clib.decode_attention(O.bf16_bits(case["q"]), kq, vq, ks[..., 0], vs[..., 0], case["sinks"], pos, None, H**-0.5, sw)
+        got = _run(case, H**-0.5, sw, S - 1)
+        U.assert_close(got, want, what=f"cfg5 sw={sw}")
+        if sw == 0:
+            got0 = got
+    got_rows = _run(case, H**-0.5, 0, pos)
+    assert np.abs(got_rows - got0).max() <= 1e-2
+
+
 def test_xla_path_and_dispatch_contract():
     from lyra_amd.kernels.decode_attention import decode_attention
 

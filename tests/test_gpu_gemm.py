@@ -151,6 +151,26 @@ def test_config3_moe_medium_shape_zipf_routing(T):
     U.assert_close(_run(down, False), _want(down, False, big=True), what="down")
 
 
+def test_config5_lyra_max_expert_shape_b128():
+    """Benchmark configuration 5, the expert matmuls of one lyra-max MoE layer at B=128: width 4096, 63 routed + 1 shared
+    expert, FP8 per-channel scales, top-(3+1) Zipf(1.1) routing: 512 rows, the shared expert holds 128 of them (two row
+    blocks)."""
+    C, Hd, E = 4096, 4096, 64
+    rng = np.random.default_rng(1005)
+    sizes = _zipf_routing(rng, 128, 63, 3, 1)
+    M = int(sizes.sum())
+    assert M == 512 and sizes[63] == 128
+    up = _case(15, M, E, C, 2 * Hd, sizes, kind="fp8", block=(C, 1))
+    _note(f"gemm cfg5 up M={M} touched={(sizes > 0).sum()}")
+    want_up = _want(up, True, big=True)
+    U.assert_close(_run(up, True), want_up, what="up+swiglu")
+    del up
+    down = _case(16, M, E, Hd, C, sizes, kind="fp8", block=(Hd, 1))
+    down["lhs"] = O.bf16_round(want_up)
+    _note("gemm cfg5 down")
+    U.assert_close(_run(down, False), _want(down, False, big=True), what="down")
+
+
 @pytest.mark.parametrize("kind,block", [("fp8", (512, 1)), ("fp8", (128, 128)), ("bf16", None)])
 def test_down_projection_with_many_units_takes_256_column_units(kind, block):
     """Without SwiGLU and with at least 1.75 rounds of 256-column units (here 34 row blocks x 16 = 544 for 256 workgroups)
