@@ -349,15 +349,43 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
         }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    // first row of every expert: thread e adds the counts of the experts before it (independent loads)
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
         int run = 0;
-        for (int e = 0; e < E; ++e) {
-            sm_start[e] = run;
-            run += sm_count[e];
+        for (int j = 0; j < e; ++j) run += sm_count[j];
+        sm_start[e] = run;
+        p.groups[e] = sm_count[e];
+    }
+    if (M <= (int)blockDim.x) {
+        // One assignment per thread.  Its rank among the assignments to the same expert = lanes below it in its wavefront
+        // with that expert (one ballot per distinct expert of the wavefront) + that expert's count in the wavefronts before.
+        const int i = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+        int* sm_wave_count = (int*)(sm_logits + (p.stage_logits ? p.tokens * p.n_routed : 0));  // [n_waves][E]
+        for (int j = threadIdx.x; j < n_waves * E; j += blockDim.x) sm_wave_count[j] = 0;
+        __syncthreads();
+        const int e = i < M ? sm_expert[i] : -1;
+        int rank = 0;
+        unsigned long long todo = __ballot(i < M);
+        while (todo) {  // same trip count for the whole wavefront
+            const int ev = __shfl(e, __ffsll((long long)todo) - 1, 64);
+            const unsigned long long same = __ballot(e == ev);
+            if (e == ev) {
+                const unsigned long long below = same & ((1ull << lane) - 1ull);
+                rank = __popcll(below);
+                if (below == 0ull) sm_wave_count[wave * E + ev] = __popcll(same);
+            }
+            todo &= ~same;
         }
+        __syncthreads();
+        if (i < M) {
+            for (int w = 0; w < wave; ++w) rank += sm_wave_count[w * E + e];
+            const int d = sm_start[e] + rank;
+            p.dest[i] = d;
+            p.row_map[d] = i / topk;
+        }
+        return;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < E; e += blockDim.x) p.groups[e] = sm_count[e];
     for (int i = threadIdx.x; i < M; i += blockDim.x) {
         const int e = sm_expert[i];
         int rank = 0;
@@ -713,13 +741,14 @@ extern "C" int lyra_moe_route(const float* logits, float* scores, int32_t* group
     if (tokens <= 0 || n_routed <= 0 || n_shared < 0 || k_routed <= 0) return LYRA_E_BADARG;
     if (k_routed > 8 || k_routed > n_routed || n_routed > 128) return LYRA_E_UNSUPPORTED;
     const int topk = k_routed + n_shared, E = n_routed + n_shared;
-    size_t lds = ((size_t)tokens * topk + 2 * E) * sizeof(int);
+    const int threads = std::min(1024, std::max(64, (tokens * topk + 63) / 64 * 64));
+    // assignments, counts and starts, per-wavefront expert counts of the ranking step
+    size_t lds = ((size_t)tokens * topk + 2 * E + (size_t)(threads / 64) * E) * sizeof(int);
     if (lds > 60000) return LYRA_E_UNSUPPORTED;
     const size_t staged = (size_t)tokens * n_routed * sizeof(float);
     const int stage = lds + staged <= 64000;
     if (stage) lds += staged;
     RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed, stage};
-    const int threads = std::min(1024, std::max(64, (tokens * topk + 63) / 64 * 64));
     hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }

@@ -151,7 +151,7 @@ def test_qkv_post_key_codes_bit_exact_at_position_zero():
 
 
 @pytest.mark.parametrize("T,n_routed,n_shared,k", [(64, 15, 1, 3), (5, 7, 1, 1), (128, 31, 1, 3), (33, 63, 1, 3), (16, 8, 0, 2), (1, 15, 1, 3),
-                                                   (256, 15, 1, 3)])
+                                                   (256, 15, 1, 3), (300, 15, 1, 3), (250, 127, 1, 3), (3, 128, 0, 8)])
 def test_moe_route(T, n_routed, n_shared, k):
     from lyra_amd.kernels import decode_fused as F
 
