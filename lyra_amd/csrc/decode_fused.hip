@@ -5,6 +5,8 @@
 #include <algorithm>
 #include <cstdlib>
 
+#include <climits>
+
 #include "lyra_device.h"
 
 namespace lyra {
@@ -298,6 +300,7 @@ struct RouteParams {
     int32_t* dest;        // [tokens * topk]: sorted row of each assignment (unpermute_map)
     int tokens, n_routed, n_shared, k_routed;
     int stage_logits;
+    int lanes;  // lanes that share the routing of one token: a power of two <= 16
 };
 
 __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
@@ -311,36 +314,60 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
     if (p.stage_logits)
         for (int i = threadIdx.x; i < p.tokens * p.n_routed; i += blockDim.x) sm_logits[i] = p.logits[i];
     __syncthreads();
-    for (int t = threadIdx.x; t < p.tokens; t += blockDim.x) {
+    // A token is routed by `lanes` neighbouring lanes (a power of two <= 16): each scans the experts sub, sub + lanes, ...
+    // for its best candidate, a butterfly of shuffles picks the largest value, on ties the lower index (lax.top_k).
+    const int lanes = p.lanes;
+    for (int base = 0; base < p.tokens * lanes; base += blockDim.x) {
+        const int gid = base + threadIdx.x;
+        const int t = min(gid / lanes, p.tokens - 1), sub = gid & (lanes - 1);
+        const bool owner = gid < p.tokens * lanes && sub == 0;
         const float* lg = (p.stage_logits ? sm_logits : p.logits) + (size_t)t * p.n_routed;
         float top[8];
         int idx[8];
         unsigned long long taken_lo = 0ull, taken_hi = 0ull;  // up to 128 routed experts
-        for (int j = 0; j < p.k_routed; ++j) {
+        // (loops over the 8 possible picks are unrolled with a guard, so that top[] and idx[] stay in registers)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j >= p.k_routed) break;
             float best = -INFINITY;
-            int bi = -1;
-            for (int e = 0; e < p.n_routed; ++e) {
+            int bi = INT_MAX;  // nothing found yet
+            for (int e = sub; e < p.n_routed; e += lanes) {
                 const bool used = e < 64 ? (taken_lo >> e) & 1ull : (taken_hi >> (e - 64)) & 1ull;
                 const float v = lg[e];
-                if (!used && (bi < 0 || v > best)) {  // strict >: ties go to the lower index (lax.top_k)
+                if (!used && (bi == INT_MAX || v > best)) {  // strict >: ties go to the lower index
                     best = v;
                     bi = e;
+                }
+            }
+            for (int off = lanes >> 1; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(best, off, 64);
+                const int oi = __shfl_xor(bi, off, 64);
+                if (oi != INT_MAX && (bi == INT_MAX || ov > best || (ov == best && oi < bi))) {
+                    best = ov;
+                    bi = oi;
                 }
             }
             if (bi < 64) taken_lo |= 1ull << bi; else taken_hi |= 1ull << (bi - 64);
             top[j] = best;
             idx[j] = bi;
         }
+        if (!owner) continue;
         float den = 0.f;
         const float top_max = top[0];
-        for (int j = 0; j < p.k_routed; ++j) {
-            top[j] = __expf(top[j] - top_max);
-            den += top[j];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j < p.k_routed) {
+                top[j] = __expf(top[j] - top_max);
+                den += top[j];
+            }
         }
-        for (int j = 0; j < p.k_routed; ++j) {
-            p.scores[(size_t)t * topk + j] = top[j] / den;
-            sm_expert[t * topk + j] = idx[j];
-            atomicAdd(&sm_count[idx[j]], 1);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j < p.k_routed) {
+                p.scores[(size_t)t * topk + j] = top[j] / den;
+                sm_expert[t * topk + j] = idx[j];
+                atomicAdd(&sm_count[idx[j]], 1);
+            }
         }
         for (int s = 0; s < p.n_shared; ++s) {
             p.scores[(size_t)t * topk + p.k_routed + s] = 1.f;  // model.py:476
@@ -741,14 +768,16 @@ extern "C" int lyra_moe_route(const float* logits, float* scores, int32_t* group
     if (tokens <= 0 || n_routed <= 0 || n_shared < 0 || k_routed <= 0) return LYRA_E_BADARG;
     if (k_routed > 8 || k_routed > n_routed || n_routed > 128) return LYRA_E_UNSUPPORTED;
     const int topk = k_routed + n_shared, E = n_routed + n_shared;
-    const int threads = std::min(1024, std::max(64, (tokens * topk + 63) / 64 * 64));
+    int lanes = 1;
+    while (lanes < 16 && 2 * lanes <= n_routed && (long)tokens * 2 * lanes <= 1024) lanes *= 2;
+    const int threads = std::min(1024, std::max(64, (std::max(tokens * topk, tokens * lanes) + 63) / 64 * 64));
     // assignments, counts and starts, per-wavefront expert counts of the ranking step
     size_t lds = ((size_t)tokens * topk + 2 * E + (size_t)(threads / 64) * E) * sizeof(int);
     if (lds > 60000) return LYRA_E_UNSUPPORTED;
     const size_t staged = (size_t)tokens * n_routed * sizeof(float);
     const int stage = lds + staged <= 64000;
     if (stage) lds += staged;
-    RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed, stage};
+    RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed, stage, lanes};
     hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
