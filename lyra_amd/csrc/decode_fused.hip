@@ -491,14 +491,20 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
     const int lo = c * p.chunk_len, hi = min(lo + p.chunk_len, p.cols);
     float bv = -INFINITY;
     int bi = 0x7FFFFFFF;
-    for (int i = lo + threadIdx.x * 4; i < hi; i += 1024) {  // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads
-        if (i + 4 <= hi) {
-            const f32x4 v = *(const f32x4*)(xr + i);
+    // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads, four of them in flight per thread; they go through a
+    // descriptor of the row's `cols` columns (loads past it return zeros) and columns at or past `hi` are not compared
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(xr), 0, (uint32_t)p.cols * 4u, 0x00020000);
+    for (int i0 = lo + threadIdx.x * 4; i0 < hi; i0 += 4096) {
+        u32x4 v[4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) take_better(bv, bi, v[k], i + k);
-        } else {
-            for (int k = 0; i + k < hi; ++k) take_better(bv, bi, xr[i + k], i + k);
-        }
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rr, (i0 + u * 1024) * 4, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = i0 + u * 1024 + k;
+                if (i < hi) take_better(bv, bi, __uint_as_float(v[u][k]), i);
+            }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
@@ -797,7 +803,8 @@ namespace lyra {
 // different shapes sharing one workspace never leave partial results where another call expects zeroed counters.
 constexpr size_t kArgmaxCounterBytes = 65536 * sizeof(int);
 static int argmax_chunks(int rows, int cols) {
-    const int want = std::max(1, 512 / std::max(1, rows));             // ~2 workgroups per compute unit
+    static const int wgs_env = [] { const char* e = getenv("LYRA_ARGMAX_WGS"); return e ? atoi(e) : 0; }();  // tuning override
+    const int want = std::max(1, (wgs_env > 0 ? wgs_env : 512) / std::max(1, rows));  // ~2 workgroups per compute unit
     const int most = std::max(1, (cols + 4095) / 4096);                // at least 4096 columns per workgroup
     return std::min(std::min(want, most), 64);
 }
@@ -812,7 +819,7 @@ extern "C" int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t
                            lyra_stream_t stream) {
     using namespace lyra;
     if (!x || !out || rows <= 0 || cols <= 0 || ld < cols) return LYRA_E_BADARG;
-    if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535) return LYRA_E_UNSUPPORTED;
+    if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535 || cols > (1 << 28)) return LYRA_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < lyra_argmax_workspace(rows, cols) || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
     ArgmaxParams p;
     p.x = x;
