@@ -207,6 +207,40 @@ def test_ragged_rows_longest_first_launch(fp8, H, N, K, B):
     U.assert_close(got_g, want_g, what="ragged + gate")
 
 
+def test_ragged_launch_replays_in_a_hip_graph():
+    """The whole-row launch captured in a HIP graph: replays follow the positions the caller updates in place between
+    them, and every replay equals the eager result for the same positions."""
+    from lyra_amd.kernels.decode_attention import decode_attention
+
+    B, N, K, S, H = 70, 8, 4, 384, 128
+    case = U.attention_case(4242, B, N, K, S, H, fp8=True)
+    q, k, v, sinks = U.attention_torch_inputs(case)
+    rng = np.random.default_rng(7)
+    pos = torch.from_numpy(rng.integers(0, S, B).astype(np.int32)).to(U.dev())
+    out_static = torch.empty_like(q)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        out_static.copy_(decode_attention(q, k, v, sinks, H**-0.5, 0, pos, implementation="pallas"))  # warm-up outside the graph
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static.copy_(decode_attention(q, k, v, sinks, H**-0.5, 0, pos, implementation="pallas"))
+    for rep in range(3):
+        new_pos = rng.integers(-1, S, B).astype(np.int32)
+        pos.copy_(torch.from_numpy(new_pos).to(U.dev()))
+        _note(f"attn ragged graph replay {rep}")
+        graph.replay()
+        torch.cuda.synchronize()
+        got = U.to_np(out_static)
+        eager = U.to_np(decode_attention(q, k, v, sinks, H**-0.5, 0, pos, implementation="pallas"))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(got, eager)
+        want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, new_pos)
+        U.assert_close(got, want, what=f"replay {rep}")
+
+
 def test_headline_shape_b64_ctx4096_fp8():
     """B=64, ctx 4096, FP8 cache at the lyra-small shape (16Q/4KV/H=128), all rows full."""
     B, N, K, S, H = 64, 16, 4, 4096, 128
