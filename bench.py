@@ -270,6 +270,14 @@ def kernel_table(dev, only=""):
         s = zipf_group_sizes(rng, B, 15, 3, 1)
         gemm(f"lyra-small expert up+SwiGLU B={B} (16x2048x4096 fp8)", int(s.sum()), 16, 2048, 4096, s, True, (2048, 1))
         gemm(f"lyra-small expert down B={B} (16x2048x2048 fp8)", int(s.sum()), 16, 2048, 2048, s, False, (2048, 1))
+    if only and "probe" in only:  # what the 64-row units of the shared expert cost: the same routing with a light shared expert
+        s = zipf_group_sizes(rng, 64, 15, 3, 1)
+        for shared_rows in (64, 32, 16):
+            t = s.copy()
+            t[15] = shared_rows
+            gemm(f"probe lyra-small expert up+SwiGLU B=64, shared expert {shared_rows} rows", int(t.sum()), 16, 2048, 4096, t, True, (2048, 1))
+            gemm(f"probe lyra-small expert down B=64, shared expert {shared_rows} rows", int(t.sum()), 16, 2048, 2048, t, False, (2048, 1))
+        print("rows per expert:", s.tolist(), file=sys.stderr)
     for name, K, N, sw in (("q/k/v", 2048, 3072, False), ("out", 2048, 2048, False), ("dense up+SwiGLU", 2048, 6144, True),
                            ("dense down", 3072, 2048, False)):
         gemm(f"lyra-small {name} projection B=64 ({K}x{N} fp8)", 64, 1, K, N, [64], sw, (K, 1))
