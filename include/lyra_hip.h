@@ -106,6 +106,12 @@ int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, i
                      int fused_swiglu, float swiglu_beta, float swiglu_limit, lyra_stream_t stream);
 
 size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu);
+/*
+ * Exact workspace bytes of a call whose weights carry scale blocks of bk rows (0 = bf16 weights or one scale per
+ * column): what lyra_decode_gemm(_ex) checks workspace_bytes against.  Never more than lyra_decode_gemm_workspace,
+ * which covers every scale block of the shape.
+ */
+size_t lyra_decode_gemm_workspace_for(int M, int G, int K, int N, int bk, int fused_swiglu);
 
 /*
  * lyra_decode_gemm with the two neighbouring model steps fused in (no counterpart kernel in the reference; the

@@ -25,6 +25,7 @@ SIGNATURES = {
         [_c.c_void_p] * 3 + [_c.c_int] * 2 + [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 7 + [_c.c_float] * 2 + [_c.c_void_p],
     ),
     "lyra_decode_gemm_workspace": (_c.c_size_t, [_c.c_int] * 5),
+    "lyra_decode_gemm_workspace_for": (_c.c_size_t, [_c.c_int] * 6),
     "lyra_decode_gemm_ex": (
         _c.c_int,
         [_c.c_void_p] * 4 + [_c.c_int] * 2 + [_c.c_void_p] * 3 + [_c.c_float, _c.c_int] + [_c.c_void_p] * 2 + [_c.c_size_t]
@@ -91,10 +92,12 @@ def check(code: int, what: str) -> None:
 
 
 _WORKSPACES: dict[tuple[str, int, int], "object"] = {}
+_SUPERSEDED: list = []  # outgrown buffers stay allocated: a captured HIP graph may still hold their address
 
 
 def workspace(kind: str, device, stream_ptr: int, nbytes: int):
-    """A reusable, zero-initialised device scratch buffer per (operator, device, stream); grows, never shrinks.
+    """A reusable, zero-initialised device scratch buffer per (operator, device, stream); grows, never shrinks, and a
+    buffer that a larger one replaces is never freed (graphs captured earlier replay against it).
 
     The attention kernel keeps arrival counters in it and returns them to zero, so it is zeroed only when
     allocated and never shared with another operator.
@@ -104,6 +107,8 @@ def workspace(kind: str, device, stream_ptr: int, nbytes: int):
     key = (kind, device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     buf = _WORKSPACES.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _SUPERSEDED.append(buf)
         buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _WORKSPACES[key] = buf
     return buf

@@ -374,7 +374,10 @@ void decode_attention_kernel(AttnParams p) {
     const Range rg = visible_range(pos, p.sw, p.S);
     const int c_lo = rg.start + c_idx * p.chunk;
     if (c_lo > rg.hi) {  // chunk holds no visible key (whole workgroup leaves together)
-        if (p.n_chunks == 1)  // position < 0: only the sink is attended and its value is 0
+        // First chunk empty = no chunk of this row holds a key (position < 0): only the sink is attended and its value is
+        // 0.  No workgroup of the row then reaches the merge, so the first one writes the zeros, however many chunks the
+        // launch has; the arrival counter is not touched and stays zero.
+        if (c_idx == 0)
             for (int idx = threadIdx.x; idx < G * H; idx += WAVES * 64)
                 store_out(p, ((size_t)b * p.N + kh * G) * H + idx, 0.f, 1.f);
         wait_all_memory();

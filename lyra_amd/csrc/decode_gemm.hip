@@ -1317,7 +1317,7 @@ struct GemmPlan {
 // split only as far as needed to fill 256 compute units.  Small ones (a few MB: the dense projections) are
 // latency bound, so they are cut into as many independent 16-row x 128-column x K-slice pieces as the
 // float32 partials allow, even though row tiles of one group then read the same weights through L2.
-static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) {
+static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, bool allow_split_k = true) {
     static const long target_env = [] {
         const char* e = getenv("LYRA_GEMM_TARGET_WGS");  // tuning override, read once
         return e ? atol(e) : 0L;
@@ -1341,7 +1341,7 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu) 
         pl.split_k = false;
         return pl;
     }
-    pl.split_k = G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && !no_split_k;
+    pl.split_k = allow_split_k && G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && !no_split_k;
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
         pl.mt = 4;
@@ -1447,14 +1447,30 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
 
 }  // namespace lyra
 
+namespace lyra {
+// Bytes of float32 partials (behind the counters) that the launch of `pl` writes.
+static size_t gemm_partial_bytes(const GemmPlan& pl, int M, int N) {
+    if (pl.grouped)  // one tile slot of 64 rows x 256 columns per workgroup
+        return (size_t)kGroupMaxWgs * 16 * kGroupTiles * 256 * sizeof(float);
+    if (pl.ksplit == 1 && !pl.split_k) return 0;
+    return ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+}
+}  // namespace lyra
+
 extern "C" size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu) {
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return 0;
-    // the split factor may depend on the scale block; size for the largest split the plan can choose
-    const lyra::GemmPlan pl = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu);
-    if (pl.grouped)  // one tile slot of 64 rows x 256 columns per workgroup, behind the counters
-        return lyra::kGemmCounterBytes + (size_t)lyra::kGroupMaxWgs * 16 * lyra::kGroupTiles * 256 * sizeof(float);
-    if (pl.ksplit == 1 && !pl.split_k) return lyra::kGemmCounterBytes;
-    return lyra::kGemmCounterBytes + ((size_t)pl.ksplit * M * N * sizeof(float) + 255) / 256 * 256;
+    // The scale block is not known here and decides both which kernel runs (a block that does not tile a K slice sends a
+    // small projection to the general kernel) and how many K slices it writes; a coarser block only ever lowers the slice
+    // count of either kernel, so the larger of the two plans without a block covers every block.
+    const lyra::GemmPlan with_split = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu, true);
+    const lyra::GemmPlan general = lyra::plan_gemm(M, G, K, N, 0, fused_swiglu, false);
+    return lyra::kGemmCounterBytes + std::max(lyra::gemm_partial_bytes(with_split, M, N), lyra::gemm_partial_bytes(general, M, N));
+}
+
+extern "C" size_t lyra_decode_gemm_workspace_for(int M, int G, int K, int N, int bk, int fused_swiglu) {
+    if (M <= 0 || G <= 0 || K <= 0 || N <= 0 || bk < 0) return 0;
+    const lyra::GemmPlan pl = lyra::plan_gemm(M, G, K, N, bk, fused_swiglu);
+    return lyra::kGemmCounterBytes + lyra::gemm_partial_bytes(pl, M, N);
 }
 
 extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
@@ -1527,7 +1543,8 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.arrivals = nullptr;
     if (pl.ksplit > 1 || pl.split_k || pl.grouped) {
         // the first kGemmCounterBytes belong to the grouped kernel's arrival counters, whichever kernel runs
-        const size_t need = lyra_decode_gemm_workspace(M, G, K, N, fused_swiglu);
+        // (checked against the plan that is launched: never more than lyra_decode_gemm_workspace answers for the shape)
+        const size_t need = kGemmCounterBytes + gemm_partial_bytes(pl, M, N);
         if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
         p.arrivals = (int*)workspace;
         p.part = (float*)((char*)workspace + kGemmCounterBytes);

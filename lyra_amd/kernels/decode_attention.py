@@ -18,6 +18,7 @@ from lyra_amd.nn.quant import QArray, dequantize, is_scaled
 _DECODE_BLOCK = 128  # lyra/kernels/decode_attention.py:29 (slab granularity of the plain path)
 _KERNEL_TILE = 32    # tokens per matrix-core tile in the HIP kernel
 _MAX_HEAD_GROUPS = 16
+_MAX_GRID_YZ = 65535
 
 
 @dataclass(frozen=True)
@@ -37,6 +38,8 @@ def select_decode_attention_config(
     sliding_window: int,
     out_dtype: torch.dtype,
     cache_dtype: torch.dtype | None = None,
+    batch: int = 1,
+    kv_heads: int = 1,
 ) -> DecodeAttentionConfig | None:
     """Support predicate of the HIP kernel (cf. decode_attention.py:41-60).
 
@@ -48,6 +51,8 @@ def select_decode_attention_config(
     if head_groups <= 0 or head_groups > _MAX_HEAD_GROUPS:
         return None
     if kv_len <= 0 or sliding_window < 0:
+        return None
+    if batch > _MAX_GRID_YZ or kv_heads > _MAX_GRID_YZ:  # batch rows and kv heads are grid dimensions of the launch
         return None
     if cache_dtype is not None and cache_dtype != torch.float8_e4m3fn:
         return None
@@ -213,7 +218,8 @@ def decode_attention(
     supported_layout = N % K == 0 and q.is_cuda
     config = (
         select_decode_attention_config(
-            head_dim=H, head_groups=HEAD_GROUPS, kv_len=S, sliding_window=sliding_window, out_dtype=dtype, cache_dtype=cache_dtype
+            head_dim=H, head_groups=HEAD_GROUPS, kv_len=S, sliding_window=sliding_window, out_dtype=dtype, cache_dtype=cache_dtype,
+            batch=B, kv_heads=K,
         )
         if supported_layout
         else None

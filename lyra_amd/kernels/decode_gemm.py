@@ -25,6 +25,9 @@ class DecodeGEMMConfig:
     fwd_dtype: torch.dtype | None = None
 
 
+_MAX_GROUPS = 8191  # the kernel's limit (LYRA_E_UNSUPPORTED beyond it)
+
+
 def _scale_layout_supported(k: int, n: int, block: tuple[int, int]) -> bool:
     bk, bn = block
     if bk <= 0 or bn <= 0 or k % bk or n % bn or bn & (bn - 1):
@@ -36,7 +39,7 @@ def _scale_layout_supported(k: int, n: int, block: tuple[int, int]) -> bool:
 
 def select_decode_gemm_config(m: int, groups: int, k: int, n: int, quant_dtype=None, block=None, fused_swiglu=False) -> DecodeGEMMConfig | None:
     """Support predicate of the HIP kernel (cf. decode_gemm.py:70-94)."""
-    if min(m, groups, k, n) <= 0:
+    if min(m, groups, k, n) <= 0 or groups > _MAX_GROUPS:
         return None
     quant_dtype = quant_dtype if quant_dtype is not None and is_scaled(quant_dtype) else None
     if k % 32 or n % 128 or (fused_swiglu and n % 256):

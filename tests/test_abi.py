@@ -82,3 +82,28 @@ def test_workspace_sizes_are_host_arithmetic():
     splits = L.lyra_decode_gemm_splits(64, 2048, 3072, 2048)
     assert splits >= 2 and L.lyra_decode_gemm_workspace(64, 1, 2048, 3072, 0) == 65536 + splits * 64 * 3072 * 4  # counters + K slices
     assert L.lyra_decode_gemm_splits(64, 2048, 100, 2048) == 0
+
+
+def test_matmul_workspace_covers_the_launched_plan_for_every_scale_block():
+    """lyra_decode_gemm_workspace does not know the scale block, which decides the kernel and its K slices: its answer
+    must cover the exact need for every block, including blocks that send a small projection to the general kernel."""
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    worse = 0
+    for M in (1, 16, 64, 128, 256, 300):
+        for K in (512, 2048, 4096, 8192, 12288):
+            for N in (512, 2048, 4096, 8192, 32768):
+                for swiglu in (0, 1):
+                    cover = L.lyra_decode_gemm_workspace(M, 1, K, N, swiglu)
+                    for bk in (0, 32, 96, 128, 256, 512, 1024, 2048, K):
+                        if bk and K % bk:
+                            continue
+                        need = L.lyra_decode_gemm_workspace_for(M, 1, K, N, bk, swiglu)
+                        assert need <= cover, (M, K, N, swiglu, bk, need, cover)
+                        worse += need > L.lyra_decode_gemm_workspace_for(M, 1, K, N, 0, swiglu)
+    assert worse > 0  # the sweep does contain blocks that need more than the plan without a block
+    # three shapes where the launched plan has more K slices than the K-split plan of the same shape
+    for (M, K, N, bk, slices) in ((16, 8192, 8192, 1024, 8), (128, 2048, 32768, 1024, 2), (16, 12288, 8192, 96, 32)):
+        assert L.lyra_decode_gemm_splits(M, K, N, bk) == 0
+        assert L.lyra_decode_gemm_workspace_for(M, 1, K, N, bk, 0) == 65536 + slices * M * N * 4

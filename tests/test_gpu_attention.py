@@ -152,6 +152,36 @@ def test_sink_extremes_and_no_visible_key():
     assert np.abs(got).max() == 0.0
 
 
+def test_row_without_visible_keys_in_a_chunked_launch_is_zero():
+    """Few (row, kv head) pairs and a long cache: the launch is cut into chunks and merged.  A row whose position is -1 has
+    no chunk with a key, so nobody reaches the merge: the output must still be written (zeros: the sink's value), and the
+    arrival counters must be left so that the next call works."""
+    from lyra_amd import _lib
+
+    B, N, K, S, H = 2, 16, 4, 4096, 128
+    assert _lib.lib.lyra_decode_attention_workspace(B, N, K, S, H, 0) > 256  # i.e. chunked
+    case = U.attention_case(77, B, N, K, S, H, fp8=True)
+    q, k, v, sinks = U.attention_torch_inputs(case)
+    L = _lib.lib
+    ws = torch.zeros(L.lyra_decode_attention_workspace(B, N, K, S, H, 0), dtype=torch.uint8, device=U.dev())
+    for pos in ([-1, 3000], [2500, -1], [4095, 4095]):
+        _note(f"attn chunked empty row pos={pos}")
+        out = torch.full((B, N, 1, H), float("nan"), dtype=torch.bfloat16, device=U.dev())
+        p = torch.tensor(pos, dtype=torch.int32, device=U.dev())
+        rc = L.lyra_decode_attention(q.data_ptr(), k.qval.data_ptr(), v.qval.data_ptr(), k.scale.data_ptr(), v.scale.data_ptr(),
+                                     sinks.data_ptr(), p.data_ptr(), 1, None, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                     B, N, K, S, H, H**-0.5, 0, _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "chunked empty row")
+        torch.cuda.synchronize()
+        got = U.to_np(out)
+        want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, np.array(pos))
+        for b in range(B):
+            if pos[b] < 0:
+                assert np.abs(got[b]).max() == 0.0
+        U.assert_close(got, want, what=f"pos={pos}")
+        assert int(ws[: 1 << 16].count_nonzero()) == 0
+
+
 def test_split_count_does_not_change_the_result():
     """Partition invariance of the log-sum-exp merge: same keys, different chunking (B changes the plan)."""
     N, K, S, H = 8, 2, 4096, 128

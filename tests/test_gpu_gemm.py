@@ -306,6 +306,20 @@ def test_long_k_slices_of_larger_projections(M, K, N, kind, block, swiglu):
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="long k slices")
 
 
+@pytest.mark.parametrize("M,K,N,block", [(16, 8192, 8192, (1024, 128)), (128, 2048, 32768, (1024, 256)), (16, 12288, 8192, (96, 128))])
+def test_scale_blocks_that_send_a_projection_to_the_general_kernel(M, K, N, block):
+    """One group of 48-160 MB whose scale blocks do not tile a K slice of the K-split kernel: the general kernel runs, with
+    more K slices than the K-split plan has; the workspace must be sized for the launch that runs."""
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    assert L.lyra_decode_gemm_splits(M, K, N, block[0]) == 0  # not the K-split kernel
+    assert L.lyra_decode_gemm_workspace_for(M, 1, K, N, block[0], 0) <= L.lyra_decode_gemm_workspace(M, 1, K, N, 0)
+    c = _case(12, M, 1, K, N, [M - 1], kind="fp8", block=block, bias=True, w_std=0.03)
+    _note(f"gemm general kernel with scale blocks M={M} K={K} N={N} block={block}")
+    U.assert_close(_run(c, False), _want(c, False, big=True), what="general kernel, blocks along K")
+
+
 @pytest.mark.parametrize("block,swiglu", [((256, 256), True), ((128, 128), False), ((512, 256), False), ((64, 128), True)])
 def test_many_experts_with_scale_blocks_along_k(block, swiglu):
     """Scale blocks shorter than K in the unit-list kernel: the accumulators are re-expressed whenever a wavefront's next
