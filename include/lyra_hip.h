@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 7
+#define LYRA_ABI_VERSION 8
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -30,6 +30,7 @@ extern "C" {
 #define LYRA_E_UNSUPPORTED (-2) /* a shape or dtype the kernels do not cover */
 #define LYRA_E_WORKSPACE (-3)   /* workspace pointer missing or too small */
 #define LYRA_E_LAUNCH (-4)      /* the HIP runtime refused the launch */
+#define LYRA_E_SCRATCH (-5)     /* lyra_decode_attention_static: the call needs more than the static scratch buffer */
 
 typedef void* lyra_stream_t; /* a hipStream_t; NULL = the default stream */
 
@@ -70,6 +71,26 @@ int lyra_decode_attention(const void* q, const void* k, const void* v, const flo
                           float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream);
 
 size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sliding_window);
+
+/*
+ * lyra_decode_attention for callers that cannot allocate device memory or hand over a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments, same kernels and bit-identical results as lyra_decode_attention, minus the workspace: split partials
+ * and arrival counters live in a device array of LYRA_STATIC_SCRATCH_BYTES that is part of the library's code object
+ * (every GPU the library runs on holds one copy until the process ends).  The call allocates and frees nothing; the
+ * first call on a device looks up the array's device address, so make that call outside a capture.  A launch that is
+ * not chunked (many (row, kv head) pairs, or a short window) does not touch the array.  A shape whose partials do not
+ * fit answers LYRA_E_SCRATCH and launches nothing: use lyra_decode_attention with a workspace for it.  The plan
+ * aims at about 256 workgroups per launch, so only launches with 16 query heads per kv head, head size 128 and
+ * close to 256 (row, kv head) pairs exceed the 4 MiB (lyra_decode_attention_workspace tells the need of a shape).
+ * All calls on one GPU share the array, and the counters a call uses are cleared at its start (a fill kernel on
+ * `stream`): calls that overlap on one GPU - different streams, or different host threads without ordering - race.
+ */
+#define LYRA_STATIC_SCRATCH_BYTES (4u << 20)
+int lyra_decode_attention_static(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                 const float* sinks, const int32_t* position, int position_stride, const void* gate,
+                                 void* out, int B, int N, int K, int S, int H, float sm_scale, int sliding_window,
+                                 int kv_dtype, int out_dtype, lyra_stream_t stream);
 
 /*
  * Zero `workspace_bytes` (a multiple of 4) of a workspace with a fill kernel on `stream` (safe to record

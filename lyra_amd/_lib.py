@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _c = ctypes
 SIGNATURES = {
@@ -19,6 +19,10 @@ SIGNATURES = {
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_workspace": (_c.c_size_t, [_c.c_int] * 6),
+    "lyra_decode_attention_static": (
+        _c.c_int,
+        [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 2 + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
     "lyra_workspace_init": (_c.c_int, [_c.c_void_p, _c.c_size_t, _c.c_void_p]),
     "lyra_decode_gemm": (
         _c.c_int,

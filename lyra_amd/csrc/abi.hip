@@ -117,6 +117,7 @@ extern "C" const char* lyra_strerror(int code) {
         case LYRA_E_UNSUPPORTED: return "shape or dtype not supported by the gfx950 kernels";
         case LYRA_E_WORKSPACE: return "workspace missing, misaligned or too small";
         case LYRA_E_LAUNCH: return "HIP runtime refused the kernel launch";
+        case LYRA_E_SCRATCH: return "the call needs more than the static scratch buffer (4 MiB): use the entry point that takes a workspace";
         default: return "unknown lyra error code";
     }
 }

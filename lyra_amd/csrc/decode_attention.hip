@@ -20,6 +20,7 @@
 // operand layout of the second, so probabilities never leave their lane.
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 #include "lyra_device.h"
 
@@ -847,12 +848,13 @@ extern "C" int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 
-extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale,
-                                     const float* v_scale, const float* sinks, const int32_t* position,
-                                     int position_stride, const void* gate, void* out, void* workspace,
-                                     size_t workspace_bytes, int B, int N, int K, int S, int H, float sm_scale,
-                                     int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
-    using namespace lyra;
+namespace lyra {
+// Validates and launches; shared by the entry point that takes the caller's workspace and the one that uses the static
+// scratch buffer.  too_small is what an insufficient workspace is reported as.
+static int run_attention(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                         const float* sinks, const int32_t* position, int position_stride, const void* gate, void* out,
+                         void* workspace, size_t workspace_bytes, int too_small, bool clear_counters, int B, int N, int K, int S,
+                         int H, float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
     if (!q || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || H <= 0 || N % K || sliding_window < 0) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
@@ -889,13 +891,20 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     p.arrivals = nullptr;
     if (pl.n_chunks > 1) {
         const AttnWorkspace w = attention_workspace(B, N, K, H, pl);
-        if (!workspace || workspace_bytes < w.total() || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
+        if (!workspace || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
+        if (workspace_bytes < w.total()) return too_small;
         p.arrivals = (int*)workspace;
         p.part_o = (float*)((char*)workspace + w.arrivals_bytes);
         p.part_ml = (float*)((char*)workspace + w.arrivals_bytes + w.o_bytes);
     }
 
     hipStream_t st = (hipStream_t)stream;
+    if (clear_counters && p.arrivals) {  // a fill kernel, not a memset node: safe to record into a graph
+        const size_t n = (size_t)B * K;
+        hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 64)), dim3(256), 0, st,
+                           (uint32_t*)p.arrivals, n);
+        if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
+    }
     const dim3 grid(pl.n_chunks, K, B), block(pl.waves * 64);
     const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16 + 32) * sizeof(float);
     const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
@@ -967,4 +976,50 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
 #undef LYRA_LAUNCH_ATTN_W
     if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
     return LYRA_OK;
+}
+
+// ---- static scratch for callers that cannot allocate -----------------------------------------------
+// One copy of this array lives on every GPU the library is loaded on, from load until the process ends.  Host code never
+// uses the array's name as an address: the device address is asked for once per device and kept.
+static __device__ __align__(256) unsigned char scratch[LYRA_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until first asked for
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device, or null if the runtime cannot tell.
+static void* static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace lyra
+
+extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale,
+                                     const float* v_scale, const float* sinks, const int32_t* position,
+                                     int position_stride, const void* gate, void* out, void* workspace,
+                                     size_t workspace_bytes, int B, int N, int K, int S, int H, float sm_scale,
+                                     int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
+    return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes,
+                               LYRA_E_WORKSPACE, false, B, N, K, S, H, sm_scale, sliding_window, kv_dtype, out_dtype, stream);
+}
+
+extern "C" int lyra_decode_attention_static(const void* q, const void* k, const void* v, const float* k_scale,
+                                            const float* v_scale, const float* sinks, const int32_t* position,
+                                            int position_stride, const void* gate, void* out, int B, int N, int K, int S, int H,
+                                            float sm_scale, int sliding_window, int kv_dtype, int out_dtype,
+                                            lyra_stream_t stream) {
+    if (!q || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
+    void* ptr = lyra::static_scratch();
+    if (!ptr) return LYRA_E_LAUNCH;
+    // the arrival counters this call uses are cleared first: the buffer keeps whatever the last call on this GPU left
+    return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, ptr,
+                               (size_t)LYRA_STATIC_SCRATCH_BYTES, LYRA_E_SCRATCH, true, B, N, K, S, H, sm_scale, sliding_window,
+                               kv_dtype, out_dtype, stream);
 }

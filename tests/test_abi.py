@@ -38,7 +38,7 @@ def test_abi_version_and_error_strings():
     text = open(HEADER).read()
     assert _lib.lib.lyra_abi_version() == int(re.search(r"#define LYRA_ABI_VERSION (\d+)", text).group(1)) == _lib.ABI_VERSION
     seen = set()
-    for code in (0, -1, -2, -3, -4):
+    for code in (0, -1, -2, -3, -4, -5):
         msg = _lib.lib.lyra_strerror(code).decode()
         assert msg and msg not in seen
         seen.add(msg)
