@@ -73,6 +73,23 @@ int lyra_decode_attention(const void* q, const void* k, const void* v, const flo
 size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sliding_window);
 
 /*
+ * lyra_decode_attention followed, in the same launch, by the model's learned exclusive self attention
+ * (lyra/model.py:351-363, enabled by use_learned_xsa, lyra/variants.py:38): after the output gate every query head n
+ * loses a learned share of its component along the new token's own value row,
+ *     out = t - tanh(xsa_alpha[n]) * <t, v^> * v^,     v^ = v_unit[b, n / (N/K), :]
+ *   v_unit    [B,K,H] bf16: the new token's value rows before cache quantisation, scaled to unit length
+ *             (lyra_qkv_post writes it)
+ *   xsa_alpha [N] float32
+ * Both NULL: exactly lyra_decode_attention.  A bf16 output is rounded wherever the JAX code holds a bf16 array (the
+ * products inside the inner product, the inner product, tanh(alpha), both products, the difference).
+ */
+int lyra_decode_attention_xsa(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                              const float* sinks, const int32_t* position, int position_stride, const void* gate,
+                              const void* v_unit, const float* xsa_alpha, void* out, void* workspace, size_t workspace_bytes,
+                              int B, int N, int K, int S, int H, float sm_scale, int sliding_window, int kv_dtype,
+                              int out_dtype, lyra_stream_t stream);
+
+/*
  * lyra_decode_attention for callers that cannot allocate device memory or hand over a workspace (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same arguments, same kernels and bit-identical results as lyra_decode_attention, minus the workspace: split partials
@@ -199,16 +216,18 @@ int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, const int32
  *   quantised with one scale per row, scale = amax/448 (1 for a zero row), code = e4m3fn_rne(clip(x/scale))
  *   (lyra/nn/quant.py:68-72, 213-231), scales into k_scale/v_scale [B,K,S].  Rows with position outside [0,S)
  *   are not appended.  H in {64,128}.
+ *   v_unit [B,K,H] bf16 or NULL: receives the new value rows scaled to unit length, bf16(v * rsqrt(sum(v^2) + 1e-10))
+ *   (model.py:353-354), which lyra_decode_attention_xsa takes.
  */
 int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,
                   const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache, float* k_scale,
-                  float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype, float eps,
+                  float* v_scale, void* v_unit, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype, float eps,
                   lyra_stream_t stream);
 /* Same, reading the projection as unsummed slices partials [splits, B, (N+2K)*H] float32 (qkv is ignored). */
 int lyra_qkv_post_sum(const void* qkv, const float* partials, int splits, const float* qnorm, const float* knorm,
                       const float* cos_t, const float* sin_t, const int32_t* position, int position_stride, void* q_out,
-                      void* k_cache, void* v_cache, float* k_scale, float* v_scale, int B, int N, int K, int S, int H,
-                      int rope_rows, int kv_dtype, float eps, lyra_stream_t stream);
+                      void* k_cache, void* v_cache, float* k_scale, float* v_scale, void* v_unit, int B, int N, int K, int S,
+                      int H, int rope_rows, int kv_dtype, float eps, lyra_stream_t stream);
 
 /*
  * lyra_moe_route: router top-k, softmax over the chosen logits, shared experts appended with score 1, and the stable

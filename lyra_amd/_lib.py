@@ -19,6 +19,10 @@ SIGNATURES = {
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_workspace": (_c.c_size_t, [_c.c_int] * 6),
+    "lyra_decode_attention_xsa": (
+        _c.c_int,
+        [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
     "lyra_decode_attention_static": (
         _c.c_int,
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 2 + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
@@ -38,7 +42,7 @@ SIGNATURES = {
     "lyra_rmsnorm_proj": (_c.c_int, [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p]),
     "lyra_qkv_post": (
         _c.c_int,
-        [_c.c_void_p] * 6 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
+        [_c.c_void_p] * 6 + [_c.c_int] + [_c.c_void_p] * 6 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
     ),
     "lyra_moe_route": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 4 + [_c.c_void_p]),
     "lyra_moe_combine": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 3 + [_c.c_float, _c.c_void_p]),
@@ -57,7 +61,7 @@ SIGNATURES = {
     ),
     "lyra_qkv_post_sum": (
         _c.c_int,
-        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
+        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] + [_c.c_void_p] * 6 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
     ),
     "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p]),
     "lyra_argmax_workspace": (_c.c_size_t, [_c.c_int] * 2),

@@ -47,6 +47,10 @@ struct AttnParams {
     int n_chunks;  // grid.x
     int out_f32;
     int scale_vec4;  // S % 4 == 0 -> scales are fetched as float4
+    // learned exclusive self attention (lyra/model.py:351-363), both null when the model has none
+    const uint16_t* xsa_v;   // [B,K,H] bf16: the new token's value rows scaled to unit length
+    const float* xsa_alpha;  // [N]
+    int xsa_lds;             // float offset of the staging area [G*H + 16] in dynamic LDS
 };
 
 constexpr int kTile = 32;
@@ -74,6 +78,44 @@ __device__ __forceinline__ void store_out(const AttnParams& p, size_t idx, float
     } else {
         if (p.gate) val = bf16_bits_to_f32(f32_to_bf16_bits(val)) * gate;
         ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(val);
+    }
+}
+
+// The value the output gate leaves, as the JAX code holds it: a bf16 output is rounded before and after the multiplication.
+__device__ __forceinline__ float gated(const AttnParams& p, float val, float gate) {
+    if (p.out_f32) return p.gate ? val * gate : val;
+    val = bf16_bits_to_f32(f32_to_bf16_bits(val));
+    return p.gate ? bf16_bits_to_f32(f32_to_bf16_bits(val * gate)) : val;
+}
+
+// Learned exclusive self attention on the G finished heads of one (batch row, kv head) (lyra/model.py:351-363):
+//   out = t - tanh(alpha_n) * <t, v^> * v^,   v^ = the new token's value row of this kv head at unit length.
+// sm_t [G*H] holds t after the gate (written by the caller, one element per thread and step), sm_coef [16] is scratch.
+// A bf16 output follows the dtype flow of the JAX code: the products inside the inner product, the inner product,
+// tanh(alpha), both products and the difference are each rounded to bf16; a float32 output rounds nowhere.
+// Every thread of the workgroup must call it (two barriers).
+template <int H>
+__device__ __forceinline__ void xsa_finish(const AttnParams& p, float* sm_t, float* sm_coef, int b, int kh, int tid, int threads) {
+    const int lane = tid & 63, wave = tid >> 6, waves = threads >> 6;
+    const int G = p.G;
+    const bool r16 = !p.out_f32;
+    auto rnd = [r16](float x) { return r16 ? bf16_bits_to_f32(f32_to_bf16_bits(x)) : x; };
+    const uint16_t* vn = p.xsa_v + ((size_t)b * p.K + kh) * H;
+    __syncthreads();
+    for (int g = wave; g < G; g += waves) {
+        float acc = 0.f;
+#pragma unroll
+        for (int c = lane; c < H; c += 64) acc += rnd(sm_t[g * H + c] * bf16_bits_to_f32(vn[c]));
+        acc = wave_sum(acc);
+        if (lane == 0) sm_coef[g] = rnd(rnd(tanhf(p.xsa_alpha[kh * G + g])) * rnd(acc));
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * H; idx += threads) {
+        const int g = idx / H, col = idx - g * H;
+        const float r = sm_t[idx] - rnd(sm_coef[g] * bf16_bits_to_f32(vn[col]));
+        const size_t o = ((size_t)b * p.N + kh * G + g) * H + col;
+        if (p.out_f32) ((float*)p.out)[o] = r;
+        else ((uint16_t*)p.out)[o] = f32_to_bf16_bits(r);
     }
 }
 
@@ -492,7 +534,8 @@ void decode_attention_kernel(AttnParams p) {
         const int n = kh * G + g;
         if (final_out) {
             const float den = l + fast_exp2(sm_sink[g] - mm);  // mm >= sink by construction
-            store_out(p, ((size_t)b * p.N + n) * H + col, o / den, sm_gate[g]);
+            if (p.xsa_v) smem[p.xsa_lds + idx] = gated(p, o / den, sm_gate[g]);
+            else store_out(p, ((size_t)b * p.N + n) * H + col, o / den, sm_gate[g]);
         } else {
             const size_t item = ((size_t)b * p.K + kh) * p.n_chunks + c_idx;
             store_agent(p.part_o + (item * G + g) * H + col, o);
@@ -502,7 +545,10 @@ void decode_attention_kernel(AttnParams p) {
             }
         }
     }
-    if (final_out) return;
+    if (final_out) {
+        if (p.xsa_v) xsa_finish<H>(p, smem + p.xsa_lds, smem + p.xsa_lds + G * H, b, kh, threadIdx.x, WAVES * 64);
+        return;
+    }
 
     // ---- merge the chunks: the workgroup that arrives last reads every partial of this kv head ----
     const int n_valid = min((rg.hi + 1 - rg.start + p.chunk - 1) / p.chunk, p.n_chunks);
@@ -559,8 +605,10 @@ void decode_attention_kernel(AttnParams p) {
                     if (c0 + u < n_valid) o += v[u] * sm_w[(c0 + u) * G + g];
             }
             const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
-            store_out(p, ((size_t)b * p.N + n) * H + col, o / sm_den[g], gate);
+            if (p.xsa_v) smem[p.xsa_lds + idx] = gated(p, o / sm_den[g], gate);
+            else store_out(p, ((size_t)b * p.N + n) * H + col, o / sm_den[g], gate);
         }
+        if (p.xsa_v) xsa_finish<H>(p, smem + p.xsa_lds, smem + p.xsa_lds + G * H, b, kh, threadIdx.x, WAVES * 64);
         return;
     }
     // more chunks than the staging area holds: plain per-thread loops (long contexts at tiny batch)
@@ -578,8 +626,10 @@ void decode_attention_kernel(AttnParams p) {
             o += load_agent(p.part_o + ((item0 + c) * G + g) * H + col) * f;
         }
         const float gate = p.gate ? bf16_bits_to_f32(p.gate[(size_t)b * p.N + n]) : 1.f;
-        store_out(p, ((size_t)b * p.N + n) * H + col, o / den, gate);
+        if (p.xsa_v) smem[p.xsa_lds + idx] = gated(p, o / den, gate);
+        else store_out(p, ((size_t)b * p.N + n) * H + col, o / den, gate);
     }
+    if (p.xsa_v) xsa_finish<H>(p, smem + p.xsa_lds, smem + p.xsa_lds + G * H, b, kh, threadIdx.x, WAVES * 64);
 }
 
 // ---- whole rows, longest first ------------------------------------------------------------------
@@ -766,8 +816,10 @@ void decode_attention_rows_kernel(AttnParams p) {
                 l += sm_l[w * 16 + g] * f;
             }
             const float den = l + fast_exp2(sm_sink[g] - mm);  // mm >= sink by construction
-            store_out(p, ((size_t)done_b * p.N + done_kh * G + g) * H + col, o / den, sm_gate[g]);
+            if (p.xsa_v) smem[p.xsa_lds + idx] = gated(p, o / den, sm_gate[g]);
+            else store_out(p, ((size_t)done_b * p.N + done_kh * G + g) * H + col, o / den, sm_gate[g]);
         }
+        if (p.xsa_v) xsa_finish<H>(p, smem + p.xsa_lds, smem + p.xsa_lds + G * H, done_b, done_kh, tid, WAVES * 64);
         if (!has_next) break;
         __syncthreads();  // the merge buffer has been read: q of the next pair may replace it
     }
@@ -853,11 +905,13 @@ namespace lyra {
 // scratch buffer.  too_small is what an insufficient workspace is reported as.
 static int run_attention(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                          const float* sinks, const int32_t* position, int position_stride, const void* gate, void* out,
-                         void* workspace, size_t workspace_bytes, int too_small, bool clear_counters, int B, int N, int K, int S,
-                         int H, float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
+                         void* workspace, size_t workspace_bytes, int too_small, bool clear_counters, const void* xsa_v,
+                         const float* xsa_alpha, int B, int N, int K, int S, int H, float sm_scale, int sliding_window,
+                         int kv_dtype, int out_dtype, lyra_stream_t stream) {
     if (!q || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || H <= 0 || N % K || sliding_window < 0) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
+    if ((xsa_v == nullptr) != (xsa_alpha == nullptr)) return LYRA_E_BADARG;
     if (kv_dtype != LYRA_DTYPE_BF16 && kv_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
     if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
     const bool fp8 = kv_dtype == LYRA_DTYPE_E4M3FN;
@@ -888,6 +942,9 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     p.out_f32 = out_dtype == LYRA_DTYPE_F32;
     const bool vec4 = (S % 4 == 0) && (((uintptr_t)k_scale | (uintptr_t)v_scale) % 16 == 0);
     p.scale_vec4 = vec4;
+    p.xsa_v = (const uint16_t*)xsa_v;
+    p.xsa_alpha = xsa_alpha;
+    p.xsa_lds = 0;
     p.arrivals = nullptr;
     if (pl.n_chunks > 1) {
         const AttnWorkspace w = attention_workspace(B, N, K, H, pl);
@@ -909,7 +966,10 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16 + 32) * sizeof(float);
     const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
     const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
-    const size_t lds = std::max(std::max(lds_merge, lds_q), lds_stage);
+    const size_t lds_xsa = xsa_v ? ((size_t)G * H + 16) * sizeof(float) : 0;  // staging area of the last step, behind the rest
+    const size_t lds_base = (std::max(std::max(lds_merge, lds_q), lds_stage) + 15) / 16 * 16;
+    const size_t lds = lds_base + lds_xsa;
+    p.xsa_lds = (int)(lds_base / sizeof(float));
     // Whole-row launch: more (row, kv head) pairs than compute units, no window.  LYRA_ATTN_ROWS=0 switches it off,
     // =1 takes it only for one position per row (rows of different lengths), =2 also for a shared position;
     // LYRA_ATTN_ROWS_WAVES (4 or 8) overrides the wavefront count.
@@ -923,7 +983,9 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
         const size_t lds_need = std::max(((size_t)waves * G * (H + 4) + 2 * waves * 16 + 32) * sizeof(float),
                                          (size_t)(waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t));
         // more than half of a compute unit's 160 KB: one workgroup per unit
-        const size_t lds_r = std::max(lds_need, (size_t)81 * 1024);
+        const size_t lds_need_x = (lds_need + 15) / 16 * 16;
+        p.xsa_lds = (int)(lds_need_x / sizeof(float));
+        const size_t lds_r = std::max(lds_need_x + lds_xsa, (size_t)81 * 1024);
         const dim3 grid_r(256), block_r(waves * 64);
 #define LYRA_LAUNCH_ATTN_R(HH, F, V, W)                                                                        \
     do {                                                                                                      \
@@ -1007,7 +1069,18 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
                                      size_t workspace_bytes, int B, int N, int K, int S, int H, float sm_scale,
                                      int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
     return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes,
-                               LYRA_E_WORKSPACE, false, B, N, K, S, H, sm_scale, sliding_window, kv_dtype, out_dtype, stream);
+                               LYRA_E_WORKSPACE, false, nullptr, nullptr, B, N, K, S, H, sm_scale, sliding_window, kv_dtype,
+                               out_dtype, stream);
+}
+
+extern "C" int lyra_decode_attention_xsa(const void* q, const void* k, const void* v, const float* k_scale,
+                                         const float* v_scale, const float* sinks, const int32_t* position,
+                                         int position_stride, const void* gate, const void* v_unit, const float* xsa_alpha,
+                                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
+                                         float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
+    return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes,
+                               LYRA_E_WORKSPACE, false, v_unit, xsa_alpha, B, N, K, S, H, sm_scale, sliding_window, kv_dtype,
+                               out_dtype, stream);
 }
 
 extern "C" int lyra_decode_attention_static(const void* q, const void* k, const void* v, const float* k_scale,
@@ -1020,6 +1093,6 @@ extern "C" int lyra_decode_attention_static(const void* q, const void* k, const 
     if (!ptr) return LYRA_E_LAUNCH;
     // the arrival counters this call uses are cleared first: the buffer keeps whatever the last call on this GPU left
     return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, ptr,
-                               (size_t)LYRA_STATIC_SCRATCH_BYTES, LYRA_E_SCRATCH, true, B, N, K, S, H, sm_scale, sliding_window,
-                               kv_dtype, out_dtype, stream);
+                               (size_t)LYRA_STATIC_SCRATCH_BYTES, LYRA_E_SCRATCH, true, nullptr, nullptr, B, N, K, S, H, sm_scale,
+                               sliding_window, kv_dtype, out_dtype, stream);
 }

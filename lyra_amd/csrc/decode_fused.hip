@@ -194,6 +194,7 @@ struct QkvPostParams {
     void* v_cache;
     float* k_scale;       // [B, K, S] or null (bf16 cache)
     float* v_scale;
+    uint16_t* v_unit;     // [B, K, H] or null: the new value rows scaled to unit length, bf16(v * rsqrt(sum v^2 + 1e-10))
     int B, N, K, S, H, seq;
     float eps;
     const float* partials;  // [splits, B, (N + 2K) * H] K slices of the projection not summed yet, or null (then qkv)
@@ -267,8 +268,16 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
         }
         return;
     }
-    if (pos < 0 || pos >= p.S) return;  // nothing to append outside the cache
     const int kh = is_k ? hd - p.N : hd - p.N - p.K;
+    if (!is_k && p.v_unit) {  // lyra/model.py:353-354: float32 sum of squares of the bf16 row, result held in bf16
+        const float inv = rsqrtf(wave_sum(a * a + c * c) + 1e-10f);
+        if (active) {
+            uint16_t* dst = p.v_unit + ((size_t)b * p.K + kh) * p.H;
+            dst[lane] = f32_to_bf16_bits(a * inv);
+            dst[lane + half] = f32_to_bf16_bits(c * inv);
+        }
+    }
+    if (pos < 0 || pos >= p.S) return;  // nothing to append outside the cache
     const size_t row = ((size_t)b * p.K + kh) * p.S + pos;
     void* cache = is_k ? p.k_cache : p.v_cache;
     float* scales = is_k ? p.k_scale : p.v_scale;
@@ -740,16 +749,16 @@ extern "C" int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, 
 
 extern "C" int lyra_qkv_post(const void* qkv, const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,
                              const int32_t* position, int position_stride, void* q_out, void* k_cache, void* v_cache,
-                             float* k_scale, float* v_scale, int B, int N, int K, int S, int H, int rope_rows, int kv_dtype,
-                             float eps, lyra_stream_t stream) {
+                             float* k_scale, float* v_scale, void* v_unit, int B, int N, int K, int S, int H, int rope_rows,
+                             int kv_dtype, float eps, lyra_stream_t stream) {
     return lyra_qkv_post_sum(qkv, nullptr, 0, qnorm, knorm, cos_t, sin_t, position, position_stride, q_out, k_cache, v_cache, k_scale,
-                             v_scale, B, N, K, S, H, rope_rows, kv_dtype, eps, stream);
+                             v_scale, v_unit, B, N, K, S, H, rope_rows, kv_dtype, eps, stream);
 }
 
 extern "C" int lyra_qkv_post_sum(const void* qkv, const float* partials, int splits, const float* qnorm, const float* knorm,
                                  const float* cos_t, const float* sin_t, const int32_t* position, int position_stride, void* q_out,
-                                 void* k_cache, void* v_cache, float* k_scale, float* v_scale, int B, int N, int K, int S, int H,
-                                 int rope_rows, int kv_dtype, float eps, lyra_stream_t stream) {
+                                 void* k_cache, void* v_cache, float* k_scale, float* v_scale, void* v_unit, int B, int N, int K,
+                                 int S, int H, int rope_rows, int kv_dtype, float eps, lyra_stream_t stream) {
     using namespace lyra;
     if (partials ? splits <= 0 : !qkv) return LYRA_E_BADARG;
     if (!cos_t || !sin_t || !position || !q_out || !k_cache || !v_cache) return LYRA_E_BADARG;
@@ -761,7 +770,7 @@ extern "C" int lyra_qkv_post_sum(const void* qkv, const float* partials, int spl
     if (fp8 != (k_scale != nullptr) || fp8 != (v_scale != nullptr)) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
     QkvPostParams p{(const uint16_t*)qkv, qnorm, knorm, cos_t, sin_t, position, position_stride, (uint16_t*)q_out,
-                    k_cache, v_cache, k_scale, v_scale, B, N, K, S, H, rope_rows, eps, partials, splits};
+                    k_cache, v_cache, k_scale, v_scale, (uint16_t*)v_unit, B, N, K, S, H, rope_rows, eps, partials, splits};
     const int items = B * (N + 2 * K);
     hipLaunchKernelGGL(qkv_post_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;

@@ -84,7 +84,8 @@ def _position_vector(position, batch: int, device) -> tuple[torch.Tensor, int]:
     return pos.reshape(batch).contiguous(), 1
 
 
-def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config: DecodeAttentionConfig, dtype, gate=None):
+def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config: DecodeAttentionConfig, dtype, gate=None,
+                      xsa_v=None, xsa_alpha=None):
     """Launch the HIP kernel (the counterpart of decode_attention.py:150-260)."""
     B, N, T, H = q.shape
     if T != 1:
@@ -121,15 +122,18 @@ def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config
     stream = torch.cuda.current_stream(dev).cuda_stream
     need = _lib.lib.lyra_decode_attention_workspace(B, N, K, S, H, int(sliding_window))
     ws = _lib.workspace("attention", dev, stream, need)
-    with torch.cuda.device(dev):
-        rc = _lib.lib.lyra_decode_attention(
-            q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(),
+    head = (q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(),
             k_scale.data_ptr() if quantized else None, v_scale.data_ptr() if quantized else None,
-            sinks_c.data_ptr(), pos.data_ptr(), stride, gate_c.data_ptr() if gate_c is not None else None,
-            out.data_ptr(), ws.data_ptr(), ws.numel(),
-            B, N, K, S, H, float(sm_scale), int(sliding_window), kv_dtype,
-            _lib.DTYPE_F32 if out_dtype == torch.float32 else _lib.DTYPE_BF16, stream,
-        )
+            sinks_c.data_ptr(), pos.data_ptr(), stride, gate_c.data_ptr() if gate_c is not None else None)
+    tail = (out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, float(sm_scale), int(sliding_window), kv_dtype,
+            _lib.DTYPE_F32 if out_dtype == torch.float32 else _lib.DTYPE_BF16, stream)
+    with torch.cuda.device(dev):
+        if xsa_v is not None:
+            vn = xsa_v.to(device=dev, dtype=torch.bfloat16).reshape(B, K, H).contiguous()
+            alpha = xsa_alpha.to(device=dev, dtype=torch.float32).reshape(N).contiguous()
+            rc = _lib.lib.lyra_decode_attention_xsa(*head, vn.data_ptr(), alpha.data_ptr(), *tail)
+        else:
+            rc = _lib.lib.lyra_decode_attention(*head, *tail)
     _lib.check(rc, "lyra_decode_attention")
     return out if out.dtype == dtype else out.to(dtype)
 
@@ -165,6 +169,17 @@ def _reference_rows(q, k, v, sinks, sm_scale, sliding_window, pos: int, dtype):
     a = unnormalized * normalizer
     out = torch.einsum("bkgts,bksh->bkgth", a, v.to(torch.float32))
     return out.to(dtype).reshape(B, N, T, H)
+
+
+def xsa_reference(t, unit_v, xsa_alpha, dtype):
+    """lyra/model.py:355-360 on t [B,N,1,H] (after the gate), unit_v [B,K,H] (the new value rows at unit length)."""
+    B, N, T, H = t.shape
+    K = unit_v.shape[1]
+    t_g = t.to(dtype).reshape(B, K, N // K, T, H)
+    vn_g = unit_v.to(dtype)[:, :, None, None, :]
+    coef = (t_g * vn_g).to(torch.float32).sum(dim=-1, keepdim=True)
+    alpha = torch.tanh(xsa_alpha.to(torch.float32)).reshape(1, K, N // K, 1, 1).to(dtype)
+    return (t_g - alpha * coef.to(dtype) * vn_g).reshape(B, N, T, H)
 
 
 def decode_attention_reference(q, k, v, sinks, sm_scale, sliding_window, position, dtype=None, gate=None):
@@ -204,8 +219,13 @@ def decode_attention(
     dtype: torch.dtype | None = None,
     implementation: Implementation = "auto",
     gate: torch.Tensor | None = None,
+    xsa_v: torch.Tensor | None = None,
+    xsa_alpha: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """q [B,N,1,H]; k, v [B,K,S,H] tensors or QArray (e4m3fn, block (1,H)); sinks [N]; returns [B,N,1,H].
+
+    ``xsa_v`` [B,K,H] (the new token's value rows at unit length) with ``xsa_alpha`` [N] fuses the learned exclusive
+    self attention of lyra/model.py:351-363 behind the gate; both default to None (the reference operator).
 
     Deliberate divergence from the reference: ``"auto"`` selects the kernel when the shape is
     supported (the reference's auto always takes XLA for this op, decode_attention.py:408).
@@ -225,12 +245,17 @@ def decode_attention(
         else None
     )
 
+    if (xsa_v is None) != (xsa_alpha is None):
+        raise ValueError("xsa_v and xsa_alpha go together")
+
     def reference():
-        return decode_attention_reference(q, k, v, sinks, sm_scale, sliding_window, position, dtype, gate=gate)
+        t = decode_attention_reference(q, k, v, sinks, sm_scale, sliding_window, position, dtype, gate=gate)
+        return t if xsa_v is None else xsa_reference(t, xsa_v, xsa_alpha, dtype)
 
     def kernel():
         assert config is not None
-        return _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config, dtype, gate=gate)
+        return _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config, dtype, gate=gate,
+                                 xsa_v=xsa_v, xsa_alpha=xsa_alpha)
 
     tiling = None if config is None else f"kv{config.tile_kv} buf{config.kv_buffer_count} {'fp8' if config.cache_dtype else 'bf16'}"
     op_shape = f"b{B} n{N} k{K} s{S} h{H} sw{sliding_window}"

@@ -140,10 +140,11 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
 
 
 def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
-             n_heads: int, n_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
+             n_heads: int, n_kv_heads: int, head_dim: int, eps: float, unit_v: bool = False):
     """QK norm + rotary embedding + KV-cache append (quantising for an FP8 cache) for one new token per sequence
     (lyra/model.py:309-336); ``pos`` is an int32 device scalar or a [B] tensor.  Returns q [B,N,H] bf16; the caches
-    are updated in place."""
+    are updated in place.  ``unit_v``: also return the new value rows scaled to unit length [B,K,H] bf16
+    (model.py:353-354), as (q, v_unit)."""
     N, K, H = n_heads, n_kv_heads, head_dim
     unsummed = isinstance(qkv, Unsummed)
     if unsummed:  # the projection arrives as K slices; they are summed while reading
@@ -167,13 +168,14 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
         S = kq.shape[2]
         assert kq.dtype == torch.bfloat16
     assert kq.is_contiguous() and vq.is_contiguous() and tuple(kq.shape) == (B, K, S, H)
+    vn = torch.empty((B, K, H), dtype=torch.bfloat16, device=dev) if unit_v else None
     rc = _L.lyra_qkv_post_sum(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None, splits if unsummed else 0,
                               _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(), _f32(sin_t).data_ptr(), pos.data_ptr(),
                               0 if pos.numel() == 1 else 1, q.data_ptr(), kq.data_ptr(), vq.data_ptr(), _ptr(ks), _ptr(vs),
-                              B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
+                              _ptr(vn), B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
                               _stream(dev))
     _lib.check(rc, "lyra_qkv_post_sum")
-    return q
+    return (q, vn) if unit_v else q
 
 
 def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,

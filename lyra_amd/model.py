@@ -53,6 +53,10 @@ class ModelConfig:
     sliding_window: int = 128
     use_qk_norm: bool = True
     use_sdpa_output_gate: bool = False
+    use_learned_xsa: bool = False
+    use_qkv_bias: bool = False
+    use_attn_out_bias: bool = False
+    use_mlp_bias: bool = False
     mlp_map: tuple[str, ...] = ()
     n_routed_experts: int = 15
     n_shared_experts: int = 1
@@ -111,10 +115,16 @@ lyra_dev = ModelConfig(name="Lyra Dev", seq_len=256, n_embd=256, n_layers=4, n_a
                        mlp_map=interleaved_moe(layers=4, first=2, every=2))
 lyra_small = ModelConfig(name="Lyra Small", use_sdpa_output_gate=True, mlp_map=interleaved_moe(layers=16, every=4, first=4))
 lyra_medium = ModelConfig(name="Lyra Medium", n_embd=4096, n_layers=32, tie_embeddings=False, n_attn_heads=32, n_kv_heads=8,
-                          use_sdpa_output_gate=True, mlp_map=interleaved_moe(32, first=4, every=4), n_routed_experts=31)
+                          use_sdpa_output_gate=True, use_learned_xsa=True, mlp_map=interleaved_moe(32, first=4, every=4),
+                          n_routed_experts=31)
 lyra_max = replace(lyra_medium, name="Lyra Max", mlp_map=moe_outer_dense(32, start_dense=2), n_routed_experts=63,
                    dense_mlp_widening=4.0)
-MODEL_VARIANTS = {"dev": lyra_dev, "lyra-small": lyra_small, "lyra-medium": lyra_medium, "lyra-max": lyra_max}
+# lyra/variants.py:62-80: every layer an expert layer, no shared expert, no QK norm, biases on every projection, YaRN
+gpt_oss_20b = ModelConfig(name="GPT-OSS 20B", rope_scale=32.0, n_embd=2880, n_layers=24, head_dim=64, n_attn_heads=64,
+                          n_kv_heads=8, mlp_map=("moe",) * 24, n_routed_experts=32, n_shared_experts=0, n_active_experts=4,
+                          tie_embeddings=False, use_qk_norm=False, use_qkv_bias=True, use_attn_out_bias=True, use_mlp_bias=True)
+MODEL_VARIANTS = {"dev": lyra_dev, "lyra-small": lyra_small, "lyra-medium": lyra_medium, "lyra-max": lyra_max,
+                  "gpt-oss-20b": gpt_oss_20b}
 
 
 def apply_inference_overrides(cfg: ModelConfig, *, fp8: bool = False, fp8_attn: bool = False, per_channel: bool = False) -> ModelConfig:
@@ -173,6 +183,9 @@ class AttentionWeights:
     qnorm_scale: torch.Tensor | None
     knorm_scale: torch.Tensor | None
     sdpa_gate: torch.Tensor | None  # [C, N] f32
+    xsa_alpha: torch.Tensor | None = None  # [N] f32 (use_learned_xsa, model.py:269)
+    qkv_bias: torch.Tensor | None = None   # [(N + 2K) H] f32: q, k and v biases side by side (use_qkv_bias, model.py:258-262)
+    out_bias: torch.Tensor | None = None   # [C] f32 (use_attn_out_bias)
 
 
 @dataclass
@@ -182,6 +195,8 @@ class MoEWeights:
     mlp_up: torch.Tensor | QArray   # [E, C, 2*hidden]   (gate half first: lyra/model.py:494-495)
     mlp_down: torch.Tensor | QArray  # [E, hidden, C]
     norm_scale: torch.Tensor
+    mlp_up_bias: torch.Tensor | None = None    # [E, 2*hidden] f32 (use_mlp_bias, model.py:399-402)
+    mlp_down_bias: torch.Tensor | None = None  # [E, C] f32
 
 
 @dataclass
@@ -189,6 +204,8 @@ class DenseMLPWeights:
     mlp_up: torch.Tensor | QArray    # [1, C, 2*hidden]
     mlp_down: torch.Tensor | QArray  # [1, hidden, C]
     norm_scale: torch.Tensor
+    mlp_up_bias: torch.Tensor | None = None    # [1, 2*hidden] f32
+    mlp_down_bias: torch.Tensor | None = None  # [1, C] f32
 
 
 @dataclass
@@ -238,6 +255,9 @@ def init_weights(cfg: ModelConfig, device, seed: int | None = None) -> ModelWeig
             qnorm_scale=ones(H) if cfg.use_qk_norm else None,
             knorm_scale=ones(H) if cfg.use_qk_norm else None,
             sdpa_gate=rnd(C, N, dtype=torch.float32) if cfg.use_sdpa_output_gate else None,
+            xsa_alpha=rnd(N, std=1.0, dtype=torch.float32) if cfg.use_learned_xsa else None,
+            qkv_bias=rnd((N + 2 * K) * H, std=0.5, dtype=torch.float32) if cfg.use_qkv_bias else None,
+            out_bias=rnd(C, std=0.5, dtype=torch.float32) if cfg.use_attn_out_bias else None,
         )
         if cfg.mlp_map[idx] == "moe":
             E, Hd = cfg.n_experts, cfg.expert_hidden
@@ -247,6 +267,8 @@ def init_weights(cfg: ModelConfig, device, seed: int | None = None) -> ModelWeig
                 mlp_up=_maybe_quantize(rnd(E, C, 2 * Hd), cfg, cfg.quantize_mlp),
                 mlp_down=_maybe_quantize(rnd(E, Hd, C), cfg, cfg.quantize_mlp),
                 norm_scale=ones(C),
+                mlp_up_bias=rnd(E, 2 * Hd, std=0.5, dtype=torch.float32) if cfg.use_mlp_bias else None,
+                mlp_down_bias=rnd(E, C, std=0.5, dtype=torch.float32) if cfg.use_mlp_bias else None,
             )
         else:
             Hd = cfg.dense_hidden
@@ -254,6 +276,8 @@ def init_weights(cfg: ModelConfig, device, seed: int | None = None) -> ModelWeig
                 mlp_up=_maybe_quantize(rnd(1, C, 2 * Hd), cfg, cfg.quantize_mlp),
                 mlp_down=_maybe_quantize(rnd(1, Hd, C), cfg, cfg.quantize_mlp),
                 norm_scale=ones(C),
+                mlp_up_bias=rnd(1, 2 * Hd, std=0.5, dtype=torch.float32) if cfg.use_mlp_bias else None,
+                mlp_down_bias=rnd(1, C, std=0.5, dtype=torch.float32) if cfg.use_mlp_bias else None,
             )
         layers.append(LayerWeights(attn=attn, mlp=mlp))
     emb = rnd(cfg.padded_vocab_size, C)
@@ -304,12 +328,12 @@ def cache_update(cache: LayerCache, k: torch.Tensor, v: torch.Tensor, pos: torch
 
 
 # ---- layers ------------------------------------------------------------------------------------------
-def _dense(x: torch.Tensor, w, cfg: ModelConfig, *, fused_swiglu=False, out_f32=False) -> torch.Tensor:
+def _dense(x: torch.Tensor, w, cfg: ModelConfig, *, fused_swiglu=False, out_f32=False, bias=None) -> torch.Tensor:
     """quant.dot for a [B, C] activation (lyra/nn/quant.py:106-108) = the one-group decode matmul."""
     gmm = gmm_op(cfg.mode, cfg.implementation)
     sizes = torch.full((1,), x.shape[0], dtype=torch.int32, device=x.device)
     lhs = x.to(torch.float32) if out_f32 else x
-    return gmm(lhs, w, sizes, fused_swiglu=fused_swiglu, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
+    return gmm(lhs, w, sizes, bias=bias, fused_swiglu=fused_swiglu, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
                quant_dtype=cfg.gemm_dtype if isinstance(w, QArray) else None)
 
 
@@ -319,6 +343,8 @@ def attention_apply(x, w: AttentionWeights, idx: int, pos, cos, sin, cache: Laye
     H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
     h = rms_norm(x, w.norm_scale, cfg.norm_eps)
     qkv = _dense(h, w.qkv, cfg)
+    if w.qkv_bias is not None:  # :310-313, bf16 array + bf16 bias
+        qkv = qkv + w.qkv_bias.to(qkv.dtype)
     q, k, v = qkv.split([N * H, K * H, K * H], dim=-1)
     q, k, v = q.reshape(B, N, H), k.reshape(B, K, H), v.reshape(B, K, H)
     if w.qnorm_scale is not None and w.knorm_scale is not None:
@@ -331,8 +357,14 @@ def attention_apply(x, w: AttentionWeights, idx: int, pos, cos, sin, cache: Laye
     if w.sdpa_gate is not None:  # :343-347, fused into the attention epilogue
         gate = (2.0 * torch.sigmoid(h.to(torch.float32) @ w.sdpa_gate)).to(x.dtype)
     attn = attn_op(cfg.mode, cfg.implementation)
-    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate)
+    xsa_v = None
+    if w.xsa_alpha is not None:  # :353-354: the new token's value rows (not their cached, quantised copy) at unit length
+        v32 = v.to(torch.float32)
+        xsa_v = (v32 * torch.rsqrt(v32.pow(2).sum(dim=-1, keepdim=True) + 1e-10)).to(x.dtype)
+    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v, xsa_alpha=w.xsa_alpha)
     t = _dense(t.reshape(B, N * H), w.out, cfg)
+    if w.out_bias is not None:  # :367-368
+        t = t + w.out_bias.to(t.dtype)
     t = t * cfg.residual_scale
     return (x + t).to(x.dtype), cache
 
@@ -376,8 +408,10 @@ def moe_apply(x, w: MoEWeights, cfg: ModelConfig):
     permute_map, unpermute_map = bpermute(active_map)
     t = xn[permute_map // topk]
     qd = cfg.gemm_dtype if isinstance(w.mlp_up, QArray) else None
-    t = gmm(t, w.mlp_up, groups, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, quant_dtype=qd)
-    t = gmm(t, w.mlp_down, groups, quant_dtype=qd)
+    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32)  # acast(bias, compute_dtype), :527-528
+    t = gmm(t, w.mlp_up, groups, bias=bf(w.mlp_up_bias), fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
+            swiglu_limit=cfg.swiglu_limit, quant_dtype=qd)
+    t = gmm(t, w.mlp_down, groups, bias=bf(w.mlp_down_bias), quant_dtype=qd)
     t = torch.einsum("fkc,fk->fc", t[unpermute_map].reshape(B, topk, C).to(torch.float32), scores).to(x.dtype)  # :557
     t = t * cfg.residual_scale
     return x + t
@@ -386,8 +420,11 @@ def moe_apply(x, w: MoEWeights, cfg: ModelConfig):
 def dense_mlp_apply(x, w: DenseMLPWeights, cfg: ModelConfig):
     """lyra/model.py:608-636 (SwiGLU fused into the up projection's epilogue)."""
     t = rms_norm(x, w.norm_scale, cfg.norm_eps)
-    t = _dense(t, w.mlp_up, cfg, fused_swiglu=True)
+    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32)
+    t = _dense(t, w.mlp_up, cfg, fused_swiglu=True, bias=bf(w.mlp_up_bias))
     t = _dense(t, w.mlp_down, cfg)
+    if w.mlp_down_bias is not None:  # :629-630
+        t = t + w.mlp_down_bias[0].to(t.dtype)
     t = t * cfg.dense_residual_scale
     return (x + t).to(x.dtype)
 
@@ -420,10 +457,15 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     qkv = F.gemm_unsummed(h, w.qkv, one)
     if qkv is None:
         qkv = F.gemm(h, w.qkv, one)
-    q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps)
+    q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps,
+                   unit_v=w.xsa_alpha is not None)
+    xsa_v = None
+    if w.xsa_alpha is not None:  # the attention launch finishes with the exclusive-self-attention step (:351-363)
+        q, xsa_v = q
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     attn = attn_op(cfg.mode, cfg.implementation)
-    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate).reshape(B, N * H)
+    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
+             xsa_alpha=w.xsa_alpha).reshape(B, N * H)
     out = F.gemm_unsummed(t, w.out, one)
     if out is None:
         return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache
@@ -471,6 +513,8 @@ def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
     """Shapes the fused launches cover (the matmul kernel's: K % 32, N % 128, N % 256 with SwiGLU)."""
     if not (cfg.fused_glue and cfg.implementation != "xla" and model.emb.is_cuda):
         return False
+    if cfg.use_qkv_bias or cfg.use_attn_out_bias or cfg.use_mlp_bias:  # the fused launches between the operators carry no biases
+        return False
     C, H = cfg.n_embd, cfg.head_dim
     widths_ok = C % 128 == 0 and ((cfg.n_attn_heads + 2 * cfg.n_kv_heads) * H) % 128 == 0 and (cfg.n_attn_heads * H) % 32 == 0
     hidden = [cfg.dense_hidden] + ([cfg.expert_hidden] if "moe" in cfg.mlp_map else [])
@@ -478,7 +522,7 @@ def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
             and cfg.n_active_routed_experts <= 8 and cfg.padded_vocab_size % 128 == 0)
 
 
-def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig):
+def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None):
     from lyra_amd.kernels import decode_fused as F
 
     h = model.emb[tokens]
@@ -487,7 +531,10 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
         h = moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
-    h = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)[0]
+    normed = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)
+    if hidden_out is not None:  # the residual stream after the last layer (the norm kernel completes it on its way)
+        hidden_out.append(normed[2] if len(normed) > 2 else h)
+    h = normed[0]
     logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
     if model.vocab_mask is None:
         logits[:, cfg.vocab_size :] = float("-inf")
@@ -495,10 +542,11 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     return logits, cache
 
 
-def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig):
-    """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one)."""
+def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None):
+    """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one).
+    ``hidden_out``: optional list that receives the residual stream after the last layer [B, C] (for parity checks)."""
     if _fused_supported(model, cfg):
-        return model_apply_fused(tokens, model, cache, cfg)
+        return model_apply_fused(tokens, model, cache, cfg, hidden_out)
     h = model.emb[tokens].to(torch.bfloat16)
     cos_t, sin_t = _rope_tables(cfg, h.device)
     pos = cache.pos
@@ -506,6 +554,8 @@ def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cf
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply(h, layer.attn, idx, pos, cos, sin, cache.layers[idx], cfg)
         h = moe_apply(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply(h, layer.mlp, cfg)
+    if hidden_out is not None:
+        hidden_out.append(h)
     h = rms_norm(h, model.norm_scale, cfg.norm_eps)
     logits = _dense(h, model.unemb_t, cfg, out_f32=True)  # f32 logits (model.py:784-790)
     logits[:, cfg.vocab_size :] = float("-inf")

@@ -27,6 +27,10 @@ formulas; the checks live in tests/test_oracle_*.py):
 * SwiGLU ........................... scalar closed forms
 * routing / bpermute ............... stable argsort + bincount; the input
                                      vector of reference tests/test_combine.py:13
+* xsa / unit_rows .................. closed forms: alpha = 0 is the identity; t parallel to v^ with tanh(alpha) -> 1
+                                     gives 0; the component of t orthogonal to v^ is unchanged and the parallel one is
+                                     scaled by 1 - tanh(alpha); head n uses kv head n // G (one-hot rows); scalar
+                                     loops on H = 8
 * sample_topk ....................... closed forms: k = 1 is the argmax, u -> 0 / u -> 1 pick the first / k-th
                                      candidate, ties to the lower index, frequencies over a grid of u against
                                      ``torch.softmax`` of the k largest logits / temperature
@@ -477,6 +481,37 @@ def rope_tables(seq_len: int, head_dim: int, rope_base: float = 150000.0, rope_s
         inv_freq = (1.0 - ramp) * (inv_freq / rope_scale) + ramp * inv_freq
     angles = np.einsum("i,j->ij", positions, inv_freq)
     return (np.cos(angles) * concentration).astype(np.float32), (np.sin(angles) * concentration).astype(np.float32)
+
+
+def unit_rows(v: np.ndarray, mode: str = "fp32") -> np.ndarray:
+    """model.py:353-354 - the new token's value rows scaled to unit length: v * rsqrt(sum(v^2) + 1e-10) in float32,
+    held as a bf16 array by the JAX code (``mode="ref"`` rounds there)."""
+    v32 = np.asarray(v, dtype=np.float32)
+    vn = v32 * (np.float32(1.0) / np.sqrt(np.sum(v32 * v32, axis=-1, keepdims=True, dtype=np.float32) + np.float32(1e-10)))
+    return bf16_round(vn) if mode == "ref" else vn.astype(np.float32)
+
+
+def xsa(t: np.ndarray, current_v: np.ndarray, xsa_alpha: np.ndarray, mode: str = "fp32") -> np.ndarray:
+    """model.py:351-363 (learned exclusive self attention) for one new token per sequence.
+
+    t [B, N, H]: attention output after the output gate; current_v [B, K, H]: the new token's value rows as the
+    projection produced them (not the cached, possibly quantised copy); xsa_alpha [N].  Query head n belongs to kv head
+    n // (N // K).  With v^ the unit row of its kv head:  t - tanh(alpha_n) * <t, v^> * v^ .
+    ``mode="ref"`` rounds to bf16 wherever the JAX code holds a bf16 array: v^, the elementwise product inside the
+    inner product, the inner product, tanh(alpha), each of the two products and the difference.
+    """
+    t = np.asarray(t, dtype=np.float32)
+    B, N, H = t.shape
+    K = current_v.shape[1]
+    G = N // K
+    ref = mode == "ref"
+    rnd = bf16_round if ref else (lambda a: np.asarray(a, dtype=np.float32))
+    vn_g = unit_rows(current_v, mode)[:, :, None, :]                         # [B, K, 1, H]
+    t_g = t.reshape(B, K, G, H)
+    coef = np.sum(rnd(t_g * vn_g), axis=-1, keepdims=True, dtype=np.float32)  # float32 sum of (bf16) products
+    alpha = rnd(np.tanh(np.asarray(xsa_alpha, dtype=np.float32))).reshape(1, K, G, 1)
+    out = rnd(t_g - rnd(rnd(alpha * rnd(coef)) * vn_g))
+    return out.reshape(B, N, H).astype(np.float32)
 
 
 def route_tokens(logits: np.ndarray, n_active_routed: int, n_routed: int, n_shared: int):

@@ -17,13 +17,16 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-def _run(case, sm_scale, sw, pos, *, dtype=torch.bfloat16, gate=None, implementation="pallas"):
+def _run(case, sm_scale, sw, pos, *, dtype=torch.bfloat16, gate=None, implementation="pallas", xsa_v=None, xsa_alpha=None):
     from lyra_amd.kernels.decode_attention import decode_attention
 
     q, k, v, sinks = U.attention_torch_inputs(case)
     p = pos if np.ndim(pos) == 0 else torch.from_numpy(np.asarray(pos, dtype=np.int32)).to(U.dev())
     g = None if gate is None else U.t_bf16(gate)
-    out = decode_attention(q, k, v, sinks, sm_scale, sw, p, dtype=dtype, implementation=implementation, gate=g)
+    xv = None if xsa_v is None else U.t_bf16(xsa_v)
+    xa = None if xsa_alpha is None else U.t_f32(xsa_alpha)
+    out = decode_attention(q, k, v, sinks, sm_scale, sw, p, dtype=dtype, implementation=implementation, gate=g, xsa_v=xv,
+                           xsa_alpha=xa)
     torch.cuda.synchronize()
     return U.to_np(out)
 
@@ -195,6 +198,63 @@ def test_split_count_does_not_change_the_result():
     for b in (0, 17, rep - 1):
         U.assert_close(got2[b : b + 1], want, what="few chunks")
     assert np.abs(got2[:1] - got1).max() <= 1e-2
+
+
+@pytest.mark.parametrize("B,N,K,S,H,sw,ragged", [
+    (2, 16, 4, 512, 128, 0, False),     # one workgroup per (row, kv head)
+    (2, 16, 4, 512, 128, 128, False),   # sliding window
+    (3, 32, 8, 4096, 128, 0, True),     # chunked launch: the last workgroup to arrive merges, then the extra step
+    (1, 16, 1, 8192, 128, 0, False),    # more chunks than the merge stages in LDS
+    (70, 8, 4, 384, 128, 0, True),      # whole rows, longest first
+    (40, 64, 8, 384, 64, 0, True),      # ... with 8 wavefronts and 64-wide heads
+])
+def test_learned_exclusive_self_attention_in_the_epilogue(B, N, K, S, H, sw, ragged):
+    """lyra/model.py:351-363 fused behind the gate: t - tanh(alpha) <t, v^> v^ with v^ the new token's unit value row."""
+    case = U.attention_case(6000 + B + N, B, N, K, S, H, fp8=True)
+    rng = np.random.default_rng(B * 7 + N)
+    pos = rng.integers(S // 2, S, B).astype(np.int32) if ragged else np.full(B, S - 1, np.int32)
+    if ragged and B > 2:
+        pos[1] = -1  # a row that sees only the sink: t = 0 stays 0
+    gate = O.bf16_round((2.0 / (1.0 + np.exp(-rng.standard_normal((B, N))))).astype(np.float32))
+    cur_v = O.bf16_round(rng.standard_normal((B, K, H)).astype(np.float32))
+    alpha = rng.standard_normal(N).astype(np.float32)
+    unit = O.unit_rows(cur_v, mode="ref")
+    p = pos if ragged else int(pos[0])
+    _note(f"attn xsa B={B} N={N} K={K} S={S} H={H} sw={sw} ragged={ragged}")
+    if B * K * S > (1 << 16):
+        (kq, ks), (vq, vs) = case["k"], case["v"]
+        t = clib.decode_attention(O.bf16_bits(case["q"]), kq, vq, ks[..., 0], vs[..., 0], case["sinks"], pos, gate, H**-0.5, sw)
+    else:
+        t = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, sw, pos, gate=gate)
+    want = O.xsa(t.reshape(B, N, H), cur_v, alpha).reshape(B, N, 1, H)
+    got = _run(case, H**-0.5, sw, p, gate=gate, xsa_v=unit, xsa_alpha=alpha)
+    U.assert_close(got, want, what="xsa bf16")
+    if ragged and B > 2:
+        assert np.all(got[1] == 0)
+    got32 = _run(case, H**-0.5, sw, p, gate=gate, xsa_v=unit, xsa_alpha=alpha, dtype=torch.float32)
+    U.assert_close(got32, want, atol=6e-3, rtol=6e-3, what="xsa f32")  # (v^ itself is a bf16 array)
+    # The attention output over hundreds of random keys is small (~0.05 per element) and what the step removes smaller
+    # still, so the bounds above barely see it: compare what the step changed, in float32, with what it should change.
+    base32 = _run(case, H**-0.5, sw, p, gate=gate, dtype=torch.float32)
+    removed_got, removed_want = base32 - got32, t.reshape(B, N, 1, H) - want
+    scale = np.abs(removed_want).max()
+    assert scale > 1e-3
+    assert np.abs(removed_got - removed_want).max() <= 0.03 * scale, (np.abs(removed_got - removed_want).max(), scale)
+    # t parallel to v^ and tanh(alpha) -> 1: the first head of every kv head loses everything
+    G = N // K
+    par = t.reshape(B, K, G, H)[:, :, 0, :]
+    keep = np.abs(par).max(-1) > 0
+    unit_par = O.unit_rows(O.bf16_round(par), mode="ref")
+    gone = _run(case, H**-0.5, sw, p, gate=gate, xsa_v=unit_par, xsa_alpha=np.full(N, 20.0, np.float32), dtype=torch.float32)
+    first = gone.reshape(B, K, G, H)[:, :, 0, :]
+    assert np.abs(first[keep]).max() <= 0.02 * np.abs(par[keep]).max()
+    # alpha = 0 switches the step off exactly: same bits as the launch without it
+    base = _run(case, H**-0.5, sw, p, gate=gate)
+    off = _run(case, H**-0.5, sw, p, gate=gate, xsa_v=unit, xsa_alpha=np.zeros(N, np.float32))
+    np.testing.assert_array_equal(off, base)
+    # the plain-framework path computes the same function
+    plain = _run(case, H**-0.5, sw, p, gate=gate, xsa_v=unit, xsa_alpha=alpha, implementation="xla")
+    U.assert_close(plain, want, what="xsa plain path")
 
 
 def test_config4_gpt_oss_shape_ragged_fp8_full_size():

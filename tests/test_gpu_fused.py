@@ -150,6 +150,37 @@ def test_qkv_post_key_codes_bit_exact_at_position_zero():
     assert np.array_equal(ck.scale[:, :, 0, 0].cpu().numpy(), ws[:, :, 0, 0])
 
 
+@pytest.mark.parametrize("H,fp8", [(128, True), (64, False)])
+def test_qkv_post_hands_over_unit_value_rows(H, fp8):
+    """The new token's value rows scaled to unit length (lyra/model.py:353-354), taken before cache quantisation; a zero
+    row stays zero (the 1e-10 under the root); rows whose position lies outside the cache are handed over all the same."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray
+
+    B, N, K, S = 7, 4, 2, 16
+    rng = np.random.default_rng(12)
+    qkv = O.bf16_round(rng.standard_normal((B, (N + 2 * K) * H), dtype=np.float32) * np.exp(rng.standard_normal((B, 1)) * 3).astype(np.float32))
+    qkv[2, (N + K) * H : (N + K + 1) * H] = 0.0
+    cos_t, sin_t = O.rope_tables(S, H)
+    dev = U.dev()
+    if fp8:
+        mk = lambda: QArray(torch.zeros((B, K, S, H), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn),
+                            torch.ones((B, K, S, 1), dtype=torch.float32, device=dev), (1, H))
+    else:
+        mk = lambda: torch.zeros((B, K, S, H), dtype=torch.bfloat16, device=dev)
+    pos = torch.tensor([0, 3, 15, 16, -1, 7, 8], dtype=torch.int32, device=dev)
+    _say(f"qkv_post unit rows H{H} fp8={fp8}")
+    q, vn = F.qkv_post(U.t_bf16(qkv), None, None, U.t_f32(cos_t), U.t_f32(sin_t), pos, mk(), mk(), N, K, H, 1e-5, unit_v=True)
+    torch.cuda.synchronize()
+    v = qkv[:, (N + K) * H :].reshape(B, K, H)
+    want = O.unit_rows(v, mode="ref")
+    got = U.to_np(vn)
+    assert np.abs(got - want).max() <= 2.0**-8  # one bf16 step at magnitude <= 1 (rsqrt vs 1/sqrt)
+    assert (got == want).mean() > 0.9
+    assert np.all(got[2, 0] == 0)
+    np.testing.assert_allclose(np.sum(got.astype(np.float64) ** 2, -1)[np.abs(v).max(-1) > 0], 1.0, atol=2e-2)
+
+
 @pytest.mark.parametrize("T,n_routed,n_shared,k", [(64, 15, 1, 3), (5, 7, 1, 1), (128, 31, 1, 3), (33, 63, 1, 3), (16, 8, 0, 2), (1, 15, 1, 3),
                                                    (256, 15, 1, 3), (300, 15, 1, 3), (250, 127, 1, 3), (3, 128, 0, 8)])
 def test_moe_route(T, n_routed, n_shared, k):

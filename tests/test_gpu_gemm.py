@@ -133,13 +133,16 @@ def _zipf_routing(rng, T, n_routed, k, n_shared):
     return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
 
 
-@pytest.mark.parametrize("T", [1, 16, 64])
-def test_config3_moe_medium_shape_zipf_routing(T):
-    """Benchmark configuration 3 (MoE matmul at lyra-medium widths): width 4096, 31 routed + 1 shared expert, FP8 per-channel scales, top-(3+1) Zipf(1.1)."""
+@pytest.mark.parametrize("T,k_routed", [(1, 3), (16, 3), (64, 3), (1, 4), (16, 4), (64, 4)])
+def test_config3_moe_medium_shape_zipf_routing(T, k_routed):
+    """Benchmark configuration 3 (MoE matmul at lyra-medium widths): width 4096, 31 routed + 1 shared expert, FP8 per-channel
+    scales, Zipf(1.1) routing: top-(3+1) as lyra/variants.py has it (4 active experts, one of them shared) and 4 routed
+    + the shared expert as the configuration's wording has it."""
     C, Hd, E = 4096, 4096, 32
-    rng = np.random.default_rng(1003 + T)
-    sizes = _zipf_routing(rng, T, 31, 3, 1)
+    rng = np.random.default_rng(1003 + T + 100 * (k_routed - 3))
+    sizes = _zipf_routing(rng, T, 31, k_routed, 1)
     M = int(sizes.sum())
+    assert M == (k_routed + 1) * T
     up = _case(5, M, E, C, 2 * Hd, sizes, kind="fp8", block=(C, 1))
     _note(f"gemm cfg3 up T={T} M={M} touched={(sizes > 0).sum()}")
     want_up = _want(up, True, big=True)

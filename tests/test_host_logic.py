@@ -163,6 +163,39 @@ def test_decode_step_driver_on_cpu_matches_oracle(fp8):
     assert int(cache.pos) == 2
 
 
+def test_decode_step_driver_with_exclusive_self_attention_and_biases_on_cpu_matches_oracle():
+    """The model options of the larger variants (use_learned_xsa, lyra/variants.py:38) and of the gpt-oss shapes (biases on
+    q/k/v, the output projection and the MLPs, no shared expert, no QK norm, YaRN tables; variants.py:62-80) through the
+    plain-framework operators: same op sequence as the oracle's decode step."""
+    from lyra_amd.model import MODEL_VARIANTS, init_cache, init_weights, model_apply
+
+    dev = torch.device("cpu")
+    base = replace(MODEL_VARIANTS["dev"], implementation="xla", seq_len=64, sliding_window=16)
+    cases = {
+        "xsa": replace(base, use_learned_xsa=True, use_sdpa_output_gate=True),
+        "gpt-oss-like": replace(base, use_qk_norm=False, use_qkv_bias=True, use_attn_out_bias=True, use_mlp_bias=True,
+                                n_shared_experts=0, n_active_experts=2, rope_scale=4.0, mlp_map=("moe", "dense", "moe", "moe")),
+    }
+    for name, cfg in cases.items():
+        w = init_weights(cfg, dev, seed=2)
+        assert (w.layers[0].attn.xsa_alpha is not None) == cfg.use_learned_xsa
+        cache = init_cache(cfg, 2, 64, dev)
+        cache.pos.fill_(0)
+        wn, cn = D.weights_to_numpy(w, cfg), D.cache_to_numpy(cache)
+        tokens = np.asarray([[3, 900], [17, 5], [4, 4]])
+        for s in range(3):
+            got, _ = model_apply(torch.from_numpy(tokens[s]), w, cache, cfg)
+            want = D.decode_step(tokens[s], wn, cn, s, cfg)
+            np.testing.assert_allclose(got[:, : cfg.vocab_size].numpy(), want[:, : cfg.vocab_size], atol=6e-2, rtol=2e-2, err_msg=name)
+        # the options are not no-ops: the same weights without them give different logits
+        first = D.decode_step(tokens[0], wn, D.cache_to_numpy(init_cache(cfg, 2, 64, dev)), 0, cfg)
+        for lw in w.layers:
+            lw.attn.xsa_alpha = lw.attn.qkv_bias = lw.attn.out_bias = None
+            lw.mlp.mlp_up_bias = lw.mlp.mlp_down_bias = None
+        other, _ = model_apply(torch.from_numpy(tokens[0]), w, init_cache(cfg, 2, 64, dev), cfg)
+        assert np.abs(other[:, : cfg.vocab_size].numpy() - first[:, : cfg.vocab_size]).max() > 0.05, name
+
+
 def test_sampling():
     from lyra_amd.generate import sample_token
     from lyra_amd.model import MODEL_VARIANTS

@@ -5,6 +5,8 @@ limits in the sink, brute-force window arithmetic over every position, a one-hot
 GQA head-mapping probe, and the input vector of the reference's own
 tests/test_decode_attention.py:54-65.
 """
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -189,3 +191,75 @@ def test_c_oracle_matches_numpy_oracle(fp8, sw):
         # summation order differs (einsum vs sequential); "ref" may flip a bf16 ulp
         tol = 2e-5 if mode == "fp32" else 1.6e-2
         np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
+
+
+# ---- learned exclusive self attention (lyra/model.py:351-363) ----------------------------------------------
+def _xsa_case(seed, B=2, N=8, K=2, H=8):
+    rng = np.random.default_rng(seed)
+    t = rng.standard_normal((B, N, H)).astype(np.float32)
+    v = rng.standard_normal((B, K, H)).astype(np.float32)
+    alpha = rng.standard_normal(N).astype(np.float32)
+    return t, v, alpha
+
+
+def test_xsa_closed_forms():
+    t, v, alpha = _xsa_case(0)
+    B, N, H = t.shape
+    K = v.shape[1]
+    G = N // K
+    # alpha = 0: tanh(0) = 0, nothing is removed
+    assert np.array_equal(O.xsa(t, v, np.zeros(N, np.float32)), t)
+    # unit rows have length 1 (the 1e-10 only matters for a zero row, which stays zero)
+    vn = O.unit_rows(v)
+    np.testing.assert_allclose(np.sum(vn * vn, -1), 1.0, atol=1e-6)
+    assert np.array_equal(O.unit_rows(np.zeros((1, 1, H), np.float32)), np.zeros((1, 1, H), np.float32))
+    # t parallel to v^ and tanh(alpha) -> 1: everything is removed
+    par = np.repeat(3.0 * vn, G, axis=1)  # head n takes kv head n // G
+    out = O.xsa(par, v, np.full(N, 20.0, np.float32))
+    assert np.abs(out).max() < 1e-5
+    # the orthogonal component is untouched, the parallel one is scaled by 1 - tanh(alpha)
+    out = O.xsa(t, v, alpha)
+    vg = np.repeat(vn, G, axis=1)
+    dot_in, dot_out = np.sum(t * vg, -1), np.sum(out * vg, -1)
+    np.testing.assert_allclose(dot_out, dot_in * (1.0 - np.tanh(alpha))[None, :], atol=1e-5)
+    np.testing.assert_allclose(out - dot_out[..., None] * vg, t - dot_in[..., None] * vg, atol=1e-5)
+    # sign: a positive alpha shrinks the component along v^ (a wrong sign would grow it)
+    pos = O.xsa(par, v, np.full(N, 0.5, np.float32))
+    assert (np.sum(pos * vg, -1) < np.sum(par * vg, -1)).all()
+
+
+def test_xsa_scalar_loops_and_head_mapping():
+    t, v, alpha = _xsa_case(1, B=2, N=6, K=3, H=8)
+    B, N, H = t.shape
+    K = v.shape[1]
+    G = N // K
+    want = np.zeros_like(t)
+    for b in range(B):
+        for n in range(N):
+            k = n // G
+            norm2 = sum(float(v[b, k, h]) ** 2 for h in range(H)) + 1e-10
+            unit = [float(v[b, k, h]) / math.sqrt(norm2) for h in range(H)]
+            coef = sum(float(t[b, n, h]) * unit[h] for h in range(H))
+            for h in range(H):
+                want[b, n, h] = float(t[b, n, h]) - math.tanh(float(alpha[n])) * coef * unit[h]
+    np.testing.assert_allclose(O.xsa(t, v, alpha), want, atol=1e-5)
+    # one-hot value rows: kv head k points along axis k, so head n loses exactly its component along axis n // G
+    v1 = np.zeros((B, K, H), np.float32)
+    for k in range(K):
+        v1[:, k, k] = 2.0
+    out = O.xsa(t, v1, np.full(N, 20.0, np.float32))
+    for n in range(N):
+        keep = np.ones(H, bool)
+        keep[n // G] = False
+        assert np.abs(out[:, n, n // G]).max() < 1e-5
+        assert np.array_equal(out[:, n, keep], t[:, n, keep])
+
+
+def test_xsa_bf16_flow_stays_close_to_float32():
+    rng = np.random.default_rng(2)
+    t = O.bf16_round(rng.standard_normal((3, 16, 128)).astype(np.float32))
+    v = O.bf16_round(rng.standard_normal((3, 4, 128)).astype(np.float32))
+    alpha = rng.standard_normal(16).astype(np.float32)
+    a, b = O.xsa(t, v, alpha, mode="ref"), O.xsa(t, v, alpha)
+    assert np.array_equal(a, O.bf16_round(a))
+    assert np.abs(a - b).max() <= 2e-2 + 1e-2 * np.abs(b).max()
