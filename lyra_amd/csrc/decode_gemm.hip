@@ -142,6 +142,35 @@ __device__ __forceinline__ void convert_pair(const RawW<FP8>& t, int pair, Pack8
     }
 }
 
+// The K-major B operands of column phases 2*cp and 2*cp + 1 from all 8 weight rows of this lane (what convert_pair does for
+// one row pair and all phases, done for all row pairs and one pair of phases).
+// SCALED: every value is multiplied by `scale` in float32 before it is rounded to bf16 - the dequantisation of the plain-JAX
+// path, bit for bit: dequantize() forms f32(code) * scale and casts to the activation dtype (lyra/nn/quant.py:82-85).
+template <bool FP8, bool SCALED = false>
+__device__ __forceinline__ void convert_colpair(const RawW<FP8>& t, int cp, Pack8& b0, Pack8& b1, float scale = 1.f) {
+    const int c = 2 * cp;
+#pragma unroll
+    for (int pr = 0; pr < 4; ++pr) {
+        const int i = 2 * pr;
+        if constexpr (FP8) {
+            f32x2 fa = fp8x2_to_f32(t.w[i][c >> 2], (c & 2) != 0);
+            f32x2 fb = fp8x2_to_f32(t.w[i + 1][c >> 2], (c & 2) != 0);
+            if constexpr (SCALED) {
+                fa[0] *= scale;
+                fa[1] *= scale;
+                fb[0] *= scale;
+                fb[1] *= scale;
+            }
+            b0.u[pr] = pack_bf16(fa[0], fb[0]);
+            b1.u[pr] = pack_bf16(fa[1], fb[1]);
+        } else {
+            const uint32_t a = t.w[i][c >> 1], b = t.w[i + 1][c >> 1];
+            b0.u[pr] = __builtin_amdgcn_perm(b, a, 0x05040100u);
+            b1.u[pr] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+        }
+    }
+}
+
 // Writes 8 consecutive result columns of one row: fused epilogue (ksplit == 1) or float32 partials.
 // Must be called by all lanes of the wavefront (SwiGLU exchanges gate and linear halves by shuffle);
 // `store` says whether this lane's row exists.
@@ -984,7 +1013,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     int seg_u = 0, seg_r0 = 0, seg_r1 = 0;  // its unit and trips [r0, r1) of it
     int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
     __amdgpu_buffer_rsrc_t wrsrc;
-    u32x4 a[DEPTH][MTM];
+    constexpr int ADEPTH = 2;  // activation steps in flight (they come from the caches; the weights, from memory, need DEPTH)
+    u32x4 a[ADEPTH][MTM];
     RawW<FP8> w[DEPTH];
     [[maybe_unused]] float step_sc[DEPTH];  // STEP_SCALES: the scale of each step in flight travels with its weights
     [[maybe_unused]] int sc_voff = kNoLoad;
@@ -1028,9 +1058,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             const bool live = valid && idx < n_my;
             const int kk = (wslot + kw * idx) << 5;
             const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
+            if (d < ADEPTH) {
 #pragma unroll
-            for (int mt = 0; mt < MTM; ++mt)
-                a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
+                for (int mt = 0; mt < MTM; ++mt)
+                    a[d % ADEPTH][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
+            }
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
             if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, live, sc_voff, kk);
@@ -1063,72 +1095,89 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 #pragma unroll
             for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        [[maybe_unused]] int cur_blk = -1;     // STEP_SCALES: scale block the accumulators are expressed in, and its scale
-        [[maybe_unused]] float s_cur = 1.f;
         // every pass issues the same loads (past the end of the segment they fetch nothing) and multiplies zeros there
         const int idx_end = min(n_my, r1 * TRIP);
-        for (int trip = r0; trip < r1; ++trip) {
+        // The steps of a wavefront form a software pipeline: while the matrix cores multiply step s, the vector ALU turns the
+        // raw weights of step s+1 into operands, two column phases at a time - the 2 * NMT matrix instructions that consume
+        // the current operands of phases 2cp, 2cp+1 are interleaved with the 16 conversions that produce their successors,
+        // which then take their place.  A unit of many rows (32 matrix instructions per step) thus hides its conversions
+        // behind them instead of doing one after the other.  The loop is instantiated per number of 16-row tiles so that a
+        // step is straight-line code the scheduler can interleave.
+        Pack8 bop[8];
+        auto k_loop = [&](auto nmt_c) {
+            constexpr int NMT = decltype(nmt_c)::value;
+            {  // operands of the item's first step; its register set is then refilled with step DEPTH
+                const int idx0 = r0 * TRIP;
+                const bool more = idx0 + DEPTH < idx_end;
+                const int kk_next = (wslot + kw * (idx0 + DEPTH)) << 5;
 #pragma unroll
-            for (int ur = 0; ur < ROUNDS; ++ur) {
+                for (int cp = 0; cp < 4; ++cp) {
+                    if constexpr (STEP_SCALES) convert_colpair<FP8, true>(w[0], cp, bop[2 * cp], bop[2 * cp + 1], step_sc[0]);
+                    else convert_colpair<FP8>(w[0], cp, bop[2 * cp], bop[2 * cp + 1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int d = 0; d < DEPTH; ++d) {
-                    const int idx = (trip * ROUNDS + ur) * DEPTH + d;
-                    const int kk = (wslot + kw * idx) << 5;
-                    const int kk_next = kk + ((kw * DEPTH) << 5);
-                    const bool more = idx + DEPTH < idx_end;
-                    Pack8 bop[8], av[MTM];
+                for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(more, w[0], pr, cur_wrsrc, cur_wvoff, kk_next, row_bytes);
+                if constexpr (STEP_SCALES) step_sc[0] = load_step_scale(p, scrsrc, more, cur_sc_voff, kk_next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            for (int trip = r0; trip < r1; ++trip) {
 #pragma unroll
-                    for (int mt = 0; mt < MTM; ++mt)
+                for (int ur = 0; ur < ROUNDS; ++ur) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) av[mt].u[i] = a[d][mt][i];
-                    float sc = 1.f;
-                    if constexpr (STEP_SCALES) sc = step_sc[d];
-                    __builtin_amdgcn_sched_barrier(0);
-                    const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
+                    for (int d = 0; d < DEPTH; ++d) {
+                        const int dn = (d + 1) % DEPTH;
+                        const int idx = (trip * ROUNDS + ur) * DEPTH + d;
+                        const int kk = (wslot + kw * idx) << 5;
+                        const int kk_w = kk + ((kw * (DEPTH + 1)) << 5);      // the next step of the following weight register set
+                        const int kk_act = kk + ((kw * ADEPTH) << 5);         // the next step of this step's activation registers
+                        const int ad = (ur * DEPTH + d) % ADEPTH;
+                        const bool more_w = idx + 1 + DEPTH < idx_end, more_act = idx + ADEPTH < idx_end;
+                        bf16x8 av[NMT];
 #pragma unroll
-                    for (int mt = 0; mt < MTM; ++mt)
-                        a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? cur_avoff[mt] : kNoLoad, soff, 0);
+                        for (int mt = 0; mt < NMT; ++mt) av[mt] = __builtin_bit_cast(bf16x8, a[ad][mt]);
 #pragma unroll
-                    for (int pr = 0; pr < 4; ++pr) {
-                        convert_pair<FP8>(w[d], pr, bop);
-                        __builtin_amdgcn_sched_barrier(0);
-                        load_w_pair_if<FP8>(more, w[d], pr, cur_wrsrc, cur_wvoff, kk_next, row_bytes);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    if constexpr (STEP_SCALES) step_sc[d] = load_step_scale(p, scrsrc, more, cur_sc_voff, kk_next);
-                    if constexpr (STEP_SCALES) {
-                        // The accumulators are kept in units of the current scale block's scale; when the block changes
-                        // they are converted (one multiply each), so the products themselves need no scaling.  A zero
-                        // scale counts as 1e-30: its block then contributes nothing that float32 can see.
-                        const int blk = scale_block_of(p, kk);
-                        if (blk != cur_blk && kk < p.K) {  // same for the whole wavefront; steps past the end change nothing
-                            cur_blk = blk;
-                            const float s_new = fabsf(sc) < 1e-30f ? 1e-30f : sc;
-                            const float ratio = s_cur * __builtin_amdgcn_rcpf(s_new);
-                            s_cur = s_new;
+                        for (int cp = 0; cp < 4; ++cp) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            Pack8 n0, n1;
+                            if constexpr (STEP_SCALES) convert_colpair<FP8, true>(w[dn], cp, n0, n1, step_sc[dn]);
+                            else convert_colpair<FP8>(w[dn], cp, n0, n1);
 #pragma unroll
-                            for (int mt = 0; mt < MTM; ++mt) {
-                                if (mt < n_mt) {
-#pragma unroll
-                                    for (int c = 0; c < 8; ++c) {
-                                        acc[mt][c][0] *= ratio;
-                                        acc[mt][c][1] *= ratio;
-                                        acc[mt][c][2] *= ratio;
-                                        acc[mt][c][3] *= ratio;
-                                    }
-                                }
+                            for (int mt = 0; mt < NMT; ++mt) {
+                                acc[mt][2 * cp] = mfma_16x16x32(av[mt], bop[2 * cp].v, acc[mt][2 * cp]);
+                                acc[mt][2 * cp + 1] = mfma_16x16x32(av[mt], bop[2 * cp + 1].v, acc[mt][2 * cp + 1]);
                             }
-                        }
-                    }
+                            // 2 * NMT matrix instructions, 16 (FP8) or 8 (bf16) vector instructions: spread evenly
+                            constexpr int kVecOps = FP8 ? (STEP_SCALES ? 32 : 16) : 8, kPer = (kVecOps + 2 * NMT - 1) / (2 * NMT);
 #pragma unroll
-                    for (int mt = 0; mt < MTM; ++mt) {
-                        if (mt < n_mt) {
-#pragma unroll
-                            for (int c = 0; c < 8; ++c) acc[mt][c] = mfma_16x16x32(av[mt].v, bop[c].v, acc[mt][c]);
+                            for (int j = 0; j < 2 * NMT; ++j) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x002, kPer, 0);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                            bop[2 * cp] = n0;
+                            bop[2 * cp + 1] = n1;
                         }
+                        __builtin_amdgcn_sched_barrier(0);
+                        // the registers just consumed are requested again: the activations for step idx + ADEPTH, the converted
+                        // weight rows for step idx + 1 + DEPTH
+                        const int soff_act = __builtin_amdgcn_readfirstlane(more_act ? kk_act * 2 : 0);
+#pragma unroll
+                        for (int mt = 0; mt < MTM; ++mt)
+                            a[ad][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more_act ? cur_avoff[mt] : kNoLoad, soff_act, 0);
+#pragma unroll
+                        for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(more_w, w[dn], pr, cur_wrsrc, cur_wvoff, kk_w, row_bytes);
+                        if constexpr (STEP_SCALES) step_sc[dn] = load_step_scale(p, scrsrc, more_w, cur_sc_voff, kk_w);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
+        };
+        switch (n_mt) {
+            case 1: k_loop(std::integral_constant<int, 1>{}); break;
+            case 2: k_loop(std::integral_constant<int, 2>{}); break;
+            case 3: k_loop(std::integral_constant<int, 3>{}); break;
+            default: k_loop(std::integral_constant<int, 4>{}); break;
         }
 
         // Scales that are constant along K are applied to the finished tile.  They are requested here, ahead of the next
@@ -1136,7 +1185,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         float colscale[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            colscale[c] = STEP_SCALES ? s_cur : 1.f;
+            colscale[c] = 1.f;  // (scale blocks along K were applied to the weights)
             if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
                 const int off = (cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift)) * 4;
                 if (c == 0) colscale[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));

@@ -100,8 +100,9 @@ def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_s
 
 
 def decode_gemm(lhs_bits, rhs, rhs_scale, block, group_sizes, bias, *, fused_swiglu=False, beta=1.702, limit=7.0,
-                ref_rounding=False, scratch=None):
-    """lhs_bits uint16 [M,K]; rhs uint8 (fp8, with rhs_scale/block) or uint16 (bf16) [G,K,N]; returns f32."""
+                ref_rounding=False, scratch=None, dequant_bf16=False):
+    """lhs_bits uint16 [M,K]; rhs uint8 (fp8, with rhs_scale/block) or uint16 (bf16) [G,K,N]; returns f32.
+    ref_rounding: dequantised weights and outputs rounded to bf16; dequant_bf16 (without it): only the dequantised weights."""
     lib = load()
     M, K = lhs_bits.shape
     G, _, N = rhs.shape
@@ -116,7 +117,7 @@ def decode_gemm(lhs_bits, rhs, rhs_scale, block, group_sizes, bias, *, fused_swi
         scratch = np.empty((G, K, N), dtype=np.float32)
     rc = lib.lyra_oracle_decode_gemm(
         _p(lhs_bits), _p(rhs), _p(sc), bk, bn, _p(gs), _p(b), _p(out), _p(scratch),
-        M, G, K, N, int(fp8), int(fused_swiglu), float(beta), float(limit), int(ref_rounding),
+        M, G, K, N, int(fp8), int(fused_swiglu), float(beta), float(limit), 1 if ref_rounding else (2 if dequant_bf16 else 0),
     )
     if rc:
         raise RuntimeError(f"lyra_oracle_decode_gemm failed: {rc}")

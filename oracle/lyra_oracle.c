@@ -277,6 +277,9 @@ int lyra_oracle_decode_gemm(const uint16_t* lhs, const void* rhs, const float* r
     if (fused_swiglu && (N % 2)) return -1;
     fp8_init();
     const int KB = rhs_fp8 ? K / bk : 0, NB = rhs_fp8 ? N / bn : 0;
+    /* ref_rounding: 0 = float32 throughout, 1 = dequantised weights and outputs rounded to bf16 as the JAX code holds them,
+       2 = only the dequantised weights rounded (quant.py:85), product and epilogue in float32 */
+    const int round_out = ref_rounding == 1;
     /* step 1: dequantise ALL experts to lhs.dtype */
 #pragma omp parallel for collapse(2) schedule(static)
     for (int g = 0; g < G; ++g) {
@@ -326,10 +329,10 @@ int lyra_oracle_decode_gemm(const uint16_t* lhs, const void* rhs, const float* r
                     float glu = fminf(t[n], limit);
                     float lin = fminf(fmaxf(t[NO + n], -limit), limit);
                     float y = (lin + 1.0f) * (glu * (1.0f / (1.0f + expf(-beta * glu))));
-                    o[n] = ref_rounding ? bf16_round(y) : y;
+                    o[n] = round_out ? bf16_round(y) : y;
                 }
             } else {
-                for (int n = 0; n < NO; ++n) o[n] = ref_rounding ? bf16_round(t[n]) : t[n];
+                for (int n = 0; n < NO; ++n) o[n] = round_out ? bf16_round(t[n]) : t[n];
             }
         }
         free(t);

@@ -424,6 +424,7 @@ def decode_gemm_reference(
     swiglu_beta: float = 1.702,
     swiglu_limit: float = 7.0,
     mode: str = "fp32",
+    dequant_bf16: bool | None = None,
 ) -> np.ndarray:
     """decode_gemm.py:368-401 / :419-449.
 
@@ -431,11 +432,13 @@ def decode_gemm_reference(
     lhs.dtype = bf16, :437) or (qval uint8 [G,K,N], scale f32 [G,K/bk,N/bn]) with
     ``block=(bk,bn)``, dequantised to lhs.dtype before the grouped product (:431).
     The lhs is never quantised on this path (quant_dtype=None at :398).
+    ``dequant_bf16`` overrides what ``mode`` says about the dequantised weights alone: True rounds them to bf16 as the
+    reference does (quant.py:85) while the product, bias and SwiGLU stay in float32 when mode="fp32".
     """
     if isinstance(rhs, tuple):
         qval, scale = rhs
         assert block is not None
-        w = dequantize(qval, scale, block, to_bf16=(mode == "ref"))
+        w = dequantize(qval, scale, block, to_bf16=(mode == "ref") if dequant_bf16 is None else dequant_bf16)
     else:
         w = np.asarray(rhs, dtype=np.float32)
         if mode == "ref":
