@@ -278,6 +278,10 @@ def kernel_table(dev, only=""):
             gemm(f"probe lyra-small expert up+SwiGLU B=64, shared expert {shared_rows} rows", int(t.sum()), 16, 2048, 4096, t, True, (2048, 1))
             gemm(f"probe lyra-small expert down B=64, shared expert {shared_rows} rows", int(t.sum()), 16, 2048, 2048, t, False, (2048, 1))
         print("rows per expert:", s.tolist(), file=sys.stderr)
+        # what a unit costs by its number of rows: every expert of the lyra-medium up projection with the same row count
+        for rows_each in (8, 16, 32, 48, 64):
+            t = np.full(32, rows_each, np.int32)
+            gemm(f"probe lyra-medium expert up+SwiGLU, {rows_each} rows for each of 32 experts", int(t.sum()), 32, 4096, 8192, t, True, (4096, 1))
     for name, K, N, sw in (("q/k/v", 2048, 3072, False), ("out", 2048, 2048, False), ("dense up+SwiGLU", 2048, 6144, True),
                            ("dense down", 3072, 2048, False)):
         gemm(f"lyra-small {name} projection B=64 ({K}x{N} fp8)", 64, 1, K, N, [64], sw, (K, 1))

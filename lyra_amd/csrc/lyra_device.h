@@ -142,6 +142,10 @@ __device__ __forceinline__ f32x4 load_agent_b128(__amdgpu_buffer_rsrc_t rsrc, in
     return v;
 }
 
+// Workgroup barrier for data exchanged through LDS: waits for this wavefront's LDS operations only.  __syncthreads() also
+// waits for every global load the wavefront has in flight, which empties the prefetch queue of a streaming kernel.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, kWave));
