@@ -1214,7 +1214,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();  // (the next item's operands stay in flight)
         constexpr int TS = 16 * MTM * kSplitPitch;  // floats per wavefront tile
         // Sum of the wavefront tiles for 4 columns of row r: vg (and vl, the second set of 128 columns of a wide unit).
         auto tile_row = [&](int r, float (&vg)[4], float (&vl)[4]) {
@@ -1333,7 +1333,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             if (p.residual) run_rows(std::true_type{});
             else run_rows(std::false_type{});
         }
-        __syncthreads();  // the tiles are free for the next unit
+        lds_barrier();  // the tiles are free for the next unit
     }
     wait_all_memory();  // (requests of an item past the end return nothing, but must not outlive the wavefront's registers)
 
