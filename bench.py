@@ -120,6 +120,90 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13):
     return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / (len(pairs) * len(layers))  # seconds per launch
 
 
+def _nbytes(w):
+    """Bytes of a weight array as the kernels read it (codes + scales for a quantised array)."""
+    from lyra_amd.nn.quant import QArray
+
+    if isinstance(w, QArray):
+        return w.qval.numel() * w.qval.element_size() + w.scale.numel() * w.scale.element_size()
+    return w.numel() * w.element_size()
+
+
+def step_algorithmic_bytes(cfg, weights, batch, ctx, touched_per_moe_layer):
+    """Bytes one decode step has to read at the least: visible K/V rows (+ scales) of every layer, every projection and
+    dense MLP weight once, the weights of the experts that have rows (counted from the step's own routing), the LM head.
+    Activations, norms' small parameters and the embedding rows are left out (a few MB)."""
+    from lyra_amd.model import MoEWeights
+
+    total, moe = 0, 0
+    for idx, layer in enumerate(weights.layers):
+        visible = min(cfg.sliding_window, ctx) if (idx % 2 == 0 and cfg.sliding_window > 0) else ctx
+        total += attention_algorithmic_bytes(batch, cfg.n_kv_heads, visible, cfg.head_dim, fp8=cfg.quantize_cache)
+        total += _nbytes(layer.attn.qkv) + _nbytes(layer.attn.out)
+        if isinstance(layer.mlp, MoEWeights):
+            per_expert = (_nbytes(layer.mlp.mlp_up) + _nbytes(layer.mlp.mlp_down)) // cfg.n_experts
+            total += per_expert * touched_per_moe_layer[moe]
+            moe += 1
+        else:
+            total += _nbytes(layer.mlp.mlp_up) + _nbytes(layer.mlp.mlp_down)
+    return total + _nbytes(weights.unemb_t)
+
+
+def time_expert_matmuls(dev, one_step, stream, rounds=10):
+    """The expert matmuls through the C ABI, HIP events on the launch stream, between replays of the decode step (as the
+    attention launch is timed): the up projection with fused SwiGLU and the down projection at the shape of a
+    lyra-medium MoE layer (benchmark configuration 3: width 4096, 31 routed + 1 shared experts of hidden 4096, 64 tokens,
+    3 routed experts per token drawn from Zipf(1.1) + the shared one, seeded) and at the shape of the lyra-small layer the
+    step itself runs (15 + 1 experts, width 2048, hidden 2048).  FP8 weights, one scale per output channel."""
+    import numpy as np
+    import torch
+
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1003)
+    out_rows = []
+    for label, E, C, Hd, n_routed in (("lyra-medium", 32, 4096, 4096, 31), ("lyra-small", 16, 2048, 2048, 15)):
+        sizes = zipf_group_sizes(np.random.default_rng(1003), 64, n_routed, 3, 1)
+        M, touched = int(sizes.sum()), int((sizes > 0).sum())
+        gs = torch.from_numpy(sizes).to(dev)
+        x = torch.randn(M, C, generator=gen, device=dev, dtype=torch.bfloat16)
+        cases = []
+        for name, K, N, swiglu in (("up+SwiGLU", C, 2 * Hd, True), ("down", Hd, C, False)):
+            w = torch.randint(0, 0x78, (E, K, N), generator=gen, device=dev, dtype=torch.uint8)
+            sc = torch.rand(E, 1, N, generator=gen, device=dev) * 0.001 + 0.0005
+            lhs = x if K == C else torch.randn(M, K, generator=gen, device=dev, dtype=torch.bfloat16)
+            out = torch.empty(M, N // 2 if swiglu else N, device=dev, dtype=torch.bfloat16)
+            ws = torch.zeros(max(L.lyra_decode_gemm_workspace(M, E, K, N, int(swiglu)), 256), dtype=torch.uint8, device=dev)
+            nbytes = touched * (K * N + N * 4) + M * K * 2 + out.numel() * 2
+
+            def launch(lhs=lhs, w=w, sc=sc, out=out, ws=ws, K=K, N=N, swiglu=swiglu):
+                rc = L.lyra_decode_gemm(lhs.data_ptr(), w.data_ptr(), sc.data_ptr(), K, 1, gs.data_ptr(), None, out.data_ptr(),
+                                        ws.data_ptr(), ws.numel(), M, E, K, N, _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, int(swiglu),
+                                        1.702, 7.0, stream.cuda_stream)
+                _lib.check(rc, "lyra_decode_gemm")
+
+            cases.append((f"{label} expert {name} ({E}x{K}x{N} fp8), 64 tokens, {touched} experts with rows", nbytes, launch, []))
+        for r in range(rounds + 2):  # the first two rounds warm up
+            one_step()
+            for _, _, launch, pairs in cases:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record(stream)
+                launch()
+                b.record(stream)
+                if r >= 2:
+                    pairs.append((a, b))
+        stream.synchronize()
+        for case, nbytes, _, pairs in cases:
+            t = sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / len(pairs)
+            out_rows.append({"kernel": "decode_gemm_group_kernel<fp8>", "case": case, "bound": "hbm", "achieved": nbytes / t / 1e9,
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
+                             "algorithmic_bytes": nbytes, "us_per_launch": t * 1e6})
+        del cases
+    return out_rows
+
+
 def _time_launches(launch, stream, warm=5, iters=50):
     import torch
 
@@ -352,6 +436,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm-roofline", action="store_true", help="skip the stand-alone expert matmul timings")
     ap.add_argument("--model", default="lyra-small", help="model variant of the decode step (the headline figure is lyra-small)")
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
@@ -379,7 +464,17 @@ def main():
     elapsed, one_step = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
     tokens_per_s = args.batch * args.steps / elapsed
 
+    # what the step's own routing touches (one eager step; the graph replays the same kernels on the same inputs)
+    groups = []
+    from lyra_amd.model import model_apply
+
+    cache.pos.fill_(args.ctx - 1)
+    model_apply(torch.arange(args.batch, device=dev) % cfg.vocab_size, weights, cache, cfg, groups_out=groups)
+    touched = [int((g > 0).sum().item()) for g in groups]
+    step_bytes = step_algorithmic_bytes(cfg, weights, args.batch, args.ctx, touched)
+
     t_attn = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step)
+    gemm_rows = time_expert_matmuls(dev, one_step, torch.cuda.current_stream(dev)) if not args.no_gemm_roofline else None
     attn_bytes = attention_algorithmic_bytes(args.batch, cfg.n_kv_heads, args.ctx, cfg.head_dim, fp8=True)
     achieved = attn_bytes / t_attn / 1e9
     traffic = None
@@ -408,6 +503,10 @@ def main():
             "batch": args.batch,
             "ctx": args.ctx,
             "us_per_layer": elapsed / args.steps / cfg.n_layers * 1e6,
+            "step_algorithmic_bytes": step_bytes,
+            "step_frac": step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,  # of the 8 TB/s roofline, whole step
+            "experts_with_rows_per_moe_layer": touched,
+            "projections": "q/k/v and output projections FP8 as well (quantize_attn; the reference's --fp8 leaves them bf16)",
         },
         "roofline": {
             "kernel": "decode_attention_kernel<128, fp8> (global layer)",
@@ -421,6 +520,8 @@ def main():
             "us_per_launch": t_attn * 1e6,
         },
     }
+    if gemm_rows is not None:
+        result["roofline"]["gemm"] = gemm_rows
     if args.traffic_probe:
         result["traffic_probe"] = traffic_probe(dev)
     if not args.no_cpu_baseline:

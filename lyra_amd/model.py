@@ -473,7 +473,7 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     return out, cache
 
 
-def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
+def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None = None):
     """moe_apply as norm+router | routing | up matmul (token gather fused) | down matmul; the combine + residual step is
     handed to the next norm as an ``Uncombined`` value."""
     from lyra_amd.kernels import decode_fused as F
@@ -485,6 +485,8 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig):
         xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
     B = x.shape[0]
     scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
+    if groups_out is not None:
+        groups_out.append(groups)
     t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
                swiglu_limit=cfg.swiglu_limit)
     t = F.gemm(t, w.mlp_down, groups)
@@ -522,7 +524,8 @@ def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
             and cfg.n_active_routed_experts <= 8 and cfg.padded_vocab_size % 128 == 0)
 
 
-def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None):
+def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None,
+                      groups_out: list | None = None):
     from lyra_amd.kernels import decode_fused as F
 
     h = model.emb[tokens]
@@ -530,7 +533,7 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     pos = cache.pos
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
-        h = moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
+        h = moe_apply_fused(h, layer.mlp, cfg, groups_out) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply_fused(h, layer.mlp, cfg)
     normed = F.rmsnorm_proj(h, model.norm_scale, cfg.norm_eps)
     if hidden_out is not None:  # the residual stream after the last layer (the norm kernel completes it on its way)
         hidden_out.append(normed[2] if len(normed) > 2 else h)
@@ -542,11 +545,13 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     return logits, cache
 
 
-def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None):
+def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None,
+                groups_out: list | None = None):
     """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one).
-    ``hidden_out``: optional list that receives the residual stream after the last layer [B, C] (for parity checks)."""
+    ``hidden_out``: optional list that receives the residual stream after the last layer [B, C] (for parity checks);
+    ``groups_out``: optional list that receives the rows-per-expert tensor of every MoE layer (fused driver only)."""
     if _fused_supported(model, cfg):
-        return model_apply_fused(tokens, model, cache, cfg, hidden_out)
+        return model_apply_fused(tokens, model, cache, cfg, hidden_out, groups_out)
     h = model.emb[tokens].to(torch.bfloat16)
     cos_t, sin_t = _rope_tables(cfg, h.device)
     pos = cache.pos
