@@ -58,12 +58,11 @@ def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup):
 
     from lyra_amd.generate import GraphedDecoder
 
-    dec = GraphedDecoder(weights, cache, cfg, batch)
-    dec.tokens.copy_(torch.randint(0, cfg.vocab_size, (batch,), device=dec.tokens.device))
-
-    def one_step():
-        cache.pos.fill_(ctx - 1)  # every timed step runs at full context
-        dec.step()
+    # every timed step runs at full context: the captured step does not move the position (ctx - 1, the last cache row);
+    # each step decodes the tokens the step before it drew
+    dec = GraphedDecoder(weights, cache, cfg, batch, advance=False)
+    dec.tokens.copy_(torch.randint(0, cfg.vocab_size, (batch,), device=dec.tokens.device).to(torch.int32))
+    one_step = dec.step
 
     for _ in range(warmup):
         one_step()

@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 8
+#define LYRA_ABI_VERSION 9
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -204,6 +204,11 @@ int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, cons
 /* Same, but the row to normalise is the residual update that ends a MoE layer (lyra/model.py:557-567; what lyra_moe_combine
  * computes): x_out = bf16(residual + bf16(bf16(sum_k scores[b,k] * rows[dest[b*topk+k]]) * out_scale)), rows [B*topk, C]
  * bf16 in sorted order, scores [B, topk] float32, dest [B*topk] int32, topk <= 16.  Same aliasing rule. */
+/* Same for the first layer of a step: row b is the embedding row table[tokens[b]] (the gather of lyra/model.py:752; table
+ * [table_rows, C] bf16, tokens [B] int32 in [0, table_rows)), also copied to x_out [B,C] as the residual stream. */
+int lyra_rmsnorm_proj_embed(const void* table, const int32_t* tokens, int table_rows, void* x_out, const float* scale, void* h,
+                            const float* proj_t, const float* bias, void* y, int B, int C, int n, int mode, float eps,
+                            lyra_stream_t stream);
 int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, const int32_t* dest, int topk, const void* residual,
                               float out_scale, void* x_out, const float* scale, void* h, const float* proj_t, const float* bias,
                               void* y, int B, int C, int n, int mode, float eps, lyra_stream_t stream);
@@ -249,9 +254,12 @@ int lyra_moe_combine(const void* rows, const float* scores, const int32_t* dest,
  * x[r, 0:cols], x float32 [rows, ld] (ld >= cols is the padded vocabulary; the padding is not looked at).
  * workspace: lyra_argmax_workspace bytes, 256-byte aligned, zero on first use (it holds arrival counters that
  * every call returns to zero, like the attention workspace).  ld % 4 == 0, x 16-byte aligned.
+ * advance (or NULL): an int32 on the device that the launch increments by one once row 0 is decided - the cache position,
+ * when the sampler is the last kernel of a decode step (lyra/generate.py:64-85 feeds position + 1 to the next step), so
+ * that a captured step can be replayed token after token without host work in between.
  */
 int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols, int ld,
-                lyra_stream_t stream);
+                int32_t* advance, lyra_stream_t stream);
 size_t lyra_argmax_workspace(int rows, int cols);
 
 /*
@@ -259,10 +267,10 @@ size_t lyra_argmax_workspace(int rows, int cols);
  * x[r, 0:cols] / temperature (ties go to the lower index, as lax.top_k), softmax over them, and the inverse CDF at
  * uniforms[r] in [0, 1) taken in that order: out[r] = index of the drawn column.  The reference draws with
  * jax.random.categorical from its own key stream; the distribution is the same, the caller supplies the randomness.
- * 1 <= k <= 8; x float32 [rows, ld], ld % 4 == 0, 16-byte aligned; workspace as for lyra_argmax (zero on first use).
+ * 1 <= k <= 8; x float32 [rows, ld], ld % 4 == 0, 16-byte aligned; workspace and advance as for lyra_argmax.
  */
 int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
-                     int cols, int ld, int k, float temperature, lyra_stream_t stream);
+                     int cols, int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream);
 size_t lyra_sample_topk_workspace(int rows, int cols, int k);
 
 

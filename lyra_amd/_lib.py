@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _c = ctypes
 SIGNATURES = {
@@ -55,6 +55,10 @@ SIGNATURES = {
         _c.c_int,
         [_c.c_void_p] * 2 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
     ),
+    "lyra_rmsnorm_proj_embed": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
+    ),
     "lyra_rmsnorm_proj_combine": (
         _c.c_int,
         [_c.c_void_p] * 3 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
@@ -63,9 +67,9 @@ SIGNATURES = {
         _c.c_int,
         [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int] + [_c.c_void_p] * 6 + [_c.c_int] * 7 + [_c.c_float, _c.c_void_p],
     ),
-    "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p]),
+    "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p] * 2),
     "lyra_argmax_workspace": (_c.c_size_t, [_c.c_int] * 2),
-    "lyra_sample_topk": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p]),
+    "lyra_sample_topk": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p, _c.c_void_p]),
     "lyra_sample_topk_workspace": (_c.c_size_t, [_c.c_int] * 3),
     "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
 }

@@ -51,6 +51,8 @@ struct NormProjParams {
     const float* comb_scores;   // [B, topk]
     const int32_t* comb_dest;   // [B, topk] sorted row of every assignment
     int comb_topk;              // <= 16
+    // or: row b is row row_index[b] of x (the embedding table: the token gather of lyra/model.py:752), copied to x_out
+    const int32_t* row_index;   // [B] or null
 };
 
 constexpr int kNormThreads = 1024;
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     // row again (cheap: the input comes from L2) so that the projection matrix, which every row needs in full, is pulled
     // through 4 compute units per row instead of one; share 0 writes the row's other outputs.
     const int b = blockIdx.x, share = blockIdx.y, shares = gridDim.y;
-    const uint16_t* xr = p.x + (size_t)b * p.C;
+    const uint16_t* xr = p.x + (size_t)(p.row_index ? p.row_index[b] : b) * p.C;
     float ss = 0.f;
     [[maybe_unused]] int comb_row[16];
     [[maybe_unused]] float comb_sc[16];
@@ -121,6 +123,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
             if (share == 0) *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
         } else {
             d = *(const u32x2*)(xr + c);
+            if (p.row_index && share == 0) *(u32x2*)(p.x_out + (size_t)b * p.C + c) = d;
         }
         const float v0 = __uint_as_float(d[0] << 16), v1 = __uint_as_float(d[0] & 0xFFFF0000u);
         const float v2 = __uint_as_float(d[1] << 16), v3 = __uint_as_float(d[1] & 0xFFFF0000u);
@@ -482,6 +485,7 @@ struct ArgmaxParams {
     int* part_i;     // [rows, chunks]
     int* arrivals;   // [rows] zero on entry, zero again on exit
     int rows, cols, ld, chunks, chunk_len;
+    int32_t* advance;  // or null: a counter (the cache position) that the launch increments by one when row 0 is done
 };
 
 __device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
@@ -540,7 +544,10 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
         take_better(bv, bi, load_agent(&p.part_v[row * p.chunks + k]), __hip_atomic_load(&p.part_i[row * p.chunks + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
-    if (threadIdx.x == 0) p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
+    if (threadIdx.x == 0) {
+        p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
+        if (p.advance && row == 0) *p.advance += 1;
+    }
 }
 
 // ---- temperature / top-k sampling ---------------------------------------------------------------------------------
@@ -560,6 +567,7 @@ struct SampleParams {
     int* arrivals;   // [rows] zero on entry, zero again on exit
     int rows, cols, ld, chunks, chunk_len, k;
     float temperature;
+    int32_t* advance;  // as in ArgmaxParams
 };
 
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
@@ -698,6 +706,7 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
             }
         }
         p.out[row] = pick;
+        if (p.advance && row == 0) *p.advance += 1;
     }
 }
 
@@ -729,7 +738,20 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
-                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0};
+                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr};
+    return launch_rmsnorm_proj(p, B, stream);
+}
+
+extern "C" int lyra_rmsnorm_proj_embed(const void* table, const int32_t* tokens, int table_rows, void* x_out, const float* scale, void* h,
+                                       const float* proj_t, const float* bias, void* y, int B, int C, int n, int mode, float eps,
+                                       lyra_stream_t stream) {
+    using namespace lyra;
+    if (!table || !tokens || !x_out || table_rows <= 0) return LYRA_E_BADARG;
+    if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
+    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
+    NormProjParams p{(const uint16_t*)table, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
+                     nullptr, 0, B, nullptr, 1.0f, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, tokens};
     return launch_rmsnorm_proj(p, B, stream);
 }
 
@@ -743,7 +765,7 @@ extern "C" int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, 
     if (C % 4 || C > 32768 || topk > 16) return LYRA_E_UNSUPPORTED;
     NormProjParams p{nullptr, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      nullptr, 0, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out,
-                     (const uint16_t*)rows, scores, dest, topk};
+                     (const uint16_t*)rows, scores, dest, topk, nullptr};
     return launch_rmsnorm_proj(p, B, stream);
 }
 
@@ -825,7 +847,7 @@ extern "C" size_t lyra_argmax_workspace(int rows, int cols) {
 }
 
 extern "C" int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols, int ld,
-                           lyra_stream_t stream) {
+                           int32_t* advance, lyra_stream_t stream) {
     using namespace lyra;
     if (!x || !out || rows <= 0 || cols <= 0 || ld < cols) return LYRA_E_BADARG;
     if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535 || cols > (1 << 28)) return LYRA_E_UNSUPPORTED;
@@ -833,6 +855,7 @@ extern "C" int lyra_argmax(const float* x, int32_t* out, void* workspace, size_t
     ArgmaxParams p;
     p.x = x;
     p.out = out;
+    p.advance = advance;
     p.rows = rows;
     p.cols = cols;
     p.ld = ld;
@@ -853,7 +876,7 @@ extern "C" size_t lyra_sample_topk_workspace(int rows, int cols, int k) {
 }
 
 extern "C" int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
-                                int cols, int ld, int k, float temperature, lyra_stream_t stream) {
+                                int cols, int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream) {
     using namespace lyra;
     if (!x || !uniforms || !out || rows <= 0 || cols <= 0 || ld < cols || k <= 0 || !(temperature > 0.f)) return LYRA_E_BADARG;
     if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535 || k > kMaxSampleK) return LYRA_E_UNSUPPORTED;
@@ -863,6 +886,7 @@ extern "C" int lyra_sample_topk(const float* x, const float* uniforms, int32_t* 
     p.x = x;
     p.uniforms = uniforms;
     p.out = out;
+    p.advance = advance;
     p.rows = rows;
     p.cols = cols;
     p.ld = ld;

@@ -139,6 +139,27 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
     return h, y
 
 
+def embed_rmsnorm_proj(table: torch.Tensor, tokens: torch.Tensor, scale: torch.Tensor, eps: float,
+                       proj: torch.Tensor | None = None, bias: torch.Tensor | None = None, gate: bool = False):
+    """The first norm of a decode step with the token gather folded in (lyra/model.py:752 + :303): rows
+    ``table[tokens]`` (table [V,C] bf16, tokens [B] int32) are normalised as in ``rmsnorm_proj``; returns (h, y | None, x)
+    with x [B,C] the gathered rows, i.e. the residual stream."""
+    V, C = table.shape
+    B = tokens.shape[0]
+    assert table.dtype == torch.bfloat16 and table.is_contiguous() and tokens.dtype == torch.int32 and tokens.is_contiguous()
+    x = torch.empty((B, C), dtype=torch.bfloat16, device=table.device)
+    h = torch.empty_like(x)
+    y, n = None, 0
+    if proj is not None:
+        n = proj.shape[1]
+        y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=x.device)
+        proj = _f32(_transposed(proj))
+    rc = _L.lyra_rmsnorm_proj_embed(table.data_ptr(), tokens.data_ptr(), V, x.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(),
+                                    _ptr(proj), _ptr(bias), _ptr(y), B, C, n, 1 if gate else 2, float(eps), _stream(x.device))
+    _lib.check(rc, "lyra_rmsnorm_proj_embed")
+    return h, y, x
+
+
 def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
              n_heads: int, n_kv_heads: int, head_dim: int, eps: float, unit_v: bool = False):
     """QK norm + rotary embedding + KV-cache append (quantising for an FP8 cache) for one new token per sequence
@@ -247,9 +268,11 @@ def moe_combine(rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, x:
     return out
 
 
-def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | None = None,
+           advance: torch.Tensor | None = None) -> torch.Tensor:
     """Greedy token choice (lyra/generate.py:46-53 at temperature 0): first index of each row's maximum over the first
-    ``cols`` columns of float32 ``logits`` [rows, ld]; returns int32 [rows]."""
+    ``cols`` columns of float32 ``logits`` [rows, ld]; returns int32 [rows].  ``advance``: an int32 device scalar (the
+    cache position) the launch increments by one."""
     rows, ld = logits.shape
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
@@ -258,13 +281,14 @@ def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | No
     assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_argmax_workspace(rows, cols))
-    rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, stream)
+    assert advance is None or (advance.dtype == torch.int32 and advance.numel() == 1)
+    rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, _ptr(advance), stream)
     _lib.check(rc, "lyra_argmax")
     return out
 
 
 def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperature: float, cols: int | None = None,
-                out: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, advance: torch.Tensor | None = None) -> torch.Tensor:
     """Temperature / top-k token choice (lyra/generate.py:46-53 at temperature > 0) for every row of float32 ``logits``
     [rows, ld] over its first ``cols`` columns: softmax of the k largest ``logits / temperature`` (ties to the lower
     index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows]."""
@@ -278,6 +302,6 @@ def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperatur
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_sample_topk_workspace(rows, cols, k))
     rc = _L.lyra_sample_topk(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,
-                             float(temperature), stream)
+                             float(temperature), _ptr(advance), stream)
     _lib.check(rc, "lyra_sample_topk")
     return out

@@ -441,6 +441,14 @@ _ONE_GROUP: dict = {}
 _SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tuning override: combine in a launch of its own
 
 
+@dataclass
+class TokenRows:
+    """The residual stream before the first layer, not gathered yet: rows ``table[tokens]``."""
+
+    table: torch.Tensor   # [V, C] bf16
+    tokens: torch.Tensor  # [B] int32
+
+
 def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
     """attention_apply as 5 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append | attention | output matmul.
     ``x`` is the residual stream or an ``Unsummed`` projection that still has to be added to it; the return value likewise
@@ -448,7 +456,9 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     from lyra_amd.kernels import decode_fused as F
 
     H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
-    if isinstance(x, (F.Unsummed, F.Uncombined)):
+    if isinstance(x, TokenRows):  # first layer of a step: the embedding rows are gathered by the norm kernel
+        h, gate, x = F.embed_rmsnorm_proj(x.table, x.tokens, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+    elif isinstance(x, (F.Unsummed, F.Uncombined)):
         h, gate, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
     else:
         h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
@@ -525,11 +535,12 @@ def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
 
 
 def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None,
-                      groups_out: list | None = None):
+                      groups_out: list | None = None, advance: bool = True):
     from lyra_amd.kernels import decode_fused as F
 
-    h = model.emb[tokens]
-    cos_t, sin_t = _rope_tables(cfg, h.device)
+    # int32 token ids are gathered by the first norm kernel (one launch fewer, and a sampler can write them in place)
+    h = TokenRows(model.emb, tokens) if tokens.dtype == torch.int32 and tokens.is_contiguous() else model.emb[tokens]
+    cos_t, sin_t = _rope_tables(cfg, model.emb.device)
     pos = cache.pos
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
@@ -541,18 +552,20 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
     if model.vocab_mask is None:
         logits[:, cfg.vocab_size :] = float("-inf")
-    cache.pos += 1
+    if advance:
+        cache.pos += 1
     return logits, cache
 
 
 def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None,
-                groups_out: list | None = None):
+                groups_out: list | None = None, advance: bool = True):
     """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one).
     ``hidden_out``: optional list that receives the residual stream after the last layer [B, C] (for parity checks);
-    ``groups_out``: optional list that receives the rows-per-expert tensor of every MoE layer (fused driver only)."""
+    ``groups_out``: optional list that receives the rows-per-expert tensor of every MoE layer (fused driver only);
+    ``advance=False`` leaves ``cache.pos`` where it is (the caller's sampler advances it, or nobody does)."""
     if _fused_supported(model, cfg):
-        return model_apply_fused(tokens, model, cache, cfg, hidden_out, groups_out)
-    h = model.emb[tokens].to(torch.bfloat16)
+        return model_apply_fused(tokens, model, cache, cfg, hidden_out, groups_out, advance)
+    h = model.emb[tokens.long()].to(torch.bfloat16)
     cos_t, sin_t = _rope_tables(cfg, h.device)
     pos = cache.pos
     cos, sin = cos_t.index_select(0, pos.to(torch.int64).reshape(1))[0], sin_t.index_select(0, pos.to(torch.int64).reshape(1))[0]
@@ -564,7 +577,8 @@ def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cf
     h = rms_norm(h, model.norm_scale, cfg.norm_eps)
     logits = _dense(h, model.unemb_t, cfg, out_f32=True)  # f32 logits (model.py:784-790)
     logits[:, cfg.vocab_size :] = float("-inf")
-    cache.pos += 1
+    if advance:
+        cache.pos += 1
     return logits, cache
 
 

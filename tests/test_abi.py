@@ -64,8 +64,8 @@ def test_argument_validation_needs_no_gpu():
     assert L.lyra_qkv_post(one, None, None, one, one, one, 0, one, one, one, None, None, None, 1, 4, 2, 16, 96, 16, 0, 1e-5, None) == -2
     assert L.lyra_moe_route(one, one, one, one, one, 4, 15, 1, 9, None) == -2  # more than 8 routed picks
     assert L.lyra_moe_combine(None, None, None, None, None, 1, 1, 1, 1.0, None) == -1
-    assert L.lyra_argmax(None, None, None, 0, 1, 1, 4, None) == -1
-    assert L.lyra_argmax(one, one, None, 0, 2, 10, 6, None) == -1  # leading dimension shorter than the row
+    assert L.lyra_argmax(None, None, None, 0, 1, 1, 4, None, None) == -1
+    assert L.lyra_argmax(one, one, None, 0, 2, 10, 6, None, None) == -1  # leading dimension shorter than the row
 
 
 def test_workspace_sizes_are_host_arithmetic():

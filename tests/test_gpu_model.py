@@ -97,10 +97,61 @@ def test_dev_model_per_channel_scales_and_graph_replay():
     dec.tokens.copy_(tok)
     for _ in range(3):
         cache.pos.fill_(17)
+        dec.tokens.copy_(tok)  # (the step replaces its tokens by the ones it drew)
         nxt = dec.step()
         torch.cuda.synchronize()
         assert torch.equal(dec.logits[:, : cfg.vocab_size], eager[:, : cfg.vocab_size])
         assert torch.equal(nxt.long(), eager.argmax(-1))
+        assert int(cache.pos.item()) == 18  # the sampler moved the position on
+
+
+def test_chained_replays_equal_eager_generate_calls_token_for_token():
+    """lyra/generate.py:64-85: every drawn token is the next step's input at the next position.  Four replays of the
+    captured step, chained on the device with no host work between them (the sampler writes the tokens where the next
+    step's first kernel reads them and advances the position), against four eager generate() calls."""
+    from lyra_amd.generate import GraphedDecoder, generate
+    from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights
+
+    cfg = apply_inference_overrides(replace(MODEL_VARIANTS["dev"], implementation="pallas", sample_temperature=0.0, seq_len=256),
+                                    fp8=True, fp8_attn=True, per_channel=True)
+    dev = U.dev()
+    w = init_weights(cfg, dev, seed=3)
+    B, start, n = 5, 30, 4
+    first = torch.tensor([5, 9, 700, 1, 33], device=dev, dtype=torch.int32)
+
+    def history(cache):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(11)
+        from lyra_amd.nn.quant import quantize
+
+        for layer in cache.layers:
+            for dst in (layer.k, layer.v):
+                hist = torch.randn(B, cfg.n_kv_heads, start, cfg.head_dim, device=dev, generator=gen).to(torch.bfloat16)
+                q = quantize(hist, dst.dtype, dst.block)
+                dst.qval.view(torch.uint8)[:, :, :start] = q.qval.view(torch.uint8)
+                dst.scale[:, :, :start] = q.scale
+        cache.pos.fill_(start)
+        return cache
+
+    eager_cache = history(init_cache(cfg, B, 256, dev))
+    tok, want = first, []
+    for _ in range(n):
+        tok, eager_cache = generate(tok, w, eager_cache, cfg)
+        want.append(tok.clone())
+    want = torch.stack(want)
+    assert int(eager_cache.pos.item()) == start + n
+
+    cache = history(init_cache(cfg, B, 256, dev))
+    dec = GraphedDecoder(w, cache, cfg, batch=B)
+    dec.tokens.copy_(first)
+    got = dec.decode(n)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert int(cache.pos.item()) == start + n
+    # the appended cache rows are the same bits either way
+    for a, b in zip(cache.layers, eager_cache.layers):
+        assert torch.equal(a.k.qval.view(torch.uint8)[:, :, start : start + n], b.k.qval.view(torch.uint8)[:, :, start : start + n])
+        assert torch.equal(a.v.scale[:, :, start : start + n], b.v.scale[:, :, start : start + n])
 
 
 def _layer_by_layer(cfg, w, cache, pos_value, layer_inputs, margins, margin):
@@ -294,6 +345,7 @@ def test_graphed_decoder_samples_inside_the_graph():
     draws = []
     for _ in range(12):
         cache.pos.fill_(9)
+        dec.tokens.copy_(torch.arange(8, device=dev) + 3)
         nxt = dec.step()
         torch.cuda.synchronize()
         top4 = torch.topk(dec.logits[:, : cfg.vocab_size], 4, dim=-1).indices
