@@ -41,6 +41,7 @@ struct GemmParams {
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
     int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
     int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
+    int snake;          // grouped kernel: odd rounds of units run over the workgroups in the opposite direction (-1: if >= 4 rounds)
     int even_spans;     // plain kernel: spans dealt out evenly over one workgroup per compute unit
     int row_block;      // K-split kernel: rows per workgroup (64 or 32)
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
@@ -1010,6 +1011,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 
     // state of the work item whose operands are in flight / being consumed
     int v = blockIdx.x;
+    bool seg_valid = false;
     int seg_u = 0, seg_r0 = 0, seg_r1 = 0;  // its unit and trips [r0, r1) of it
     int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
     __amdgpu_buffer_rsrc_t wrsrc;
@@ -1022,8 +1024,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         const_cast<float*>(FP8 ? p.scale : nullptr), 0, FP8 ? (uint32_t)p.G * (uint32_t)p.KB * (uint32_t)p.NB * 4u : 0u, 0x00020000);
 
     // Looks work item vv up and requests its first DEPTH steps (an item past the end requests nothing).
+    // After full rounds, the left-over units go to the workgroups at the far end: the heavy units come first in the list, so
+    // the workgroups at the near end have had the most to do in the first round (lyra-medium expert matmuls at 64 tokens:
+    // -10 %).  With four or more full rounds, odd rounds also run over the workgroups in the opposite direction, which evens
+    // out what is left of that slope (lyra-max up projection at 128 tokens: -5 %; with two rounds it costs 4 %).
+    const bool snake = p.snake < 0 ? n_whole >= 4 * (int)nwg : p.snake != 0;
     auto open_segment = [&](int vv) {
-        const bool valid = vv < n_work;
+        bool valid = vv < n_work;
+        if (n_whole > 0 && vv >= n_whole) {
+            const int rev = (int)nwg - 1 - (vv - n_whole);
+            valid = rev >= 0 && rev < tail;
+            vv = n_whole + rev;
+        } else if (snake && vv < n_whole && ((vv / (int)nwg) & 1)) {
+            const int r = vv / (int)nwg;
+            vv = r * (int)nwg + ((int)nwg - 1 - (vv - r * (int)nwg));  // odd rounds run the other way
+        }
+        seg_valid = valid;
         if constexpr (SLICED) {
             const int ti = vv - n_whole;  // >= 0: slice ti / tail of tail unit ti % tail
             const int sl = (valid && ti >= 0) ? ti / tail : 0;
@@ -1079,7 +1095,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         p.part, 0, (uint32_t)(kGroupMaxWgs * 16 * MTM) * (uint32_t)tile_cols * 4u, 0x00020000);
 
     open_segment(v);
-    while (v < n_work) {
+    while (seg_valid) {
         const int cur_u = seg_u, r0 = seg_r0, r1 = seg_r1;
         const int cur_g = g, cur_row0 = row0, cur_rows = rows, cur_span = span, cur_ncol = ncol;
         const int n_mt = (cur_rows + 15) >> 4;
@@ -1585,6 +1601,11 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         return e ? atoi(e) : 64;
     }();
     p.max_slices = max_slices_env;
+    static const int snake_env = [] {
+        const char* e = getenv("LYRA_GEMM_SNAKE");  // tuning override, read once: 0 never, 1 always
+        return e ? atoi(e) : -1;
+    }();
+    p.snake = snake_env;
     p.even_spans = 0;
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
