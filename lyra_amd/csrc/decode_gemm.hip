@@ -886,9 +886,11 @@ __device__ __forceinline__ void finish4(const GemmParams& p, f32x4 v, f32x4 l, f
 // ---- several groups (MoE experts), a handful of rows each: workgroups walk a list of (row block, column span) units -----
 // A unit is up to 64 rows of one expert times one 128-column span over the whole K extent (256-1024 KB of weights).
 // Every workgroup first builds the same unit list in LDS from group_sizes (experts without rows contribute nothing, so
-// their weights are never read; the last groups - shared experts, which carry the most rows - come first) and then takes
-// units blockIdx.x, blockIdx.x + gridDim.x, ...: at any time the workgroups stream neighbouring column spans of the same
-// weight rows.  Within a unit its 4 wavefronts interleave over K in steps of 32 rows with DEPTH steps of weights and
+// their weights are never read; the units with the most rows, which cost the most, come first) and then takes one unit
+// of every round of gridDim.x units: at any time the workgroups stream neighbouring column spans of the same weight
+// rows, which is what keeps the DRAM pages they touch open (handing every workgroup a run of consecutive units
+// instead, so that shares could be cut to equal cost, was built and was 6-40 % slower for that reason).  The units left
+// over after the last full round go to the workgroups that had the lightest units in the first.  Within a unit its 4 wavefronts interleave over K in steps of 32 rows with DEPTH steps of weights and
 // activations in flight each; their partial tiles are summed through LDS in a fixed order and bias / SwiGLU / residual
 // follow.  The first operands of the next unit are requested before the current unit's tile is summed and written, so a
 // compute unit keeps streaming across unit boundaries.
@@ -925,6 +927,23 @@ __device__ __forceinline__ int wg_scan_exclusive(int v, int* sm4, int lane, int 
     return base + incl - v;
 }
 
+// The same over four 16-bit counts packed into 64 bits (no field may exceed 65535 in total).
+__device__ __forceinline__ unsigned long long wg_scan_exclusive4(unsigned long long v, unsigned long long* sm4, int lane, int wave,
+                                                                 unsigned long long& total) {
+    unsigned long long incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned long long u = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += u;
+    }
+    if (lane == 63) sm4[wave] = incl;
+    __syncthreads();
+    unsigned long long base = 0;
+    for (int wv = 0; wv < wave; ++wv) base += sm4[wv];
+    total = sm4[0] + sm4[1] + sm4[2] + sm4[3];
+    return base + incl - v;
+}
+
 // WIDE_DYN: an instantiation for launches without SwiGLU that may have enough units for the wider ones (decided below,
 // once the unit list is known; the other instantiations know their layout from the start).
 template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false>
@@ -935,7 +954,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     constexpr int TRIP = ROUNDS * DEPTH;  // steps of one wavefront per trip
     extern __shared__ float sm_part[];  // [kSplitWaves][16 * MTM][kSplitPitch]
     __shared__ int sm_blk[kMaxRowBlocks][3];  // (group, first row, rows) of every row block, heavy groups first
-    __shared__ int sm_scan[12];
+    __shared__ int sm_scan[8];
+    __shared__ unsigned long long sm_scan4[4];
     __shared__ int sm_last;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
@@ -993,6 +1013,30 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
         }
     }
+    if (n_blocks_all * (p.N >> 8) > (int)gridDim.x) {
+        // More than one round of units: the list is put in the order of cost, in four classes by the number of 16-row
+        // tiles a block fills - all blocks of 49-64 rows (in group order from the last group down), then those of 33-48,
+        // 17-32 and 1-16 rows - so that, whatever the order of the groups, the units at the end of the list are the light
+        // ones.  One prefix sum over the four counts, packed into 64 bits, places every block.  (A single round gains
+        // nothing from the order, and the second prefix sum would cost it 0.8 us.)
+        const int my_full = my_cnt / (16 * MTM), my_rem = my_cnt - my_full * (16 * MTM);
+        const int my_class = my_rem > 0 ? MTM - ((my_rem + 15) >> 4) : 0;  // class of the partly filled block
+        unsigned long long all4;
+        const unsigned long long before4 = wg_scan_exclusive4(
+            (unsigned long long)my_full + (my_rem > 0 ? 1ull << (16 * my_class) : 0ull), sm_scan4, lane, wave, all4);
+        int class_base = 0;  // blocks of the classes before my_class
+        for (int c = 0; c < my_class; ++c) class_base += (int)((all4 >> (16 * c)) & 0xFFFF);
+        const int full_base = (int)(before4 & 0xFFFF);
+        const int rem_at = class_base + (int)((before4 >> (16 * my_class)) & 0xFFFF) + (my_class == 0 ? my_full : 0);
+        for (int i = 0; i < my_blocks; ++i) {  // (after the barrier in the prefix sum: every block is written again, elsewhere)
+            const int j = i < my_full ? full_base + i : rem_at;
+            if (j < kMaxRowBlocks) {
+                sm_blk[j][0] = p.G - 1 - t;
+                sm_blk[j][1] = my_before + i * 16 * MTM;
+                sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
+            }
+        }
+    }
     __syncthreads();
     const int nwg = gridDim.x;
     // Without SwiGLU the wider units are taken when they still fill 1.75 rounds of workgroups (lyra-max down projection at
@@ -1010,7 +1054,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
 
     // state of the work item whose operands are in flight / being consumed
-    int v = blockIdx.x;
+    int v = blockIdx.x, round = 0;  // (v = round * nwg + blockIdx.x)
     bool seg_valid = false;
     int seg_u = 0, seg_r0 = 0, seg_r1 = 0;  // its unit and trips [r0, r1) of it
     int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
@@ -1035,9 +1079,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             const int rev = (int)nwg - 1 - (vv - n_whole);
             valid = rev >= 0 && rev < tail;
             vv = n_whole + rev;
-        } else if (snake && vv < n_whole && ((vv / (int)nwg) & 1)) {
-            const int r = vv / (int)nwg;
-            vv = r * (int)nwg + ((int)nwg - 1 - (vv - r * (int)nwg));  // odd rounds run the other way
+        } else if (snake && vv < n_whole && (round & 1)) {
+            vv = vv - (int)blockIdx.x + ((int)nwg - 1 - (int)blockIdx.x);  // odd rounds run the other way
         }
         seg_valid = valid;
         if constexpr (SLICED) {
@@ -1214,6 +1257,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         __builtin_amdgcn_sched_barrier(0);
         // the next item's first operands fly while this tile is summed and written
         v += nwg;
+        ++round;
         open_segment(v);
 
         float* mine = sm_part + wave * (16 * MTM * kSplitPitch);
