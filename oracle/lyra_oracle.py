@@ -31,6 +31,9 @@ formulas; the checks live in tests/test_oracle_*.py):
                                      gives 0; the component of t orthogonal to v^ is unchanged and the parallel one is
                                      scaled by 1 - tanh(alpha); head n uses kv head n // G (one-hot rows); scalar
                                      loops on H = 8
+* rope_tables / rotate ............. rotation of the complex pair (x_i, x_{i+H/2}) by pos * base^(-2i/H); YaRN branch:
+                                     magnitude (0.1 ln s + 1), untouched / interpolated pairs and the linear ramp between
+                                     the hand-computed landmarks 8.09 and 17.39 at the gpt-oss setting
 * sample_topk ....................... closed forms: k = 1 is the argmax, u -> 0 / u -> 1 pick the first / k-th
                                      candidate, ties to the lower index, frequencies over a grid of u against
                                      ``torch.softmax`` of the k largest logits / temperature

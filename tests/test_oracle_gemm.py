@@ -175,6 +175,40 @@ def test_rms_norm_and_rotate_against_torch():
     np.testing.assert_allclose(r[0, 32:], z.imag, rtol=1e-4, atol=1e-5)
 
 
+def test_yarn_rope_tables_landmarks():
+    """The YaRN branch of the rotary tables (lyra/model.py:164-174) at the gpt-oss setting (variants.py:62-80: base
+    150000, scale 32, original length 4096, head dim 64, beta 32, alpha 1), pinned by what the published method fixes:
+    the magnitude cos^2 + sin^2 = (0.1 ln(scale) + 1)^2 everywhere; frequencies that turn more than beta times within the
+    original length are left alone, those that turn less than alpha times are interpolated (angle / scale), and the
+    boundaries fall where i = (H/2) ln(L / (turns 2 pi)) / ln(base): 8.1 and 17.4 here (worked out by hand), so pairs
+    0..8 are untouched, 18..31 fully interpolated, and the ones between blend linearly."""
+    H, L, scale, base = 64, 4096, 32.0, 150000.0
+    cos, sin = O.rope_tables(L, H, rope_base=base, rope_scale=scale, ntk_alpha=1.0, ntk_beta=32.0)
+    assert cos.shape == (L * 32, 32)
+    conc = 0.1 * np.log(32.0) + 1.0
+    np.testing.assert_allclose(cos.astype(np.float64) ** 2 + sin.astype(np.float64) ** 2, conc * conc, rtol=2e-6)
+    plain = 1.0 / base ** (np.arange(32) / 32.0)  # radians per position of pair i without scaling
+    pos = 1000
+    angle = np.arctan2(sin[pos].astype(np.float64), cos[pos].astype(np.float64))  # mod 2 pi
+    wrap = lambda a: (a + np.pi) % (2 * np.pi) - np.pi
+    np.testing.assert_allclose(wrap(angle[:9] - pos * plain[:9]), 0.0, atol=2e-4)             # untouched
+    np.testing.assert_allclose(wrap(angle[18:] - pos * plain[18:] / scale), 0.0, atol=2e-6)   # interpolated
+    # between the landmarks the rate lies strictly between the two, falling from one to the other
+    rate = np.arctan2(sin[1].astype(np.float64), cos[1].astype(np.float64))  # radians per position (all < pi here)
+    share = (rate[9:18] - plain[9:18] / scale) / (plain[9:18] - plain[9:18] / scale)  # 1 = untouched, 0 = interpolated
+    assert np.all(share > 0) and np.all(share < 1) and np.all(np.diff(share) < 0)
+    np.testing.assert_allclose(np.diff(share), np.diff(share)[0], rtol=1e-3)  # a linear ramp ...
+    np.testing.assert_allclose(-1.0 / np.diff(share)[0], 17.39 - 8.09, rtol=2e-3)  # ... as long as the landmarks are apart
+    # the host-side tables of the package are the same numbers
+    from dataclasses import replace
+
+    from lyra_amd.model import MODEL_VARIANTS, precompute_freq_cis
+    cfg = replace(MODEL_VARIANTS["gpt-oss-20b"], seq_len=L)
+    assert cfg.rope_scale == scale and cfg.rope_base == base and cfg.head_dim == H
+    c2, s2 = precompute_freq_cis(cfg)
+    assert np.array_equal(c2, cos) and np.array_equal(s2, sin)
+
+
 def test_sample_topk_closed_forms():
     """lyra/generate.py:46-53 restated with a caller-supplied uniform number: k = 1 is the argmax whatever the number;
     u -> 0 picks the largest logit, u -> 1 the k-th largest; ties go to the lower index; and over a fine grid of uniform
