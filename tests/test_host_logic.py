@@ -196,6 +196,84 @@ def test_decode_step_driver_with_exclusive_self_attention_and_biases_on_cpu_matc
         assert np.abs(other[:, : cfg.vocab_size].numpy() - first[:, : cfg.vocab_size]).max() > 0.05, name
 
 
+def test_oracle_decode_step_skeleton_is_pinned_by_what_the_model_structure_fixes():
+    """oracle/decode_step.py is a composition of pinned pieces; the composition itself is pinned here by consequences of the
+    model's structure (lyra/model.py:284-374, 734-793) that do not depend on how the step is written down:
+      * with every output projection and every down projection zero, every layer adds nothing: the residual stream stays
+        the embedding rows through all layers, and the logits are the final norm of those rows times the unembedding
+        (torch), -inf beyond the vocabulary;
+      * the step writes, at the position it is given, the new token's keys - normalised, then rotated by that position -
+        and its values as projected (torch, complex rotation), and touches no other cache row;
+      * at position 0 with zero sinks' weight removed (sink logit -1e4) a token attends only to itself: the attention
+        output is its own value row whatever q and k are, so the first layer's contribution is out_proj(gate * v)."""
+    from lyra_amd.model import MODEL_VARIANTS, init_cache, init_weights
+
+    dev = torch.device("cpu")
+    cfg = replace(MODEL_VARIANTS["dev"], implementation="xla", seq_len=64, sliding_window=16, use_sdpa_output_gate=True)
+    w = init_weights(cfg, dev, seed=5)
+    for lw in w.layers:  # make the attention weights large enough that every piece matters
+        lw.attn.qkv = (lw.attn.qkv.float() * 8).to(torch.bfloat16)
+    tokens = np.asarray([11, 700, 42])
+    B, C, H, N, K = 3, cfg.n_embd, cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
+    bf = lambda t: t.to(torch.bfloat16).float()
+
+    # 1. layers that add nothing
+    wn = D.weights_to_numpy(w, cfg)
+    for lw in wn["layers"]:
+        lw["attn"]["out"] = np.zeros_like(lw["attn"]["out"])
+        lw["mlp"]["mlp_down"] = np.zeros_like(lw["mlp"]["mlp_down"])
+    cn = D.cache_to_numpy(init_cache(cfg, B, 64, dev))
+    hidden = []
+    logits = D.decode_step(tokens, wn, cn, 7, cfg, hidden_out=hidden)
+    emb = bf(w.emb.float()[torch.from_numpy(tokens)])
+    assert len(hidden) == cfg.n_layers + 1
+    for h in hidden:
+        assert np.array_equal(h, emb.numpy())
+    normed = bf(torch.nn.functional.rms_norm(emb, (C,), w.norm_scale.float(), eps=cfg.norm_eps))
+    want = normed @ w.unemb_t.float().reshape(C, -1)
+    np.testing.assert_allclose(logits[:, : cfg.vocab_size], want[:, : cfg.vocab_size].numpy(), rtol=1e-4, atol=1e-4)
+    assert np.isneginf(logits[:, cfg.vocab_size :]).all()
+
+    # 2. what the step writes into the cache (layer 0), and only there
+    wn = D.weights_to_numpy(w, cfg)
+    cn = D.cache_to_numpy(init_cache(cfg, B, 64, dev))
+    before_k = cn["k"][0].copy()
+    pos = 9
+    D.decode_step(tokens, wn, cn, pos, cfg)
+    a = w.layers[0].attn
+    hn = bf(torch.nn.functional.rms_norm(emb, (C,), a.norm_scale.float(), eps=cfg.norm_eps))
+    qkv = bf(hn @ a.qkv.float()[0])
+    k_new = qkv[:, N * H : (N + K) * H].reshape(B, K, H)
+    v_new = qkv[:, (N + K) * H :].reshape(B, K, H)
+    if cfg.use_qk_norm:
+        k_new = bf(torch.nn.functional.rms_norm(k_new, (H,), a.knorm_scale.float(), eps=cfg.norm_eps))
+    rate = 1.0 / cfg.rope_base ** (np.arange(0, H, 2) / H)
+    z = (k_new[..., : H // 2].numpy() + 1j * k_new[..., H // 2 :].numpy()) * np.exp(1j * pos * rate)
+    k_rot = bf(torch.from_numpy(np.concatenate([z.real, z.imag], -1).astype(np.float32)))
+    np.testing.assert_allclose(cn["k"][0][:, :, pos], k_rot.numpy(), rtol=2e-2, atol=2e-3)  # (one bf16 step of slack)
+    assert np.array_equal(cn["v"][0][:, :, pos], v_new.numpy())
+    untouched = np.ones(64, bool)
+    untouched[pos] = False
+    assert np.array_equal(cn["k"][0][:, :, untouched], before_k[:, :, untouched])
+
+    # 3. a lone token attends to itself
+    wn = D.weights_to_numpy(w, cfg)
+    for lw in wn["layers"]:
+        lw["attn"]["sinks"] = np.full_like(lw["attn"]["sinks"], -1e4)
+    wn["layers"] = wn["layers"][:1]
+    wn["layers"][0]["mlp"]["mlp_down"] = np.zeros_like(wn["layers"][0]["mlp"]["mlp_down"])
+    one_layer = replace(cfg, n_layers=1, mlp_map=cfg.mlp_map[:1])
+    cn = D.cache_to_numpy(init_cache(one_layer, B, 64, dev))
+    hidden = []
+    D.decode_step(tokens, wn, cn, 0, one_layer, hidden_out=hidden)
+    gate = bf(2 * torch.sigmoid(hn @ a.sdpa_gate.float()))  # [B, N]
+    G = N // K
+    own = bf(bf(v_new.repeat_interleave(G, dim=1)) * gate[:, :, None]).reshape(B, N * H)
+    contrib = bf(bf(own @ a.out.float()[0]) * one_layer.residual_scale)
+    np.testing.assert_allclose(hidden[1], bf(emb + contrib).numpy(), rtol=2e-2, atol=2e-2)
+    assert np.abs(contrib.numpy()).max() > 0.05  # (the contribution is not lost in that tolerance)
+
+
 def test_sampling():
     from lyra_amd.generate import sample_token
     from lyra_amd.model import MODEL_VARIANTS
