@@ -282,6 +282,23 @@ def test_many_experts_unit_list(G, M, K, N, swiglu):
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list")
 
 
+@pytest.mark.parametrize("K,N,swiglu", [(512, 2048, True), (512, 2048, False), (256, 8192, True), (256, 8192, False)])
+def test_units_listed_by_cost_over_several_rounds(K, N, swiglu):
+    """More (row block, column span) units than one round of workgroups: the row blocks are listed by cost class (full
+    blocks and 49-63 rows, 33-48, 17-32, 1-16 rows), the left-over units go to the far-end workgroups and, from four full
+    rounds on (the two wider shapes), odd rounds run backwards.  Experts with several full blocks plus a remainder of
+    every class, empty experts between them, a heavy expert in the middle of the list and rows left over at the end; the
+    result must not depend on any of that."""
+    sizes = np.array([3, 0, 200, 64, 0, 33, 17, 16, 1, 48, 49, 0, 32, 130, 5, 63] + [2, 0, 7, 11] * 8, np.int32)
+    G, M = sizes.size, int(sizes.sum()) + 6
+    c = _case(21, M, G, K, N, sizes, kind="fp8", block=(K, 1), bias=True, w_std=0.05)
+    _note(f"gemm cost-ordered unit list G={G} M={M} K={K} N={N} swiglu={swiglu}")
+    want = _want(c, swiglu, big=True)
+    first = _run(c, swiglu)
+    U.assert_close(first, want, what="cost-ordered unit list")
+    assert np.array_equal(_run(c, swiglu), first)
+
+
 @pytest.mark.parametrize("kind,block,swiglu", [
     ("fp8", (2048, 1), True), ("fp8", (2048, 1), False), ("fp8", (256, 256), True), ("bf16", None, False),
 ])
