@@ -50,6 +50,11 @@ struct GemmParams {
     int post_scale;
 };
 
+// Results go out with plain stores; only the float32 K slices that the next kernel sums are written through at agent
+// scope (store_through): a K-split launch leaves 3-8 MB of them, and written back at the end of the kernel instead they
+// cost the decode step 1.5 %.  (Writing every result through - expert outputs, logits - was measured too: 0.5 % slower than
+// the slices alone.)
+template <typename T> __device__ __forceinline__ void out_store(void* base, size_t off, T v) { *(T*)((char*)base + off) = v; }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
 // Index of the scale block (along K) that weight row k lies in.
@@ -179,9 +184,9 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
                                            int ks, bool store, bool is_lin_lane) {
     if (p.ksplit > 1) {
         if (store) {
-            float* dst = p.part + ((size_t)ks * p.M + row) * p.N + ncol;
-            *(f32x4*)dst = f32x4{t[0], t[1], t[2], t[3]};
-            *(f32x4*)(dst + 4) = f32x4{t[4], t[5], t[6], t[7]};
+            const size_t dst = (((size_t)ks * p.M + row) * p.N + ncol) * 4;
+            store_through(p.part, dst, f32x4{t[0], t[1], t[2], t[3]});
+            store_through(p.part, dst + 16, f32x4{t[4], t[5], t[6], t[7]});
         }
         return;
     }
@@ -206,14 +211,14 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
             for (int c = 0; c < 8; ++c) t[c] = residual_epilogue(p, t[c], (size_t)row * NO + out_col + c);
         }
         if (p.out_f32) {
-            float* dst = (float*)p.out + (size_t)row * NO + out_col;
-            *(f32x4*)dst = f32x4{t[0], t[1], t[2], t[3]};
-            *(f32x4*)(dst + 4) = f32x4{t[4], t[5], t[6], t[7]};
+            const size_t dst = ((size_t)row * NO + out_col) * 4;
+            out_store(p.out, dst, f32x4{t[0], t[1], t[2], t[3]});
+            out_store(p.out, dst + 16, f32x4{t[4], t[5], t[6], t[7]});
         } else {
             u32x4 d;
 #pragma unroll
             for (int c = 0; c < 4; ++c) d[c] = pack_bf16(t[2 * c], t[2 * c + 1]);
-            *(u32x4*)((uint16_t*)p.out + (size_t)row * NO + out_col) = d;
+            out_store(p.out, ((size_t)row * NO + out_col) * 2, d);
         }
     }
 }
@@ -433,12 +438,12 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
         for (int c = 0; c < 4; ++c) a[c] = residual_epilogue(p, a[c], (size_t)row * NO + col + c);
     }
     if (p.out_f32) {
-        *(f32x4*)((float*)p.out + (size_t)row * NO + col) = f32x4{a[0], a[1], a[2], a[3]};
+        out_store(p.out, ((size_t)row * NO + col) * 4, f32x4{a[0], a[1], a[2], a[3]});
     } else {
         u32x2 d;
         d[0] = pack_bf16(a[0], a[1]);
         d[1] = pack_bf16(a[2], a[3]);
-        *(u32x2*)((uint16_t*)p.out + (size_t)row * NO + col) = d;
+        out_store(p.out, ((size_t)row * NO + col) * 2, d);
     }
 }
 
@@ -628,20 +633,20 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
             o[0] = round_bf16(round_bf16(o[0]) * p.out_scale) + eres[0];
             o[1] = round_bf16(round_bf16(o[1]) * p.out_scale) + eres[1];
         }
-        if (p.out_f32) *(f32x2*)((float*)p.out + oidx) = f32x2{o[0], o[1]};
-        else *(uint32_t*)((uint16_t*)p.out + oidx) = pack_bf16(o[0], o[1]);
+        if (p.out_f32) out_store(p.out, oidx * 4, f32x2{o[0], o[1]});
+        else out_store(p.out, oidx * 2, pack_bf16(o[0], o[1]));
     } else {
         if (p.post_scale) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) v[c] = round_bf16(round_bf16(v[c]) * p.out_scale) + eres[c];
         }
         if (p.out_f32) {
-            *(f32x4*)((float*)p.out + oidx) = f32x4{v[0], v[1], v[2], v[3]};
+            out_store(p.out, oidx * 4, f32x4{v[0], v[1], v[2], v[3]});
         } else {
             u32x2 d;
             d[0] = pack_bf16(v[0], v[1]);
             d[1] = pack_bf16(v[2], v[3]);
-            *(u32x2*)((uint16_t*)p.out + oidx) = d;
+            out_store(p.out, oidx * 2, d);
         }
     }
 }
@@ -819,7 +824,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
             const f32x4 t = *(const f32x4*)(sm_part + wv * (64 * kSplitPitch) + r * kSplitPitch + 4 * q);
             v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
         }
-        *(f32x4*)(p.part + ((size_t)ks * p.M + row) * p.N + span * 128 + 4 * q) = v;
+        store_through(p.part, (((size_t)ks * p.M + row) * p.N + span * 128 + 4 * q) * 4, v);
     }
 }
 
@@ -841,12 +846,12 @@ __device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[
         o[c] = a;
     }
     if (p.out_f32) {
-        *(f32x4*)((float*)p.out + oidx) = f32x4{o[0], o[1], o[2], o[3]};
+        out_store(p.out, oidx * 4, f32x4{o[0], o[1], o[2], o[3]});
     } else {
         u32x2 d;
         d[0] = pack_bf16(o[0], o[1]);
         d[1] = pack_bf16(o[2], o[3]);
-        *(u32x2*)((uint16_t*)p.out + oidx) = d;
+        out_store(p.out, oidx * 2, d);
     }
 }
 
@@ -874,12 +879,12 @@ __device__ __forceinline__ void finish4(const GemmParams& p, f32x4 v, f32x4 l, f
         o[c] = a;
     }
     if (p.out_f32) {
-        *(f32x4*)((float*)p.out + oidx) = f32x4{o[0], o[1], o[2], o[3]};
+        out_store(p.out, oidx * 4, f32x4{o[0], o[1], o[2], o[3]});
     } else {
         u32x2 d;
         d[0] = pack_bf16(o[0], o[1]);
         d[1] = pack_bf16(o[2], o[3]);
-        *(u32x2*)((uint16_t*)p.out + oidx) = d;
+        out_store(p.out, oidx * 2, d);
     }
 }
 
@@ -1604,6 +1609,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
     if (K % 32 || N % 128 || (fused_swiglu && N % 256) || G > 8191) return LYRA_E_UNSUPPORTED;
+    if ((size_t)M * N * 4 >= (1ull << 31)) return LYRA_E_UNSUPPORTED;  // results are stored through 31-bit buffer offsets
 
     GemmParams p;
     p.scale_mode = 0;
@@ -1659,6 +1665,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         // the first kGemmCounterBytes belong to the grouped kernel's arrival counters, whichever kernel runs
         // (checked against the plan that is launched: never more than lyra_decode_gemm_workspace answers for the shape)
         const size_t need = kGemmCounterBytes + gemm_partial_bytes(pl, M, N);
+        if (need >= (1ull << 31)) return LYRA_E_UNSUPPORTED;
         if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 256)) return LYRA_E_WORKSPACE;
         p.arrivals = (int*)workspace;
         p.part = (float*)((char*)workspace + kGemmCounterBytes);
@@ -1807,6 +1814,7 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     }
     const GemmPlan pl = plan_gemm(M, 1, K, N, fp8 ? bk : 0, 0);
     if (!pl.split_k) return LYRA_E_UNSUPPORTED;
+    if ((size_t)pl.ksplit * M * N * sizeof(float) >= (1ull << 31)) return LYRA_E_UNSUPPORTED;
     if (partials_bytes < (size_t)pl.ksplit * M * N * sizeof(float) || ((uintptr_t)partials % 16)) return LYRA_E_WORKSPACE;
     p.lhs = (const uint16_t*)lhs;
     p.rhs = (const uint8_t*)rhs;

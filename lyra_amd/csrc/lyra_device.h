@@ -126,6 +126,44 @@ __device__ __forceinline__ int add_agent(int* p, int v) {
 __device__ __forceinline__ void store_agent(int* p, int v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Stores of results that a later kernel reads.  Every XCD has its own L2, so what a kernel leaves dirty there is written
+// back when the kernel ends, and the next kernel waits for that; a store at agent scope is written through as it is
+// issued, while the kernel still has work to do.
+__device__ __forceinline__ void store_through(uint16_t* p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_through(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_through(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_through(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_through(u32x2* p, u32x2 v) {
+    __hip_atomic_store((unsigned long long*)p, (unsigned long long)v[0] | ((unsigned long long)v[1] << 32), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_through(u32x4* p, u32x4 v) {
+    store_through((u32x2*)p, u32x2{v[0], v[1]});
+    store_through((u32x2*)p + 1, u32x2{v[2], v[3]});
+}
+__device__ __forceinline__ void store_through(f32x2* p, f32x2 v) { store_through((u32x2*)p, u32x2{__float_as_uint(v[0]), __float_as_uint(v[1])}); }
+__device__ __forceinline__ void store_through(f32x4* p, f32x4 v) {
+    store_through((u32x4*)p, u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])});
+}
+// ... and through a buffer descriptor on a wave-uniform base pointer (offsets in bytes, below 2 GB): 4, 8 and 16 bytes.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t through_rsrc(void* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7FFFFFFFu, 0x00020000);
+}
+__device__ __forceinline__ void store_through(void* base, size_t off, uint32_t v) {
+    __builtin_amdgcn_raw_buffer_store_b32(v, through_rsrc(base), (int)off, 0, 16);
+}
+__device__ __forceinline__ void store_through(void* base, size_t off, u32x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(v, through_rsrc(base), (int)off, 0, 16);
+}
+__device__ __forceinline__ void store_through(void* base, size_t off, u32x4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, through_rsrc(base), (int)off, 0, 16);
+}
+__device__ __forceinline__ void store_through(void* base, size_t off, f32x2 v) {
+    store_through(base, off, u32x2{__float_as_uint(v[0]), __float_as_uint(v[1])});
+}
+__device__ __forceinline__ void store_through(void* base, size_t off, f32x4 v) {
+    store_through(base, off, u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])});
+}
 __device__ __forceinline__ void wait_all_memory() { __builtin_amdgcn_s_waitcnt(0); }
 // 16-byte forms of store_agent / load_agent through a buffer descriptor (cache-policy bit 4 = sc1: agent scope on gfx950).
 __device__ __forceinline__ void store_agent_b128(__amdgpu_buffer_rsrc_t rsrc, int voff, f32x4 v) {
