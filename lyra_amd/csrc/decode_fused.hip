@@ -13,10 +13,9 @@ namespace lyra {
 
 __device__ __forceinline__ float bf16r(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
-__device__ __forceinline__ float block_sum(float v, float* sm) {  // blockDim.x <= 1024, multiple of 64
+__device__ __forceinline__ float block_sum(float v, float* sm) {  // blockDim.x <= 1024, multiple of 64; sm: 16 floats nobody else uses
     v = wave_sum(v);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-    __syncthreads();
     if (lane == 0) sm[wave] = v;
     __syncthreads();
     float t = lane < nw ? sm[lane] : 0.f;
@@ -60,13 +59,28 @@ constexpr int kNormThreads = 1024;
 // COMBINE: the instantiation whose rows come from a MoE layer's combine step (comb_rows set).
 template <bool COMBINE>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjParams p) {
-    extern __shared__ float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
+    extern __shared__ __align__(16) float sm_h[];  // [C] normalised row (bf16 values as float32), then 16 floats of reduction scratch
     float* sm_red = sm_h + p.C;
     // blockIdx.y: which share of the projection outputs this workgroup computes.  The shares of a row each normalise the
     // row again (cheap: the input comes from L2) so that the projection matrix, which every row needs in full, is pulled
     // through 4 compute units per row instead of one; share 0 writes the row's other outputs.
     const int b = blockIdx.x, share = blockIdx.y, shares = gridDim.y;
+    // The weights of the first projection output of this wavefront do not depend on the row: they are requested before
+    // anything else, so that they arrive while the row is being read and normalised (otherwise the projection is a
+    // second memory round trip behind the norm: 1.4 us of a 4.7 us launch).
+    const int per_share = (p.n + shares - 1) / shares, j_end = min(p.n, (share + 1) * per_share);
+    const int j_first = share * per_share + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // (the same in every lane)
+    u32x4 w_first[8];
+    if (p.proj_t && j_first < j_end) {  // (only the wavefronts that have an output: a load that fetches nothing still takes its
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(  // turn in the address unit)
+            const_cast<float*>(p.proj_t) + (size_t)j_first * p.C, 0, (uint32_t)p.C * 4u, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w_first[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (i * 256 + (int)(threadIdx.x & 63) * 4) * 4, 0, 0);
+    }
     const uint16_t* xr = p.x + (size_t)(p.row_index ? p.row_index[b] : b) * p.C;
+    // (the norm weights of this thread's first 4 columns, likewise requested ahead of the row)
+    const int c_first = min((int)threadIdx.x * 4, p.C - 4);
+    const f32x4 sc_first = *(const f32x4*)(p.scale + c_first);
     float ss = 0.f;
     [[maybe_unused]] int comb_row[16];
     [[maybe_unused]] float comb_sc[16];
@@ -106,9 +120,17 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
             f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
             for (int s0 = 0; s0 < p.splits; s0 += 8) {
                 u32x4 u[8];
+                if (p.splits - s0 <= 4) {  // (4 or fewer left: no loads for slices that do not exist)
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    u[j] = __builtin_amdgcn_raw_buffer_load_b128(pr, s0 + j < p.splits ? (s0 + j) * slab + mine : kNoLoad, 0, 0);
+                    for (int j = 0; j < 4; ++j)
+                        u[j] = __builtin_amdgcn_raw_buffer_load_b128(pr, s0 + j < p.splits ? (s0 + j) * slab + mine : kNoLoad, 0, 0);
+#pragma unroll
+                    for (int j = 4; j < 8; ++j) u[j] = u32x4{0u, 0u, 0u, 0u};
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        u[j] = __builtin_amdgcn_raw_buffer_load_b128(pr, s0 + j < p.splits ? (s0 + j) * slab + mine : kNoLoad, 0, 0);
+                }
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     t[0] += __uint_as_float(u[j][0]); t[1] += __uint_as_float(u[j][1]);
@@ -133,7 +155,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     ss = block_sum(ss, sm_red);
     const float inv = rsqrtf(ss / (float)p.C + p.eps);
     for (int c = threadIdx.x * 4; c < p.C; c += kNormThreads * 4) {  // each thread revisits its own elements
-        const f32x4 sc = *(const f32x4*)(p.scale + c);
+        const f32x4 sc = c == c_first ? sc_first : *(const f32x4*)(p.scale + c);
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = sm_h[c + i] * inv * sc[i];
@@ -148,9 +170,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     }
     if (!p.proj_t) return;
     __syncthreads();
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int per_share = (p.n + shares - 1) / shares, j_end = min(p.n, (share + 1) * per_share);
-    for (int j = share * per_share + wave; j < j_end; j += kNormThreads / 64) {
+    const int lane = threadIdx.x & 63;
+    for (int j = j_first; j < j_end; j += kNormThreads / 64) {
         // one output per wavefront at a time; its weight row is requested 8 x 16 bytes per lane at once (offsets past
         // the row read as zeros), so a row of up to 2048 columns costs one memory round trip
         const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.proj_t) + (size_t)j * p.C, 0,
@@ -158,8 +179,13 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
         float acc = 0.f;
         for (int c0 = 0; c0 < p.C; c0 += 2048) {
             u32x4 w[8];
+            if (j == j_first && c0 == 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (c0 + i * 256 + lane * 4) * 4, 0, 0);
+                for (int i = 0; i < 8; ++i) w[i] = w_first[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (c0 + i * 256 + lane * 4) * 4, 0, 0);
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int c = min(c0 + i * 256 + lane * 4, p.C - 4);  // (clamped reads meet zero weights)

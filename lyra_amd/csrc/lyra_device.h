@@ -184,15 +184,25 @@ __device__ __forceinline__ f32x4 load_agent_b128(__amdgpu_buffer_rsrc_t rsrc, in
 // waits for every global load the wavefront has in flight, which empties the prefetch queue of a streaming kernel.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Reductions over the 64 lanes of a wavefront, result in every lane: within a row of 16 lanes by DPP (lane pairs, quads,
+// mirrored halves of 8, mirrored row), then across the four rows by the lane swaps above.  A dozen ALU instructions; the
+// same butterfly through __shfl_xor goes through LDS six times (~0.3 us each time a small kernel reduces a row).
+template <int CTRL> __device__ __forceinline__ float dpp_row(float x) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, kWave));
-    return x;
+    x = fmaxf(x, dpp_row<0xB1>(x));   // quad_perm [1, 0, 3, 2]
+    x = fmaxf(x, dpp_row<0x4E>(x));   // quad_perm [2, 3, 0, 1]
+    x = fmaxf(x, dpp_row<0x141>(x));  // row_half_mirror
+    x = fmaxf(x, dpp_row<0x140>(x));  // row_mirror
+    return group4_max(x);
 }
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, kWave);
-    return x;
+    x += dpp_row<0xB1>(x);
+    x += dpp_row<0x4E>(x);
+    x += dpp_row<0x141>(x);
+    x += dpp_row<0x140>(x);
+    return group4_sum(x);
 }
 
 }  // namespace lyra
