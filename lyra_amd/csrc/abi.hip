@@ -99,8 +99,7 @@ __global__ __launch_bounds__(64) void selftest_kernel(int32_t* report) {
 
     int vals[7] = {bad_mfma, bad_cvt, bad_cvt_bf16, bad_pack, bad_perm, bad_denorm, bad_rows};
     for (int i = 0; i < 7; ++i) {
-        int v = vals[i];
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+        const int v = wave_sum(vals[i]);
         if (lane == 0) report[i] = v;
     }
     if (lane == 0) report[7] = LYRA_ABI_VERSION;

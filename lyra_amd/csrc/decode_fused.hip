@@ -377,14 +377,12 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
                     bi = e;
                 }
             }
-            for (int off = lanes >> 1; off > 0; off >>= 1) {
-                const float ov = __shfl_xor(best, off, 64);
-                const int oi = __shfl_xor(bi, off, 64);
-                if (oi != INT_MAX && (bi == INT_MAX || ov > best || (ov == best && oi < bi))) {
-                    best = ov;
-                    bi = oi;
+            wave_best(best, bi, [](float& v, int& i, float ov, int oi) {
+                if (oi != INT_MAX && (i == INT_MAX || ov > v || (ov == v && oi < i))) {
+                    v = ov;
+                    i = oi;
                 }
-            }
+            }, lanes);
             if (bi < 64) taken_lo |= 1ull << bi; else taken_hi |= 1ull << (bi - 64);
             top[j] = best;
             idx[j] = bi;
@@ -545,8 +543,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
                 if (i < hi) take_better(bv, bi, __uint_as_float(v[u][k]), i);
             }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+    wave_best(bv, bi, [](float& v, int& i, float ov, int oi) { take_better(v, i, ov, oi); });
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (lane == 0) {
         sm_v[wave] = bv;
@@ -568,8 +565,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(ArgmaxParams p) {
     bi = 0x7FFFFFFF;
     for (int k = threadIdx.x; k < p.chunks; k += 64)
         take_better(bv, bi, load_agent(&p.part_v[row * p.chunks + k]), __hip_atomic_load(&p.part_i[row * p.chunks + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) take_better(bv, bi, __shfl_xor(bv, o, kWave), __shfl_xor(bi, o, kWave));
+    wave_best(bv, bi, [](float& v, int& i, float ov, int oi) { take_better(v, i, ov, oi); });
     if (threadIdx.x == 0) {
         p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
         if (p.advance && row == 0) *p.advance += 1;
@@ -633,15 +629,12 @@ __device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[k
             }
         float bv = hv;
         int bi = hi;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, kWave);
-            const int oi = __shfl_xor(bi, o, kWave);
-            if (better(ov, oi, bv, bi)) {
-                bv = ov;
-                bi = oi;
+        wave_best(bv, bi, [](float& v, int& i, float ov, int oi) {
+            if (better(ov, oi, v, i)) {
+                v = ov;
+                i = oi;
             }
-        }
+        });
         if (lane == 0) {
             sm_wv[wave] = bv;
             sm_wi[wave] = bi;

@@ -245,8 +245,7 @@ void decode_gemm_kernel(GemmParams p) {
     // rows of this group: [off, off + cnt)
     int part_sum = 0;
     for (int i = lane; i < g; i += 64) part_sum += p.group_sizes[i];
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) part_sum += __shfl_xor(part_sum, o, kWave);
+    part_sum = wave_sum(part_sum);
     const int off = min(part_sum, p.M);
     const int cnt = min(p.group_sizes[g], p.M - off);
     const int pad_from = (g == p.G - 1 && rpar == 0 && p.ksplit == 1 && ks == 0) ? off + cnt : p.M;  // rows past the last group
@@ -918,12 +917,7 @@ constexpr size_t kGemmCounterBytes = 65536;  // start of a matmul workspace: arr
 
 // Exclusive prefix sum of one int per thread over the 256 threads of a workgroup (sm4: 4 ints of LDS, free on entry).
 __device__ __forceinline__ int wg_scan_exclusive(int v, int* sm4, int lane, int wave, int& total) {
-    int incl = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int u = __shfl_up(incl, o, kWave);
-        if (lane >= o) incl += u;
-    }
+    const int incl = wave_scan_inclusive(v);
     if (lane == 63) sm4[wave] = incl;
     __syncthreads();
     int base = 0;
@@ -935,12 +929,9 @@ __device__ __forceinline__ int wg_scan_exclusive(int v, int* sm4, int lane, int 
 // The same over four 16-bit counts packed into 64 bits (no field may exceed 65535 in total).
 __device__ __forceinline__ unsigned long long wg_scan_exclusive4(unsigned long long v, unsigned long long* sm4, int lane, int wave,
                                                                  unsigned long long& total) {
-    unsigned long long incl = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const unsigned long long u = __shfl_up(incl, o, kWave);
-        if (lane >= o) incl += u;
-    }
+    // (no field of the low or of the high word overflows into the other word, so the two words are summed on their own)
+    const unsigned long long incl = (unsigned long long)(unsigned)wave_scan_inclusive((int)(unsigned)v) |
+                                    ((unsigned long long)(unsigned)wave_scan_inclusive((int)(unsigned)(v >> 32)) << 32);
     if (lane == 63) sm4[wave] = incl;
     __syncthreads();
     unsigned long long base = 0;

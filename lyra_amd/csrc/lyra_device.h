@@ -187,9 +187,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // Reductions over the 64 lanes of a wavefront, result in every lane: within a row of 16 lanes by DPP (lane pairs, quads,
 // mirrored halves of 8, mirrored row), then across the four rows by the lane swaps above.  A dozen ALU instructions; the
 // same butterfly through __shfl_xor goes through LDS six times (~0.3 us each time a small kernel reduces a row).
-template <int CTRL> __device__ __forceinline__ float dpp_row(float x) {
-    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xF, 0xF, true));
-}
+template <int CTRL> __device__ __forceinline__ int dpp_row(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, true); }
+template <int CTRL> __device__ __forceinline__ float dpp_row(float x) { return __uint_as_float((uint32_t)dpp_row<CTRL>((int)__float_as_uint(x))); }
 __device__ __forceinline__ float wave_max(float x) {
     x = fmaxf(x, dpp_row<0xB1>(x));   // quad_perm [1, 0, 3, 2]
     x = fmaxf(x, dpp_row<0x4E>(x));   // quad_perm [2, 3, 0, 1]
@@ -203,6 +202,50 @@ __device__ __forceinline__ float wave_sum(float x) {
     x += dpp_row<0x141>(x);
     x += dpp_row<0x140>(x);
     return group4_sum(x);
+}
+__device__ __forceinline__ int wave_sum(int x) {
+    x += dpp_row<0xB1>(x);
+    x += dpp_row<0x4E>(x);
+    x += dpp_row<0x141>(x);
+    x += dpp_row<0x140>(x);
+    const uint32_t u = (uint32_t)x;
+    auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t t = h[0] + h[1];
+    auto r = __builtin_amdgcn_permlane16_swap(t, t, false, false);
+    return (int)(r[0] + r[1]);
+}
+// The same butterfly for a (value, index) pair with a caller's rule: take(v, i, ov, oi) replaces (v, i) by (ov, oi) where
+// the other pair wins.  The rule must not depend on the order in which pairs meet (a total order with ties broken by index).
+// `lanes`: how many neighbouring lanes (a power of two, aligned) form one group; 64 = the whole wavefront.
+template <typename Take>
+__device__ __forceinline__ void wave_best(float& v, int& i, Take take, int lanes = 64) {
+    if (lanes > 1) take(v, i, dpp_row<0xB1>(v), dpp_row<0xB1>(i));
+    if (lanes > 2) take(v, i, dpp_row<0x4E>(v), dpp_row<0x4E>(i));
+    if (lanes > 4) take(v, i, dpp_row<0x141>(v), dpp_row<0x141>(i));
+    if (lanes > 8) take(v, i, dpp_row<0x140>(v), dpp_row<0x140>(i));
+    if (lanes > 16) {
+        auto rv = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        auto ri = __builtin_amdgcn_permlane16_swap((uint32_t)i, (uint32_t)i, false, false);
+        v = __uint_as_float(rv[0]), i = (int)ri[0];
+        take(v, i, __uint_as_float(rv[1]), (int)ri[1]);
+    }
+    if (lanes > 32) {
+        auto hv = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        auto hi = __builtin_amdgcn_permlane32_swap((uint32_t)i, (uint32_t)i, false, false);
+        v = __uint_as_float(hv[0]), i = (int)hi[0];
+        take(v, i, __uint_as_float(hv[1]), (int)hi[1]);
+    }
+}
+// Inclusive prefix sum over the lanes of a wavefront: within rows of 16 by shifted DPP reads, then the last lane of a row
+// (of the first half) is added to the rows behind it.
+__device__ __forceinline__ int wave_scan_inclusive(int x) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);  // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);  // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);  // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);  // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+    return x;
 }
 
 }  // namespace lyra
