@@ -243,21 +243,35 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
     const int b = item / heads, hd = item - b * heads;
     const int half = p.H >> 1;
     const bool active = lane < half;
+    // Everything that does not depend on the projection is requested first, in the order of its own dependencies - the
+    // position, then the rotary row it selects, and the norm weights - so that the row's values, which come last out of
+    // the kernel before, are the only thing the wavefront still waits for when they arrive.
+    const int pos = p.position[(size_t)b * p.pos_stride];
+    const bool is_q = hd < p.N, is_k = !is_q && hd < p.N + p.K;
+    const float* ns = is_q ? p.qnorm : (is_k ? p.knorm : nullptr);
+    float ns_a = 0.f, ns_c = 0.f, cs = 0.f, sn = 0.f;
+    if ((is_q || is_k) && active) {
+        if (ns) ns_a = ns[lane], ns_c = ns[lane + half];
+        const int rp = min(max(pos, 0), p.seq - 1);
+        cs = p.cos_t[(size_t)rp * half + lane];
+        sn = p.sin_t[(size_t)rp * half + lane];
+    }
     float a = 0.f, c = 0.f;
     if (p.partials) {
         if (active) {
             const size_t slab = (size_t)p.B * heads * p.H;
             const float* src = p.partials + ((size_t)b * heads + hd) * p.H;
-            for (int s0 = 0; s0 < p.splits; s0 += 8) {  // 8 slices in flight; added in slice order
-                float ua[8], uc[8];
+            for (int s0 = 0; s0 < p.splits; s0 += 4) {  // 4 slices in flight; added in slice order
+                float ua[4], uc[4];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int sidx = min(s0 + j, p.splits - 1);
-                    ua[j] = src[sidx * slab + lane];
-                    uc[j] = src[sidx * slab + lane + half];
+                for (int j = 0; j < 4; ++j) {
+                    if (s0 + j < p.splits) {
+                        ua[j] = src[(s0 + j) * slab + lane];
+                        uc[j] = src[(s0 + j) * slab + lane + half];
+                    }
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
+                for (int j = 0; j < 4; ++j) {
                     if (s0 + j < p.splits) {
                         a += ua[j];
                         c += uc[j];
@@ -272,19 +286,13 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
         a = bf16_bits_to_f32(src[lane]);
         c = bf16_bits_to_f32(src[lane + half]);
     }
-    const int pos = p.position[(size_t)b * p.pos_stride];
-    const bool is_q = hd < p.N, is_k = !is_q && hd < p.N + p.K;
     if (is_q || is_k) {
-        const float* ns = is_q ? p.qnorm : p.knorm;
         if (ns) {
             const float ss = wave_sum(a * a + c * c);
             const float inv = rsqrtf(ss / (float)p.H + p.eps);
-            a = bf16r(a * inv * (active ? ns[lane] : 0.f));
-            c = bf16r(c * inv * (active ? ns[lane + half] : 0.f));
+            a = bf16r(a * inv * ns_a);
+            c = bf16r(c * inv * ns_c);
         }
-        const int rp = min(max(pos, 0), p.seq - 1);
-        const float cs = active ? p.cos_t[(size_t)rp * half + lane] : 0.f;
-        const float sn = active ? p.sin_t[(size_t)rp * half + lane] : 0.f;
         const float ra = bf16r(a * cs - c * sn), rc = bf16r(c * cs + a * sn);
         a = ra;
         c = rc;

@@ -400,26 +400,40 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long)p.M * quads) return;
     const int row = (int)(idx / quads), col = (int)(idx - (long)row * quads) * 4;
+    // The slices are requested before the row's group is looked up (that is a chain of loads of its own, and the row exists
+    // whatever its group): 4 slices in flight, added in slice order.
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.ksplit; s0 += 4) {
+        f32x4 va[4], vb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j < p.ksplit) {
+                const float* src = p.part + ((size_t)(s0 + j) * p.M + row) * p.N;
+                va[j] = *(const f32x4*)(src + col);
+                if (p.swiglu) vb[j] = *(const f32x4*)(src + NO + col);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j < p.ksplit) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) a[c] += va[j][c];
+                if (p.swiglu) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) b[c] += vb[j][c];
+                }
+            }
+        }
+    }
     int total = 0, g = p.G - 1;
     for (int i = 0; i < p.G; ++i) {
         const int nt = total + p.group_sizes[i];
         if (row >= total && row < nt) g = i;
         total = nt;
     }
-    const bool live = row < total;
-    float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
-    if (live) {
-        for (int s = 0; s < p.ksplit; ++s) {
-            const float* src = p.part + ((size_t)s * p.M + row) * p.N;
-            const f32x4 va = *(const f32x4*)(src + col);
+    if (row >= total) {  // rows past the last group: zero product (lax.ragged_dot), bias of the last group
 #pragma unroll
-            for (int c = 0; c < 4; ++c) a[c] += va[c];
-            if (p.swiglu) {
-                const f32x4 vb = *(const f32x4*)(src + NO + col);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) b[c] += vb[c];
-            }
-        }
+        for (int c = 0; c < 4; ++c) a[c] = b[c] = 0.f;
     }
     if (p.bias) {
 #pragma unroll
