@@ -718,7 +718,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
         const int kk = step_row(d);
         const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
+        for (int mt = 0; mt < 4; ++mt) {  // (row tiles the block does not have are not requested: a load that fetches nothing
+            if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);  // still takes its turn)
+            else a[d][mt] = u32x4{0u, 0u, 0u, 0u};
+        }
     }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
@@ -776,7 +779,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
                 const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt)
-                    a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff[mt] : kNoLoad, soff, 0);
+                    if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff[mt] : kNoLoad, soff, 0);
 #pragma unroll
                 for (int pr = 0; pr < 4; ++pr) {
                     convert_pair<FP8>(w[d], pr, bop);
