@@ -1133,7 +1133,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             if (d < ADEPTH) {
 #pragma unroll
                 for (int mt = 0; mt < MTM; ++mt)
-                    a[d % ADEPTH][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
+                    if (mt * 16 < rows) a[d % ADEPTH][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);
             }
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(live, w[d], pr, wrsrc, wvoff, kk, row_bytes);
@@ -1235,7 +1235,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         // weight rows for step idx + 1 + DEPTH
                         const int soff_act = __builtin_amdgcn_readfirstlane(more_act ? kk_act * 2 : 0);
 #pragma unroll
-                        for (int mt = 0; mt < MTM; ++mt)
+                        for (int mt = 0; mt < NMT; ++mt)  // (only the row tiles the unit has)
                             a[ad][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more_act ? cur_avoff[mt] : kNoLoad, soff_act, 0);
 #pragma unroll
                         for (int pr = 0; pr < 4; ++pr) load_w_pair_if<FP8>(more_w, w[dn], pr, cur_wrsrc, cur_wvoff, kk_w, row_bytes);
