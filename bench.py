@@ -153,7 +153,8 @@ def time_expert_matmuls(dev, one_step, stream, rounds=10):
     attention launch is timed): the up projection with fused SwiGLU and the down projection at the shape of a
     lyra-medium MoE layer (benchmark configuration 3: width 4096, 31 routed + 1 shared experts of hidden 4096, 64 tokens,
     3 routed experts per token drawn from Zipf(1.1) + the shared one, seeded) and at the shape of the lyra-small layer the
-    step itself runs (15 + 1 experts, width 2048, hidden 2048).  FP8 weights, one scale per output channel."""
+    step itself runs (15 + 1 experts, width 2048, hidden 2048).  FP8 weights, one scale per output channel.  The group
+    sizes are the instances `--kernels` times as "lyra-medium expert ... T=64" and "lyra-small expert ... B=64"."""
     import numpy as np
     import torch
 
@@ -163,8 +164,8 @@ def time_expert_matmuls(dev, one_step, stream, rounds=10):
     gen = torch.Generator(device=dev)
     gen.manual_seed(1003)
     out_rows = []
-    for label, E, C, Hd, n_routed in (("lyra-medium", 32, 4096, 4096, 31), ("lyra-small", 16, 2048, 2048, 15)):
-        sizes = zipf_group_sizes(np.random.default_rng(1003), 64, n_routed, 3, 1)
+    routing = benchmark_routing()
+    for label, E, C, Hd, sizes in (("lyra-medium", 32, 4096, 4096, routing["medium_T64"]), ("lyra-small", 16, 2048, 2048, routing["small_B64"])):
         M, touched = int(sizes.sum()), int((sizes > 0).sum())
         gs = torch.from_numpy(sizes).to(dev)
         x = torch.randn(M, C, generator=gen, device=dev, dtype=torch.bfloat16)
@@ -216,6 +217,22 @@ def _time_launches(launch, stream, warm=5, iters=50):
     stop.record(stream)
     stop.synchronize()
     return start.elapsed_time(stop) * 1e-3 / iters
+
+
+def benchmark_routing():
+    """The routing instances of the operator table and of `roofline.gemm`, drawn in one fixed order from one seeded generator
+    so that both measure the same group sizes: rows per expert for lyra-medium at 1, 16 and 64 tokens, a second 64-token draw
+    (the scale-block case), lyra-max at 128 tokens, lyra-small at 8 and 64 tokens."""
+    import numpy as np
+
+    rng = np.random.default_rng(1003)
+    r = {f"medium_T{T}": zipf_group_sizes(rng, T, 31, 3, 1) for T in (1, 16, 64)}
+    r["medium_T64_blocks"] = zipf_group_sizes(rng, 64, 31, 3, 1)
+    r["max_B128"] = zipf_group_sizes(rng, 128, 63, 3, 1)
+    r["small_B8"] = zipf_group_sizes(rng, 8, 15, 3, 1)
+    r["small_B64"] = zipf_group_sizes(rng, 64, 15, 3, 1)
+    r["probe"] = zipf_group_sizes(rng, 64, 15, 3, 1)
+    return r
 
 
 def zipf_group_sizes(rng, tokens, n_routed, k_routed, n_shared):
@@ -322,7 +339,7 @@ def kernel_table(dev, only=""):
                      "cold_us": cold * 1e6, "hot_us": hot * 1e6})
         del weights
 
-    rng = np.random.default_rng(1003)
+    routing = benchmark_routing()
     attention("lyra-small B=1 ctx 512 bf16 global", 1, 16, 4, 128, 512, 0, False)
     attention("lyra-small B=8 ctx 4096 fp8 global", 8, 16, 4, 128, 4096, 0, True)
     attention("lyra-small B=64 ctx 4096 fp8 global (headline)", 64, 16, 4, 128, 4096, 0, True)
@@ -338,23 +355,23 @@ def kernel_table(dev, only=""):
     attention("lyra-medium B=64 ctx 4096 fp8 global, one position per row", 64, 32, 8, 128, 4096, 0, True, np.full(64, 4096))
     attention("lyra-max B=128 ctx 4096 fp8 global, one position per row", 128, 32, 8, 128, 4096, 0, True, np.full(128, 4096))
     for T in (1, 16, 64):
-        s = zipf_group_sizes(rng, T, 31, 3, 1)
+        s = routing[f"medium_T{T}"]
         gemm(f"lyra-medium expert up+SwiGLU T={T} (32x4096x8192 fp8)", int(s.sum()), 32, 4096, 8192, s, True, (4096, 1))
         gemm(f"lyra-medium expert down T={T} (32x4096x4096 fp8)", int(s.sum()), 32, 4096, 4096, s, False, (4096, 1))
     even = np.array([8] * 31 + [64], np.int32)  # evenly routed tokens (what a load-balancing loss aims at) + the shared expert
     gemm("lyra-medium expert up+SwiGLU T=64, even routing (32x4096x8192 fp8)", int(even.sum()), 32, 4096, 8192, even, True, (4096, 1))
     gemm("lyra-medium expert down T=64, even routing (32x4096x4096 fp8)", int(even.sum()), 32, 4096, 4096, even, False, (4096, 1))
-    s = zipf_group_sizes(rng, 64, 31, 3, 1)
+    s = routing["medium_T64_blocks"]
     gemm("lyra-medium expert up+SwiGLU T=64, scale blocks (256,256)", int(s.sum()), 32, 4096, 8192, s, True, (256, 256))
-    s = zipf_group_sizes(rng, 128, 63, 3, 1)
+    s = routing["max_B128"]
     gemm("lyra-max expert up+SwiGLU B=128 (64x4096x8192 fp8)", int(s.sum()), 64, 4096, 8192, s, True, (4096, 1))
     gemm("lyra-max expert down B=128 (64x4096x4096 fp8)", int(s.sum()), 64, 4096, 4096, s, False, (4096, 1))
     for B in (8, 64):
-        s = zipf_group_sizes(rng, B, 15, 3, 1)
+        s = routing[f"small_B{B}"]
         gemm(f"lyra-small expert up+SwiGLU B={B} (16x2048x4096 fp8)", int(s.sum()), 16, 2048, 4096, s, True, (2048, 1))
         gemm(f"lyra-small expert down B={B} (16x2048x2048 fp8)", int(s.sum()), 16, 2048, 2048, s, False, (2048, 1))
     if only and "probe" in only:  # what the 64-row units of the shared expert cost: the same routing with a light shared expert
-        s = zipf_group_sizes(rng, 64, 15, 3, 1)
+        s = routing["probe"]
         for shared_rows in (64, 32, 16):
             t = s.copy()
             t[15] = shared_rows
