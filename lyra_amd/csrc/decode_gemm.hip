@@ -680,7 +680,9 @@ constexpr int kSplitPitch = 132;  // floats per row of a partial tile in LDS (12
 // takes DEPTH consecutive steps instead of every 4th.
 // LOOP: slices longer than 4 * DEPTH steps (larger matrices, cut less finely so that one round of workgroups covers them):
 // the DEPTH register sets are refilled as they are used, wavefronts interleave, STEP_SCALES is 0 or 2.
-template <bool FP8, int DEPTH, int STEP_SCALES, bool LOOP>
+// MT: 16-row tiles the instantiation holds (1, 2 or 4 = row blocks of 16, 32, 64 rows): a launch with smaller blocks runs
+// less code - these launches are bound by the instructions one wavefront per SIMD gets through, not by arithmetic.
+template <bool FP8, int DEPTH, int STEP_SCALES, bool LOOP, int MT = 4>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
@@ -699,18 +701,18 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
         const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
     const int wvoff = 8 * kb * row_bytes + ncol * ES;
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
-    int avoff[4];
+    int avoff[MT];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
         const int arow = row0 + mt * 16 + x;
         const bool mine = arow < p.M && mt * 16 < p.row_block;
         const int asrc = mine ? (p.row_map ? p.row_map[arow] : arow) : 0;
         avoff[mt] = mine ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
     }
-    const int n_mt = min(p.row_block >> 4, (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
+    const int n_mt = min(min(p.row_block >> 4, MT), (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
 
     // all operands are requested before anything is waited for, in the order they are consumed
-    u32x4 a[DEPTH][4];
+    u32x4 a[DEPTH][MT];
     RawW<FP8> w[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
@@ -718,7 +720,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
         const int kk = step_row(d);
         const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {  // (row tiles the block does not have are not requested: a load that fetches nothing
+        for (int mt = 0; mt < MT; ++mt) {  // (row tiles the block does not have are not requested: a load that fetches nothing
             if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);  // still takes its turn)
             else a[d][mt] = u32x4{0u, 0u, 0u, 0u};
         }
@@ -752,9 +754,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int cnt = min(p.group_sizes[0], p.M);  // rows at or beyond it multiply zeros (lax.ragged_dot)
     __builtin_amdgcn_sched_barrier(0);
 
-    f32x4 acc[4][8];
+    f32x4 acc[MT][8];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -762,9 +764,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int idx = base + d;
-            Pack8 bop[8], av[4];
+            Pack8 bop[8], av[MT];
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
+            for (int mt = 0; mt < MT; ++mt) {
                 const bool a_ok = row0 + mt * 16 + x < cnt;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) av[mt].u[i] = a_ok ? a[d][mt][i] : 0u;
@@ -778,7 +780,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
                 __builtin_amdgcn_sched_barrier(0);
                 const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt)
+                for (int mt = 0; mt < MT; ++mt)
                     if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff[mt] : kNoLoad, soff, 0);
 #pragma unroll
                 for (int pr = 0; pr < 4; ++pr) {
@@ -793,7 +795,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
                 for (int pr = 0; pr < 4; ++pr) convert_pair<FP8>(w[d], pr, bop);
             }
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
+            for (int mt = 0; mt < MT; ++mt) {
                 if (mt < n_mt) {
                     if constexpr (STEP_SCALES == 2) {
 #pragma unroll
@@ -816,7 +818,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 
     float* mine = sm_part + wave * (64 * kSplitPitch);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
         if (mt < n_mt) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -1532,12 +1534,18 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
     // scales that change along K: free when every wavefront's rows (32 * depth) lie within one scale block
     const int step_scales =
         !(fp8 && p.scale_mode == 1 && p.bk < p.K) ? 0 : ((!loop && p.bk % (32 * std::max(1, std::min(depth, 4))) == 0) ? 1 : 2);
-#define LYRA_SPLITK(F, D, S)                                                                                          \
+#define LYRA_SPLITK_M(F, D, S, M_)                                                                                    \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S, false>,   \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S, false, M_>, \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S, false>), grid, block, lds, st, p);                     \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S, false, M_>), grid, block, lds, st, p);                 \
+    } while (0)
+#define LYRA_SPLITK(F, D, S)                              \
+    do {                                                  \
+        if (pl.row_block <= 16) LYRA_SPLITK_M(F, D, S, 1); \
+        else if (pl.row_block <= 32) LYRA_SPLITK_M(F, D, S, 2); \
+        else LYRA_SPLITK_M(F, D, S, 4);                   \
     } while (0)
 #define LYRA_SPLITK_LOOP(F, S)                                                                                        \
     do {                                                                                                              \
@@ -1564,6 +1572,7 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
 #undef LYRA_SPLITK_D
 #undef LYRA_SPLITK_LOOP
 #undef LYRA_SPLITK
+#undef LYRA_SPLITK_M
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 
