@@ -1,0 +1,119 @@
+"""GPU parity of both operators at shapes drawn from a seeded generator (through the C ABI, against the CPU oracle).
+
+The named tests pin the shapes of the model variants; these draws walk the rest of the supported domain - K that is
+not a multiple of 128, 1 to 40 groups with empty groups and padding rows, every supported scale-block layout, odd
+cache lengths, every head-group count up to 16, windows of any width, one position per row including rows that see
+no key - so that every launch plan (one pass, K slices, unit list, general kernel; whole rows, chunks) meets sizes
+nobody chose for it.  Tolerance as in the named tests: |got - want| <= 2e-2 + 1e-2*|want| against the fp32 oracle.
+Each case is printed before it runs.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lyra_oracle as O
+from tests import gpu_util as U
+from tests.test_gpu_attention import _run as run_attention
+from tests.test_gpu_gemm import _case as gemm_case, _run as run_gemm, _want as gemm_want
+
+pytestmark = pytest.mark.gpu
+
+
+def _note(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _blocks_for(rng, K, N):
+    """A supported scale-block layout for a (K, N) weight (lyra_amd/kernels/decode_gemm.py: _scale_layout_supported)."""
+    bks = [K] + [b for b in (32, 64, 96, 128, 256, 512) if K % b == 0 and b < K]
+    bk = int(rng.choice(bks))
+    bns = [b for b in (1, 8, 16, 64, 128, 256) if N % b == 0 and (bk == K or b % 8 == 0)]
+    return bk, int(rng.choice(bns))
+
+
+def _draw_gemm(seed):
+    rng = np.random.default_rng(seed)
+    swiglu = bool(rng.integers(0, 2))
+    G = int(rng.choice([1, 1, 2, 3, 5, 8, 17, 40]))
+    K = 32 * int(rng.choice([1, 2, 3, 5, 8, 9, 16, 23, 32, 64, 90]))
+    n_unit = 256 if swiglu else 128
+    N = n_unit * int(rng.choice([1, 1, 2, 3, 5, 8, 11]))
+    while G * K * N > (1 << 23):  # keeps the numpy oracle in fractions of a second
+        if G > 2:
+            G = max(1, G // 2)
+        elif N > n_unit:
+            N -= n_unit
+        else:
+            K = max(32, K // 2 // 32 * 32)
+    M = int(rng.choice([1, 2, 7, 16, 17, 33, 64, 65, 130, 300]))
+    # group sizes: some groups empty, the sum sometimes short of M (the rest are padding rows)
+    cuts = np.sort(rng.integers(0, M + 1, G - 1)) if G > 1 else np.zeros(0, np.int64)
+    sizes = np.diff(np.concatenate([[0], cuts, [M]])).astype(np.int32)
+    if G > 1:
+        sizes[rng.integers(0, G)] = 0
+    if rng.integers(0, 3) == 0:
+        sizes[-1] = sizes[-1] // 2
+    kind = "fp8" if rng.integers(0, 4) else "bf16"
+    block = _blocks_for(rng, K, N) if kind == "fp8" else None
+    bias = bool(rng.integers(0, 2))
+    return dict(M=M, G=G, K=K, N=N, sizes=sizes.tolist(), kind=kind, block=block, bias=bias, swiglu=swiglu)
+
+
+@pytest.mark.parametrize("seed", range(128))
+def test_decode_gemm_at_drawn_shapes(seed):
+    d = _draw_gemm(7000 + seed)
+    _note(f"gemm draw {seed}: {d}")
+    c = gemm_case(seed, d["M"], d["G"], d["K"], d["N"], d["sizes"], kind=d["kind"], block=d["block"], bias=d["bias"], w_std=0.05)
+    want = gemm_want(c, d["swiglu"])
+    got = run_gemm(c, d["swiglu"])
+    U.assert_close(got, want, what=f"draw {seed}")
+
+
+def _draw_attention(seed):
+    rng = np.random.default_rng(seed)
+    H = int(rng.choice([64, 128]))
+    K = int(rng.choice([1, 2, 3, 4, 8]))
+    G = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16]))
+    B = int(rng.choice([1, 2, 3, 5, 9, 17, 40, 70]))
+    S = int(rng.integers(1, 1500))
+    while B * K * S * H > (1 << 23):
+        if B > 2:
+            B = max(1, B // 2)
+        else:
+            S = max(1, S // 2)
+    sw = int(rng.choice([0, 0, 1, 5, 31, 32, 33, 128, 200, 1000]))
+    fp8 = bool(rng.integers(0, 2))
+    ragged = bool(rng.integers(0, 2))
+    if ragged:
+        pos = rng.integers(0, S, B).astype(np.int32)
+        if B >= 3:
+            pos[rng.integers(0, B)] = -1  # the row sees only its sink
+        pos[B - 1] = S - 1
+    else:
+        pos = int(rng.integers(0, S))
+    gate = bool(rng.integers(0, 2))
+    f32 = bool(rng.integers(0, 4) == 0)
+    return dict(B=B, N=K * G, K=K, S=S, H=H, sw=sw, fp8=fp8, pos=pos, gate=gate, f32=f32)
+
+
+@pytest.mark.parametrize("seed", range(128))
+def test_decode_attention_at_drawn_shapes(seed):
+    d = _draw_attention(9000 + seed)
+    _note(f"attention draw {seed}: { {k: (v.tolist() if isinstance(v, np.ndarray) else v) for k, v in d.items()} }")
+    case = U.attention_case(seed, d["B"], d["N"], d["K"], d["S"], d["H"], fp8=d["fp8"])
+    rng = np.random.default_rng(seed)
+    gate = O.bf16_round((2.0 / (1.0 + np.exp(-rng.standard_normal((d["B"], d["N"]))))).astype(np.float32)) if d["gate"] else None
+    sm_scale = d["H"] ** -0.5
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], sm_scale, d["sw"], d["pos"])
+    if gate is not None:
+        want = want * gate[:, :, None, None]
+    if d["f32"]:
+        got = run_attention(case, sm_scale, d["sw"], d["pos"], gate=gate, dtype=torch.float32)
+        U.assert_close(got, want, atol=4e-3 if gate is None else 8e-3, rtol=4e-3, what=f"draw {seed} f32")
+    else:
+        got = run_attention(case, sm_scale, d["sw"], d["pos"], gate=gate)
+        U.assert_close(got, want, what=f"draw {seed}")
+    if isinstance(d["pos"], np.ndarray):
+        assert np.all(got[d["pos"] < 0] == 0), "a row that sees no key attends only to its sink, whose value is zero"
