@@ -359,6 +359,19 @@ def test_many_experts_with_scale_blocks_along_k(block, swiglu):
     U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what="unit list, k scale blocks")
 
 
+@pytest.mark.parametrize("M,K,N,kind,block", [(5, 416, 131968, "bf16", None), (64, 416, 131200, "bf16", None), (33, 416, 132096, "fp8", (416, 1)),
+                                             (64, 288, 204800, "bf16", None), (17, 480, 131328, "fp8", (96, 128))])
+def test_very_wide_projection_one_workgroup_per_compute_unit(M, K, N, kind, block):
+    """A single projection with more than 1024 spans of 128 columns (the LM head): one workgroup per compute unit, the
+    spans dealt out evenly.  Span counts that do not divide by the number of workgroups, with bias, 1 to 4 row tiles
+    (K is chosen so that the plan is neither the one-pass nor the K-slice kernel)."""
+    c = _case(31, M, 1, K, N, [M], kind=kind, block=block, bias=True, w_std=0.05)
+    _note(f"gemm very wide M={M} K={K} N={N} kind={kind} block={block}")
+    want = _want(c, False, big=True)
+    U.assert_close(_run(c, False), want, what=f"N={N}")
+    U.assert_close(_run(c, False, out_f32=True), want, atol=2e-3, rtol=2e-3, what=f"N={N} f32")
+
+
 @pytest.mark.parametrize("G,M", [(1, 20), (6, 20)])
 def test_zero_and_extreme_block_scales(G, M):
     """Scales a quantiser never produces but a caller may pass: exactly zero (the block must contribute nothing), and
