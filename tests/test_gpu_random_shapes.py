@@ -117,3 +117,40 @@ def test_decode_attention_at_drawn_shapes(seed):
         U.assert_close(got, want, what=f"draw {seed}")
     if isinstance(d["pos"], np.ndarray):
         assert np.all(got[d["pos"] < 0] == 0), "a row that sees no key attends only to its sink, whose value is zero"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_step_kernels_at_drawn_shapes(seed):
+    """The checks of tests/test_gpu_fused.py (norm + projection, QK norm + RoPE + cache append, routing, combine, argmax,
+    top-k sampling) at drawn sizes: widths that are not powers of two, 1 to 300 rows, up to 128 routed experts."""
+    from tests import test_gpu_fused as TF
+
+    rng = np.random.default_rng(11000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    B, C, n = int(rng.integers(1, 131)), pick([64, 100, 256, 1000, 2048, 2880, 4096, 8192]), pick([0, 1, 3, 8, 15, 16, 31, 63, 64, 100, 128])
+    mode = "none" if n == 0 else pick(["gate", "logits"])
+    _note(f"fused draw {seed}: rmsnorm_proj B={B} C={C} n={n} {mode}")
+    TF.test_rmsnorm_proj(B, C, n, mode)
+
+    K, G, H = pick([1, 2, 4, 8]), pick([1, 2, 4, 8]), pick([64, 128])
+    B, S = int(rng.integers(1, 71)), int(rng.integers(2, 600))
+    fp8, qknorm, per_row = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    _note(f"fused draw {seed}: qkv_post B={B} N={K * G} K={K} S={S} H={H} fp8={fp8} qknorm={qknorm} per_row={per_row}")
+    TF.test_qkv_post(B, K * G, K, S, H, fp8, qknorm, per_row)
+
+    T, n_routed, n_shared = int(rng.integers(1, 301)), int(rng.integers(2, 129)), int(rng.integers(0, 2))
+    k = int(rng.integers(1, min(8, n_routed) + 1))
+    _note(f"fused draw {seed}: moe_route T={T} routed={n_routed} shared={n_shared} k={k}")
+    TF.test_moe_route(T, n_routed, n_shared, k)
+
+    T, topk, C = int(rng.integers(1, 131)), int(rng.integers(1, 9)), 8 * int(rng.integers(1, 600))
+    _note(f"fused draw {seed}: moe_combine T={T} topk={topk} C={C}")
+    TF.test_moe_combine(T, topk, C)
+
+    rows, cols = int(rng.integers(1, 131)), int(rng.integers(1, 60000))
+    ld = (cols + 3) // 4 * 4 + 4 * int(rng.integers(0, 3))
+    _note(f"fused draw {seed}: argmax rows={rows} cols={cols} ld={ld}")
+    TF.test_argmax_first_maximum(rows, cols, ld)
+    kk, temperature = int(rng.integers(1, 9)), float(rng.choice([0.3, 0.8, 1.0, 1.5]))
+    _note(f"fused draw {seed}: sample_topk rows={rows} cols={cols} ld={ld} k={kk} T={temperature}")
+    TF.test_sample_topk_matches_oracle(rows, cols, ld, kk, temperature)
