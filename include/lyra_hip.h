@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 9
+#define LYRA_ABI_VERSION 10
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -86,6 +86,26 @@ size_t lyra_decode_attention_workspace(int B, int N, int K, int S, int H, int sl
 int lyra_decode_attention_xsa(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                               const float* sinks, const int32_t* position, int position_stride, const void* gate,
                               const void* v_unit, const float* xsa_alpha, void* out, void* workspace, size_t workspace_bytes,
+                              int B, int N, int K, int S, int H, float sm_scale, int sliding_window, int kv_dtype,
+                              int out_dtype, lyra_stream_t stream);
+
+/*
+ * lyra_qkv_post_sum and lyra_decode_attention in one launch: what lies between the fused q/k/v projection and the output
+ * projection of an attention layer (lyra/model.py:309-347: QK norm, rotary embedding, cache_update :204-212 / qupdate
+ * lyra/nn/quant.py:89-98, decode_attention with the output gate).  Every workgroup of the attention kernel first builds
+ * the q rows of its kv head from the projection, and the workgroup whose keys include the new token's appends that
+ * token's key and value rows to the caches before it reads them.  Arguments as in lyra_qkv_post_sum (qkv / partials /
+ * splits, qnorm, knorm, cos_t, sin_t, rope_rows, eps) and lyra_decode_attention; k, v, k_scale, v_scale are written at
+ * index position[b] (rows with a position outside [0,S) are not appended).  q is never materialised.
+ * Results and cache contents are bit-identical to the two calls.  LYRA_E_UNSUPPORTED (nothing launched) for a ragged
+ * batch without a window and with more than 256 (row, kv head) pairs, which lyra_decode_attention hands to its whole-row
+ * kernel: call the two entry points then.  No learned exclusive self attention here (lyra_decode_attention_xsa needs the
+ * v_unit rows lyra_qkv_post writes).
+ */
+int lyra_decode_attention_qkv(const void* qkv, const float* partials, int splits, const float* qnorm, const float* knorm,
+                              const float* cos_t, const float* sin_t, int rope_rows, float eps, void* k, void* v,
+                              float* k_scale, float* v_scale, const float* sinks, const int32_t* position,
+                              int position_stride, const void* gate, void* out, void* workspace, size_t workspace_bytes,
                               int B, int N, int K, int S, int H, float sm_scale, int sliding_window, int kv_dtype,
                               int out_dtype, lyra_stream_t stream);
 

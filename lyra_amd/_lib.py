@@ -8,7 +8,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 9
+ABI_VERSION = 10
+E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 
 _c = ctypes
 SIGNATURES = {
@@ -22,6 +23,11 @@ SIGNATURES = {
     "lyra_decode_attention_xsa": (
         _c.c_int,
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
+    "lyra_decode_attention_qkv": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 4 + [_c.c_int, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] + [_c.c_void_p] * 3
+        + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_static": (
         _c.c_int,

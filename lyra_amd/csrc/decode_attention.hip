@@ -51,6 +51,17 @@ struct AttnParams {
     const uint16_t* xsa_v;   // [B,K,H] bf16: the new token's value rows scaled to unit length
     const float* xsa_alpha;  // [N]
     int xsa_lds;             // float offset of the staging area [G*H + 16] in dynamic LDS
+    // lyra_decode_attention_qkv: the step in front of the attention (QK norm, rotary embedding, cache append) is done by
+    // this launch; q is then not read.  The caches behind k, v, ks, vs are written (one row per batch row and kv head).
+    const float* qkv_partials;  // [splits, B, (N + 2K) * H] float32 slices of the q/k/v projection, or null (then qkv)
+    const uint16_t* qkv;        // [B, (N + 2K) * H] bf16
+    int qkv_splits;
+    const float* qnorm;  // [H] or null (both)
+    const float* knorm;
+    const float* cos_t;  // [rope_rows, H/2]
+    const float* sin_t;
+    int rope_rows;
+    float norm_eps;
 };
 
 constexpr int kTile = 32;
@@ -358,9 +369,132 @@ __device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_
     }
 }
 
-template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY, int DEPTH>
+// ---- what lyra_qkv_post does for one (batch row, kv head), inside the attention launch -------------------------------
+// Same arithmetic in the same order, so results and cache contents are bit-identical to the two launches.  Wavefront w
+// takes the query heads w, w + WAVES, ... of the G: sum of the projection's slices, QK norm, rotary embedding -> row t of
+// the q tile in LDS.  The last wavefront also finishes the new token's key and value rows (norm, rotary embedding,
+// quantisation) and leaves their bytes in LDS.  All of this is requested when the kernel starts, next to the first cache
+// tiles, and done before the barrier that releases the wavefronts into their loops.  Behind the barrier, in the workgroup
+// whose chunk holds the new token's key, the wavefront that will read that key's tile copies the two rows into the
+// caches: they are written and read by one wavefront, whose memory operations are served in the order it issued them, so
+// nobody waits for the stores.
+constexpr int kHeadSlices = 8;   // slices of a head held in registers
+constexpr int kFirstSlices = 4;  // ... of which are requested when the kernel starts
+struct HeadSlices {
+    float a[kHeadSlices], c[kHeadSlices];  // the first slices of elements `lane` and `lane + H/2`
+    uint16_t qa, qc;                       // ... or the two elements of the summed projection (bf16)
+};
+
+// Requests the slices of head hd for this lane (elements `lane` and `lane + H/2`).  Every load is issued whatever the
+// arguments - through descriptors, with an offset outside them for what does not exist (slices beyond the last, the other
+// of the two input forms, idle lanes) - so that no load sits inside a branch and the compiler keeps an exact count of
+// what is in flight.
+// The slices come in two requests, J0 = 0 and J0 = kFirstSlices: projections of many rows have at most kFirstSlices, and a
+// load that returns nothing still takes its turn in the address unit.
+template <int H, int J0 = 0>
+__device__ __forceinline__ void request_head(const AttnParams& p, __amdgpu_buffer_rsrc_t part_rsrc, __amdgpu_buffer_rsrc_t qkv_rsrc,
+                                             int b, int hd, bool live, int lane, HeadSlices& hs) {
+    constexpr int half = H / 2;
+    const int heads = p.N + 2 * p.K;
+    const bool on = live && lane < half;
+    const int slab = p.B * heads * H;                 // floats per slice (the host keeps splits * slab * 4 below 2^31)
+    const int at = (b * heads + hd) * H + lane;       // element `lane` of the head within a slice
+#pragma unroll
+    for (int j = J0; j < (J0 == 0 ? kFirstSlices : kHeadSlices); ++j) {
+        const int off = on && j < p.qkv_splits ? (j * slab + at) * 4 : kNoLoad;
+        hs.a[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(part_rsrc, off, 0, 0));
+        hs.c[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(part_rsrc, off, half * 4, 0));
+    }
+    if constexpr (J0 != 0) return;
+#pragma unroll
+    for (int j = kFirstSlices; j < kHeadSlices; ++j) hs.a[j] = hs.c[j] = 0.f;
+    // the summed form of the projection (bf16); a null descriptor when the slices are given
+    const int off16 = on ? at * 2 : kNoLoad;
+    hs.qa = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(qkv_rsrc, off16, 0, 0);
+    hs.qc = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(qkv_rsrc, off16, half * 2, 0);
+}
+
+// The projection's bf16 output for this lane's two elements of head hd: the slices added in slice order, then rounded.
+template <int H>
+__device__ __forceinline__ void sum_head(const AttnParams& p, __amdgpu_buffer_rsrc_t part_rsrc, int b, int hd, int lane,
+                                         const HeadSlices& hs, float& a, float& c) {
+    constexpr int half = H / 2;
+    if (!p.qkv_partials) {
+        a = bf16_bits_to_f32(hs.qa);
+        c = bf16_bits_to_f32(hs.qc);
+        return;
+    }
+    a = 0.f + hs.a[0];
+    c = 0.f + hs.c[0];
+#pragma unroll
+    for (int j = 1; j < kHeadSlices; ++j) {
+        if (j < p.qkv_splits) {
+            a += hs.a[j];
+            c += hs.c[j];
+        }
+    }
+    if (p.qkv_splits > kHeadSlices) {  // (more slices than are requested at once: the rest one by one)
+        const int heads = p.N + 2 * p.K;
+        const int slab = p.B * heads * H, at = (b * heads + hd) * H + lane;
+        for (int j = kHeadSlices; j < p.qkv_splits; ++j) {
+            const int off = lane < half ? (j * slab + at) * 4 : kNoLoad;
+            a += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(part_rsrc, off, 0, 0));
+            c += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(part_rsrc, off, half * 4, 0));
+        }
+    }
+    a = bf16r(a);
+    c = bf16r(c);
+}
+
+// The cache bytes of one finished row (this lane's elements a, c) of the key (slot 0) or value (slot 1) head, left in
+// LDS: H codes and the row's scale for an FP8 cache, H bf16 values otherwise.  stage: [2][H * ES] bytes, then 2 floats.
+template <int H, bool FP8>
+__device__ __forceinline__ void stage_row(uint8_t* stage, int slot, int lane, float a, float c) {
+    constexpr int half = H / 2, ES = FP8 ? 1 : 2;
+    const bool active = lane < half;
+    if constexpr (FP8) {
+        const float amax = wave_max(fmaxf(fabsf(a), fabsf(c)));
+        const float scale = amax > 0.f ? amax / 448.f : 1.f;
+        const float inv = 1.0f / scale;
+        if (active) {
+            uint8_t* dst = stage + slot * H;
+            dst[lane] = f32_to_e4m3fn(fminf(fmaxf(a * inv, -448.f), 448.f));
+            dst[lane + half] = f32_to_e4m3fn(fminf(fmaxf(c * inv, -448.f), 448.f));
+        }
+        if (lane == 0) ((float*)(stage + 2 * H * ES))[slot] = scale;
+    } else if (active) {
+        uint16_t* dst = (uint16_t*)stage + slot * H;
+        dst[lane] = f32_to_bf16_bits(a);
+        dst[lane + half] = f32_to_bf16_bits(c);
+    }
+}
+
+// Copies the two staged rows into the caches at key `pos` of this workgroup's slab (one dword per lane and row).  Every
+// wavefront issues the stores, through the slab's descriptors and with an offset outside them where nothing is to be
+// written (`live` false: not the wavefront that owns the new key), so that no memory operation sits inside a branch:
+// behind a branch the compiler no longer knows how many operations are in flight and makes the tile loop wait for all of
+// them in every pass.
+template <int H, bool FP8>
+__device__ __forceinline__ void append_staged(const Slab& sl, const uint8_t* stage, int pos, bool live, int lane) {
+    constexpr int ES = FP8 ? 1 : 2, DW = H * ES / 4;  // dwords per row (16 to 64)
+    const bool on = live && lane < DW;
+    const uint32_t kd = ((const uint32_t*)stage)[lane & (DW - 1)], vd = ((const uint32_t*)stage)[DW + (lane & (DW - 1))];
+    const int off = on ? pos * (H * ES) + lane * 4 : kNoLoad;
+    __builtin_amdgcn_raw_buffer_store_b32(kd, sl.k, off, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(vd, sl.v, off, 0, 0);
+    if constexpr (FP8) {
+        const float* sc = (const float*)(stage + 2 * H * ES);
+        const int soff = live && lane == 0 ? pos * 4 : kNoLoad;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sc[0]), sl.ks, soff, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sc[1]), sl.vs, soff, 0, 0);
+    }
+}
+
+// QKV: the launch also does the step in front of the attention (lyra_decode_attention_qkv).
+template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY, int DEPTH, bool QKV = false>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(DEPTH > 1 ? 2 : (WAVES >= 8 ? 4 : 3))))
 void decode_attention_kernel(AttnParams p) {
+    static_assert(!QKV || DEPTH == 1, "the fused front step knows one register set per wavefront");
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int CB = H / 16;
     constexpr int HP = H + 4;  // LDS row pitch of the merge buffer in floats
@@ -371,6 +505,13 @@ void decode_attention_kernel(AttnParams p) {
     const int x = lane & 15, kb = lane >> 4;
     const int c_idx = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
     const int G = p.G;
+
+    // The position first: loads return in the order they were issued, so requested behind the cache tiles and the
+    // projection slices it would arrive last, and everything that follows from it (rotary row, window, the owner of the
+    // new key) would start that much later.
+    const uint32_t pos_raw = __builtin_amdgcn_raw_buffer_load_b32(
+        make_rsrc(p.position, (uint32_t)(p.pos_stride ? p.B : 1) * 4u), 0, b * p.pos_stride * 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
 
     const size_t head_row = ((size_t)b * p.K + kh) * p.S;
     Slab sl;
@@ -385,9 +526,19 @@ void decode_attention_kernel(AttnParams p) {
     // q of this kv head's G query heads (thread t: row t / (H/8), 16-byte piece t % (H/8); rows >= G lie past the end of
     // the descriptor and read as zeros) and the sink logits: requested first, so that their arrival does not wait for
     // the cache tiles behind them (loads return in order).
-    const __amdgpu_buffer_rsrc_t qrsrc = make_rsrc(p.q + ((size_t)b * p.N + kh * G) * H, (uint32_t)(G * H * 2));
     const int q_row = threadIdx.x / (H / 8), q_piece = threadIdx.x % (H / 8);
-    const u32x4 q_raw = __builtin_amdgcn_raw_buffer_load_b128(qrsrc, (q_row * H + q_piece * 8) * 2, 0, 0);
+    u32x4 q_raw = u32x4{0u, 0u, 0u, 0u};
+    [[maybe_unused]] const int qkv_heads = p.N + 2 * p.K;
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t part_rsrc = make_rsrc(
+        p.qkv_partials, p.qkv_partials ? (uint32_t)p.qkv_splits * (uint32_t)p.B * (uint32_t)qkv_heads * (uint32_t)H * 4u : 0u);
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t qkv_rsrc =
+        make_rsrc(p.qkv, (QKV && !p.qkv_partials) ? (uint32_t)p.B * (uint32_t)qkv_heads * (uint32_t)H * 2u : 0u);
+    [[maybe_unused]] HeadSlices hq, hkv;  // QKV: the projection slices of this wavefront's first query head (head `wave` of the G)
+    [[maybe_unused]] float qn_a = 0.f, qn_c = 0.f, kn_a = 0.f, kn_c = 0.f;
+    if constexpr (!QKV) {
+        const __amdgpu_buffer_rsrc_t qrsrc = make_rsrc(p.q + ((size_t)b * p.N + kh * G) * H, (uint32_t)(G * H * 2));
+        q_raw = __builtin_amdgcn_raw_buffer_load_b128(qrsrc, (q_row * H + q_piece * 8) * 2, 0, 0);
+    }
     const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(p.sinks + kh * G, (uint32_t)(G * 4));
     const float sink_raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(srsrc, x * 4, 0, 0));
     // ... and the output gates of these heads (an absent gate reads as zeros and is replaced by 1 below)
@@ -412,8 +563,22 @@ void decode_attention_kernel(AttnParams p) {
             load_v<H, FP8>(rv[d], sl, early_base, true);
         }
     }
+    if constexpr (QKV) {
+        // (behind the cache tiles: those come from memory and gate the loop, these from the caches)
+        request_head<H>(p, part_rsrc, qkv_rsrc, b, kh * G + wave, wave < G, lane, hq);
+        // (the last wavefront: the key head too, the one before it the value head; used only where the chunk turns out to
+        // hold the new key)
+        request_head<H>(p, part_rsrc, qkv_rsrc, b, wave == WAVES - 1 ? p.N + kh : p.N + p.K + kh, wave >= WAVES - 2, lane, hkv);
+        const __amdgpu_buffer_rsrc_t qn_rsrc = make_rsrc(p.qnorm, p.qnorm ? (uint32_t)H * 4u : 0u);
+        const __amdgpu_buffer_rsrc_t kn_rsrc = make_rsrc(p.knorm, p.knorm ? (uint32_t)H * 4u : 0u);
+        const int noff = lane < H / 2 ? lane * 4 : kNoLoad;
+        qn_a = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(qn_rsrc, noff, 0, 0));
+        qn_c = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(qn_rsrc, noff, H / 2 * 4, 0));
+        kn_a = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(kn_rsrc, noff, 0, 0));
+        kn_c = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(kn_rsrc, noff, H / 2 * 4, 0));
+    }
 
-    const int pos = p.position[(size_t)b * p.pos_stride];
+    const int pos = __builtin_amdgcn_readfirstlane((int)pos_raw);  // (waited for here, with everything above in flight)
     const Range rg = visible_range(pos, p.sw, p.S);
     const int c_lo = rg.start + c_idx * p.chunk;
     if (c_lo > rg.hi) {  // chunk holds no visible key (whole workgroup leaves together)
@@ -428,6 +593,13 @@ void decode_attention_kernel(AttnParams p) {
     }
     const int c_hi = min(c_lo + p.chunk, rg.hi + 1);
     const int n_tiles = (c_hi - c_lo + kTile - 1) / kTile;
+    // QKV: this workgroup appends the new token's key and value when its chunk holds them, through the wavefront that
+    // reads that key's tile (kv_wave); when the tile is that wavefront's first, it is requested a second time after the
+    // rows have been written (`redo`).
+    [[maybe_unused]] const bool owner = QKV && pos >= 0 && pos < p.S && pos >= c_lo && pos < c_lo + p.chunk;
+    [[maybe_unused]] const int kv_wave = owner ? ((pos - c_lo) / kTile) % WAVES : -1;
+    [[maybe_unused]] const bool redo = owner && wave == kv_wave && (pos - c_lo) / kTile < WAVES;
+    [[maybe_unused]] float rope_cs = 0.f, rope_sn = 0.f;
     if constexpr (!early) {  // sliding window: the first key follows from the position
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
@@ -441,7 +613,42 @@ void decode_attention_kernel(AttnParams p) {
 
     uint16_t* sm_q = (uint16_t*)smem;
     static_assert(WAVES * 64 >= 16 * (H / 8), "one q piece per thread");
-    *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = q_raw;  // every thread stores (rows >= G hold zeros; rows >= 16 are never read)
+    if constexpr (QKV) {
+        if (q_row >= G) *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = q_raw;  // zeros
+        constexpr int half = H / 2;
+        if (p.qkv_splits > kFirstSlices) {  // (projections of few rows are cut into more slices)
+            request_head<H, kFirstSlices>(p, part_rsrc, qkv_rsrc, b, kh * G + wave, wave < G, lane, hq);
+            request_head<H, kFirstSlices>(p, part_rsrc, qkv_rsrc, b, wave == WAVES - 1 ? p.N + kh : p.N + p.K + kh,
+                                          owner && wave >= WAVES - 2, lane, hkv);
+        }
+        {
+            const int rp = min(max(pos, 0), p.rope_rows - 1);
+            const uint32_t rope_bytes = (uint32_t)p.rope_rows * (uint32_t)half * 4u;
+            const int roff = lane < half ? (rp * half + lane) * 4 : kNoLoad;
+            rope_cs = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(make_rsrc(p.cos_t, rope_bytes), roff, 0, 0));
+            rope_sn = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(make_rsrc(p.sin_t, rope_bytes), roff, 0, 0));
+        }
+        for (int t = wave; t < G; t += WAVES) {
+            if (t != wave) request_head<H>(p, part_rsrc, qkv_rsrc, b, kh * G + t, true, lane, hq);  // (more than WAVES query heads per kv head)
+            float a, c;
+            sum_head<H>(p, part_rsrc, b, kh * G + t, lane, hq, a, c);
+            head_norm_rope(a, c, p.qnorm != nullptr, qn_a, qn_c, rope_cs, rope_sn, p.norm_eps, H);
+            if (lane < half) {
+                sm_q[t * QP + lane] = f32_to_bf16_bits(a);
+                sm_q[t * QP + lane + half] = f32_to_bf16_bits(c);
+            }
+        }
+        if (owner && wave >= WAVES - 2) {  // the new token's key and value rows, as the caches will hold them
+            uint8_t* stage = (uint8_t*)(smem + p.xsa_lds);
+            const bool is_k = wave == WAVES - 1;
+            float a, c;
+            sum_head<H>(p, part_rsrc, b, is_k ? p.N + kh : p.N + p.K + kh, lane, hkv, a, c);
+            if (is_k) head_norm_rope(a, c, p.knorm != nullptr, kn_a, kn_c, rope_cs, rope_sn, p.norm_eps, H);
+            stage_row<H, FP8>(stage, is_k ? 0 : 1, lane, a, c);
+        }
+    } else {
+        *(u32x4*)(sm_q + q_row * QP + q_piece * 8) = q_raw;  // every thread stores (rows >= G hold zeros; rows >= 16 are never read)
+    }
 
     Acc<H> acc;
     const float sink2 = x < G ? sink_raw * kLog2e : 0.f;
@@ -450,6 +657,20 @@ void decode_attention_kernel(AttnParams p) {
 #pragma unroll
     for (int c = 0; c < CB; ++c) acc.o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
+    if constexpr (QKV) {
+        // Everything requested so far is needed by now.  Waiting for all of it here, on every path, also tells the compiler
+        // what is in flight when the tile loop starts: after the branches of the front step it otherwise assumes the worst
+        // and makes every pass of the loop wait for nearly all of its loads at once (47 instead of 38 us per launch).
+        wait_all_memory();
+        append_staged<H, FP8>(sl, (const uint8_t*)(smem + p.xsa_lds), pos, wave == kv_wave, lane);  // (0 <= pos < S where live)
+        if (redo) {  // the first tile of this wavefront holds the rows just appended: requested again (now from the caches)
+            const int base = c_lo + wave * kTile;
+            load_k<H, FP8>(rk[0], sl, base, true);
+            if constexpr (FP8) load_s<VEC4>(rs[0], sl, base, true);
+            load_v<H, FP8>(rv[0], sl, base, true);
+            wait_all_memory();  // (leaves this rare path with nothing in flight, like no path the compiler has to guess about)
+        }
+    }
 
     // Loads for a tile past the end are issued all the same, with a lane offset no buffer contains (they return zeros
     // without touching memory): the number of loads in flight is then identical on every path and each wait covers
@@ -903,12 +1124,31 @@ extern "C" int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra
 namespace lyra {
 // Validates and launches; shared by the entry point that takes the caller's workspace and the one that uses the static
 // scratch buffer.  too_small is what an insufficient workspace is reported as.
+// The step in front of the attention, when the launch is to do it (lyra_decode_attention_qkv).
+struct QkvFront {
+    const void* qkv;
+    const float* partials;
+    int splits;
+    const float *qnorm, *knorm, *cos_t, *sin_t;
+    int rope_rows;
+    float eps;
+};
+
 static int run_attention(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                          const float* sinks, const int32_t* position, int position_stride, const void* gate, void* out,
                          void* workspace, size_t workspace_bytes, int too_small, bool clear_counters, const void* xsa_v,
                          const float* xsa_alpha, int B, int N, int K, int S, int H, float sm_scale, int sliding_window,
-                         int kv_dtype, int out_dtype, lyra_stream_t stream) {
-    if (!q || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
+                         int kv_dtype, int out_dtype, lyra_stream_t stream, const QkvFront* front = nullptr) {
+    if ((!q && !front) || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
+    if (front) {
+        if ((front->partials ? front->splits <= 0 : !front->qkv) || !front->cos_t || !front->sin_t || front->rope_rows <= 0)
+            return LYRA_E_BADARG;
+        if ((front->qnorm == nullptr) != (front->knorm == nullptr)) return LYRA_E_BADARG;
+        if (xsa_v) return LYRA_E_UNSUPPORTED;  // the unit-length value row is handed over by lyra_qkv_post only
+        const double width = (double)(N + 2 * K) * H;
+        if ((double)std::max(front->splits, 1) * B * width * 4 >= 2147483648.0 || (double)front->rope_rows * H * 2 >= 2147483648.0)
+            return LYRA_E_UNSUPPORTED;  // (byte offsets into the slices and the rotary tables are 32-bit)
+    }
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || H <= 0 || N % K || sliding_window < 0) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
     if ((xsa_v == nullptr) != (xsa_alpha == nullptr)) return LYRA_E_BADARG;
@@ -945,6 +1185,23 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     p.xsa_v = (const uint16_t*)xsa_v;
     p.xsa_alpha = xsa_alpha;
     p.xsa_lds = 0;
+    p.qkv_partials = nullptr;
+    p.qkv = nullptr;
+    p.qkv_splits = 0;
+    p.qnorm = p.knorm = p.cos_t = p.sin_t = nullptr;
+    p.rope_rows = 0;
+    p.norm_eps = 0.f;
+    if (front) {
+        p.qkv_partials = front->partials;
+        p.qkv = (const uint16_t*)front->qkv;
+        p.qkv_splits = front->splits;
+        p.qnorm = front->qnorm;
+        p.knorm = front->knorm;
+        p.cos_t = front->cos_t;
+        p.sin_t = front->sin_t;
+        p.rope_rows = front->rope_rows;
+        p.norm_eps = front->eps;
+    }
     p.arrivals = nullptr;
     if (pl.n_chunks > 1) {
         const AttnWorkspace w = attention_workspace(B, N, K, H, pl);
@@ -966,7 +1223,8 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     const size_t lds_merge = ((size_t)pl.waves * G * (H + 4) + 2 * pl.waves * 16 + 32) * sizeof(float);
     const size_t lds_q = (size_t)(pl.waves * 64 / (H / 8)) * (H + 8) * sizeof(uint16_t);  // one 16-byte piece of q per thread
     const size_t lds_stage = pl.n_chunks > 1 ? kMergeStageFloats * sizeof(float) : 0;
-    const size_t lds_xsa = xsa_v ? ((size_t)G * H + 16) * sizeof(float) : 0;  // staging area of the last step, behind the rest
+    // behind the rest: the staging area of the exclusive-self-attention step, or (front step) of the new key and value rows
+    const size_t lds_xsa = xsa_v ? ((size_t)G * H + 16) * sizeof(float) : (front ? (size_t)2 * H * 2 + 16 : 0);
     const size_t lds_base = (std::max(std::max(lds_merge, lds_q), lds_stage) + 15) / 16 * 16;
     const size_t lds = lds_base + lds_xsa;
     p.xsa_lds = (int)(lds_base / sizeof(float));
@@ -978,6 +1236,8 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     static const long rows_waves_env = env_long("LYRA_ATTN_ROWS_WAVES");
     const bool rows = rows_mode > 0 && (position_stride == 1 || rows_mode > 1) && sliding_window == 0 && pl.n_chunks == 1 &&
                       (long)B * K > 256 && B <= kMaxRankedRows;
+    // the front step exists in the chunked kernel with 4 wavefronts only; the caller takes the two launches otherwise
+    if (front && (rows || pl.waves != 4)) return LYRA_E_UNSUPPORTED;
     if (rows) {
         const int waves = (rows_waves_env == 4 || rows_waves_env == 8) ? (int)rows_waves_env : (H == 64 ? 8 : 4);
         const size_t lds_need = std::max(((size_t)waves * G * (H + 4) + 2 * waves * 16 + 32) * sizeof(float),
@@ -1021,7 +1281,10 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     } while (0)
 #define LYRA_LAUNCH_ATTN(HH, F, V)                              \
     do {                                                        \
-        if (pl.waves == 4) LYRA_LAUNCH_ATTN_W(HH, F, V, 4);     \
+        if (front) {                                            \
+            if (sliding_window == 0) hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, 4, true, 1, true>), grid, block, lds, st, p); \
+            else hipLaunchKernelGGL((decode_attention_kernel<HH, F, V, 4, false, 1, true>), grid, block, lds, st, p); \
+        } else if (pl.waves == 4) LYRA_LAUNCH_ATTN_W(HH, F, V, 4); \
         else if (pl.waves == 8) LYRA_LAUNCH_ATTN_W(HH, F, V, 8); \
         else LYRA_LAUNCH_ATTN_W(HH, F, V, 16);                  \
     } while (0)
@@ -1062,6 +1325,19 @@ static void* static_scratch() {
     return g_scratch_ptr[dev];
 }
 }  // namespace lyra
+
+extern "C" int lyra_decode_attention_qkv(const void* qkv, const float* partials, int splits, const float* qnorm,
+                                         const float* knorm, const float* cos_t, const float* sin_t, int rope_rows, float eps,
+                                         void* k, void* v, float* k_scale, float* v_scale, const float* sinks,
+                                         const int32_t* position, int position_stride, const void* gate, void* out,
+                                         void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
+                                         float sm_scale, int sliding_window, int kv_dtype, int out_dtype,
+                                         lyra_stream_t stream) {
+    const lyra::QkvFront front{qkv, partials, splits, qnorm, knorm, cos_t, sin_t, rope_rows, eps};
+    return lyra::run_attention(nullptr, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace,
+                               workspace_bytes, LYRA_E_WORKSPACE, false, nullptr, nullptr, B, N, K, S, H, sm_scale,
+                               sliding_window, kv_dtype, out_dtype, stream, &front);
+}
 
 extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v, const float* k_scale,
                                      const float* v_scale, const float* sinks, const int32_t* position,

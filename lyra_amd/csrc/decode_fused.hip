@@ -11,8 +11,6 @@
 
 namespace lyra {
 
-__device__ __forceinline__ float bf16r(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
-
 __device__ __forceinline__ float block_sum(float v, float* sm) {  // blockDim.x <= 1024, multiple of 64; sm: 16 floats nobody else uses
     v = wave_sum(v);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
@@ -230,11 +228,6 @@ struct QkvPostParams {
     int splits;
 };
 
-__device__ __forceinline__ uint8_t f32_to_e4m3fn(float v) {  // round to nearest even; |v| <= 448 by construction
-    const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false);
-    return (uint8_t)(packed & 0xFF);
-}
-
 __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
     const int lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, head) over N + 2K heads
@@ -286,17 +279,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
         a = bf16_bits_to_f32(src[lane]);
         c = bf16_bits_to_f32(src[lane + half]);
     }
-    if (is_q || is_k) {
-        if (ns) {
-            const float ss = wave_sum(a * a + c * c);
-            const float inv = rsqrtf(ss / (float)p.H + p.eps);
-            a = bf16r(a * inv * ns_a);
-            c = bf16r(c * inv * ns_c);
-        }
-        const float ra = bf16r(a * cs - c * sn), rc = bf16r(c * cs + a * sn);
-        a = ra;
-        c = rc;
-    }
+    if (is_q || is_k) head_norm_rope(a, c, ns != nullptr, ns_a, ns_c, cs, sn, p.eps, p.H);
     if (is_q) {
         if (active) {
             uint16_t* dst = p.q_out + ((size_t)b * p.N + hd) * p.H;

@@ -77,6 +77,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return __builtin_bit_cast(uint16_t, h);
 }
 
+// a float32 value rounded to bf16 and back (where the JAX code holds a bf16 array)
+__device__ __forceinline__ float bf16r(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// float32 -> e4m3fn code, round to nearest even; |v| <= 448 by construction
+__device__ __forceinline__ uint8_t f32_to_e4m3fn(float v) {
+    const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false);
+    return (uint8_t)(packed & 0xFF);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Exchange between the four 16-lane rows of a wavefront without going through LDS.
@@ -246,6 +255,24 @@ __device__ __forceinline__ int wave_scan_inclusive(int x) {
     x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
     x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
     return x;
+}
+
+// QK norm (when `norm`) and rotary embedding of one head row held as two halves per lane (a: element `lane`, c: element
+// `lane + H/2`), rounded to bf16 wherever the JAX code holds a bf16 array (lyra/model.py:183-191, 315-323).  Every lane of
+// the wavefront calls it (idle lanes with zeros).  One definition, with the contraction of products and sums into fused
+// multiply-adds switched off, so that every kernel that uses it rounds identically.
+__device__ __forceinline__ void head_norm_rope(float& a, float& c, bool norm, float ns_a, float ns_c, float cs, float sn,
+                                               float eps, int H) {
+#pragma clang fp contract(off)
+    if (norm) {
+        const float ss = wave_sum(a * a + c * c);
+        const float inv = rsqrtf(ss / (float)H + eps);
+        a = bf16r(a * inv * ns_a);
+        c = bf16r(c * inv * ns_c);
+    }
+    const float ra = bf16r(a * cs - c * sn), rc = bf16r(c * cs + a * sn);
+    a = ra;
+    c = rc;
 }
 
 }  // namespace lyra

@@ -199,6 +199,53 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
     return (q, vn) if unit_v else q
 
 
+def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v, sinks,
+                  sm_scale: float, sliding_window: int, n_heads: int, n_kv_heads: int, head_dim: int, eps: float, gate=None):
+    """``qkv_post`` and the decode attention in one launch (lyra/model.py:309-347): the attention kernel's workgroups sum
+    the projection's slices, apply QK norm and the rotary embedding, append the new key and value rows to the caches (in
+    place) and attend.  Results and cache contents are bit-identical to the two launches.  Returns [B, N*H] bf16, or None
+    when the launch does not exist for this shape (a ragged batch of more than 256 (row, kv head) pairs, which the
+    whole-row kernel takes): the caller then runs the two launches."""
+    N, K, H = n_heads, n_kv_heads, head_dim
+    unsummed = isinstance(qkv, Unsummed)
+    if unsummed:
+        part = qkv.partials
+        splits, B, width = part.shape
+        assert width == (N + 2 * K) * H and qkv.residual is None
+        dev = part.device
+    else:
+        B = qkv.shape[0]
+        assert qkv.dtype == torch.bfloat16 and qkv.is_contiguous() and qkv.shape[1] == (N + 2 * K) * H
+        dev = qkv.device
+    assert pos.dtype == torch.int32
+    fp8 = isinstance(cache_k, QArray)
+    if fp8:
+        assert tuple(cache_k.block) == (1, H) and cache_k.scale.dtype == torch.float32
+        kq, vq, ks, vs = cache_k.qval, cache_v.qval, cache_k.scale, cache_v.scale
+    else:
+        kq, vq, ks, vs = cache_k, cache_v, None, None
+        assert kq.dtype == torch.bfloat16
+    S = kq.shape[2]
+    assert kq.is_contiguous() and vq.is_contiguous() and tuple(kq.shape) == (B, K, S, H)
+    assert sinks.dtype == torch.float32 and sinks.numel() == N and sinks.is_contiguous()
+    if gate is not None:
+        assert gate.dtype == torch.bfloat16 and gate.is_contiguous() and gate.numel() == B * N
+    out = torch.empty((B, N * H), dtype=torch.bfloat16, device=dev)
+    stream = _stream(dev)
+    need = _L.lyra_decode_attention_workspace(B, N, K, S, H, int(sliding_window))
+    ws = _lib.workspace("attention", dev, stream, need)
+    rc = _L.lyra_decode_attention_qkv(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None,
+                                      splits if unsummed else 0, _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(),
+                                      _f32(sin_t).data_ptr(), cos_t.shape[0], float(eps), kq.data_ptr(), vq.data_ptr(), _ptr(ks),
+                                      _ptr(vs), sinks.data_ptr(), pos.data_ptr(), 0 if pos.numel() == 1 else 1, _ptr(gate),
+                                      out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, float(sm_scale),
+                                      int(sliding_window), _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_BF16, stream)
+    if rc == _lib.E_UNSUPPORTED:
+        return None
+    _lib.check(rc, "lyra_decode_attention_qkv")
+    return out
+
+
 def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,
          residual: torch.Tensor | None = None, out_scale: float | None = None, fused_swiglu: bool = False,
          swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False,

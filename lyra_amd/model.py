@@ -439,6 +439,7 @@ def _one_group(rows: int, device) -> torch.Tensor:
 
 _ONE_GROUP: dict = {}
 _SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tuning override: combine in a launch of its own
+_SEPARATE_QKV_POST = os.environ.get("LYRA_QKV_POST_KERNEL") is not None  # tuning override: QK norm + RoPE + cache append in a launch of its own
 
 
 @dataclass
@@ -450,7 +451,7 @@ class TokenRows:
 
 
 def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
-    """attention_apply as 5 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append | attention | output matmul.
+    """attention_apply as 4 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append + attention | output matmul.
     ``x`` is the residual stream or an ``Unsummed`` projection that still has to be added to it; the return value likewise
     (dense projections run split over K and leave the sum of their slices to the kernel that consumes them)."""
     from lyra_amd.kernels import decode_fused as F
@@ -467,15 +468,20 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     qkv = F.gemm_unsummed(h, w.qkv, one)
     if qkv is None:
         qkv = F.gemm(h, w.qkv, one)
-    q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps,
-                   unit_v=w.xsa_alpha is not None)
-    xsa_v = None
-    if w.xsa_alpha is not None:  # the attention launch finishes with the exclusive-self-attention step (:351-363)
-        q, xsa_v = q
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
-    attn = attn_op(cfg.mode, cfg.implementation)
-    t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
-             xsa_alpha=w.xsa_alpha).reshape(B, N * H)
+    t = None
+    if w.xsa_alpha is None and not _SEPARATE_QKV_POST:  # QK norm + RoPE + cache append inside the attention launch
+        t = F.attention_qkv(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, w.sinks, H**-0.5,
+                            sliding_window, N, K, H, cfg.norm_eps, gate=gate)
+    if t is None:  # (learned exclusive self attention, or a ragged batch the whole-row attention kernel takes)
+        q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps,
+                       unit_v=w.xsa_alpha is not None)
+        xsa_v = None
+        if w.xsa_alpha is not None:  # the attention launch finishes with the exclusive-self-attention step (:351-363)
+            q, xsa_v = q
+        attn = attn_op(cfg.mode, cfg.implementation)
+        t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
+                 xsa_alpha=w.xsa_alpha).reshape(B, N * H)
     out = F.gemm_unsummed(t, w.out, one)
     if out is None:
         return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache

@@ -432,3 +432,82 @@ def test_sample_token_draws_from_the_topk_softmax():
     want = torch.softmax(torch.from_numpy(row[top] / np.float32(0.8)), 0).numpy()
     got = np.array([(picks == t).mean() for t in top])
     np.testing.assert_allclose(got, want, atol=0.015)  # 32768 draws: ~4 standard errors
+
+
+@pytest.mark.parametrize("B,N,K,S,H,fp8,qknorm,sw,unsummed,positions", [
+    (64, 16, 4, 4096, 128, True, True, 0, True, "full"),        # headline shape: one workgroup per (row, kv head)
+    (64, 16, 4, 4096, 128, True, True, 128, True, "full"),      # sliding layer
+    (8, 16, 4, 4096, 128, True, True, 0, True, "ragged"),       # chunked launch: only one chunk holds the new key
+    (8, 16, 4, 4096, 128, True, True, 128, True, "ragged"),
+    (3, 8, 2, 300, 64, True, False, 0, False, "short"),         # positions inside the tiles requested before the append
+    (5, 8, 8, 515, 64, False, True, 0, True, "short"),
+    (4, 32, 2, 700, 128, False, False, 33, False, "ragged"),    # 16 query heads per kv head, bf16 cache
+    (10, 6, 2, 1000, 128, True, True, 0, True, "edges"),        # tile and chunk boundaries, first row, outside the cache
+    (70, 4, 4, 200, 64, True, True, 0, True, "ragged"),         # 280 pairs, one position per row: the whole-row kernel's case, refused
+])
+def test_attention_with_the_front_step_equals_the_two_launches(B, N, K, S, H, fp8, qknorm, sw, unsummed, positions):
+    """lyra_decode_attention_qkv against lyra_qkv_post(_sum) followed by lyra_decode_attention on copies of the same
+    caches: outputs and every byte of the caches must be identical."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.kernels.decode_attention import decode_attention
+    from lyra_amd.nn.quant import QArray, quantize
+
+    _say(f"attention_qkv B{B} N{N} K{K} S{S} H{H} fp8={fp8} qknorm={qknorm} sw={sw} unsummed={unsummed} {positions}")
+    dev = U.dev()
+    rng = np.random.default_rng(B * 3 + N + S)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(S + B)
+    width = (N + 2 * K) * H
+    if unsummed:
+        part = torch.randn(3, B, width, device=dev, generator=gen) * 0.8
+        qkv_a, qkv_b = F.Unsummed(part, None, 1.0), F.Unsummed(part.clone(), None, 1.0)
+    else:
+        t = (torch.randn(B, width, device=dev, generator=gen) * 2).to(torch.bfloat16)
+        qkv_a, qkv_b = t, t.clone()
+    qn = U.t_f32((1 + 0.1 * rng.standard_normal(H)).astype(np.float32)) if qknorm else None
+    kn = U.t_f32((1 + 0.1 * rng.standard_normal(H)).astype(np.float32)) if qknorm else None
+    cos_t, sin_t = O.rope_tables(S, H)
+    cos_t, sin_t = U.t_f32(cos_t), U.t_f32(sin_t)
+    if positions == "full":
+        pos = torch.tensor(S - 1, dtype=torch.int32, device=dev)
+    else:
+        if positions == "short":
+            vals = rng.integers(0, 130, B)
+        elif positions == "edges":
+            vals = np.array([0, S - 1] + [31, 32, 127, 128, 255, 256, S, -1][: max(0, B - 2)])[:B]
+        else:
+            vals = rng.integers(0, S, B)
+            vals[0] = S - 1
+        pos = torch.from_numpy(np.asarray(vals, dtype=np.int32)).to(dev)
+    hist = torch.randn(B, K, S, H, device=dev, generator=gen).to(torch.bfloat16)
+    hist2 = torch.randn(B, K, S, H, device=dev, generator=gen).to(torch.bfloat16)
+
+    def caches():
+        if fp8:
+            qk, qv = quantize(hist, torch.float8_e4m3fn, (1, H)), quantize(hist2, torch.float8_e4m3fn, (1, H))
+            return QArray(qk.qval.clone(), qk.scale.clone(), (1, H)), QArray(qv.qval.clone(), qv.scale.clone(), (1, H))
+        return hist.clone(), hist2.clone()
+
+    sinks = U.t_f32(rng.standard_normal(N).astype(np.float32))
+    gate = (2 * torch.sigmoid(torch.randn(B, N, device=dev, generator=gen))).to(torch.bfloat16)
+    ka, va = caches()
+    kb_, vb = caches()
+    got = F.attention_qkv(qkv_a, qn, kn, cos_t, sin_t, pos, ka, va, sinks, H**-0.5, sw, N, K, H, 1e-5, gate=gate)
+    if positions == "ragged" and sw == 0 and B * K > 256:
+        assert got is None  # the whole-row kernel's case: the caller runs the two launches
+        return
+    assert got is not None
+    q = F.qkv_post(qkv_b, qn, kn, cos_t, sin_t, pos, kb_, vb, N, K, H, 1e-5)
+    want = decode_attention(q[:, :, None, :], kb_, vb, sinks, H**-0.5, sw, pos, gate=gate, implementation="pallas").reshape(B, N * H)
+    torch.cuda.synchronize()
+    for name, a, b in (("k", ka, kb_), ("v", va, vb)):
+        if fp8:
+            assert torch.equal(a.qval.view(torch.uint8), b.qval.view(torch.uint8)), f"{name} codes differ"
+            assert torch.equal(a.scale, b.scale), f"{name} scales differ"
+        else:
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"{name} cache differs"
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16)), \
+        f"outputs differ in {(got != want).sum().item()} of {got.numel()} values, max {(got.float() - want.float()).abs().max().item()}"
+    # a second call on the same caches (the row is appended again, identically) must give the same result
+    got2 = F.attention_qkv(qkv_a, qn, kn, cos_t, sin_t, pos, ka, va, sinks, H**-0.5, sw, N, K, H, 1e-5, gate=gate)
+    assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
