@@ -76,15 +76,18 @@ def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup):
     return elapsed, one_step
 
 
-def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13):
+def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13, front=False):
     """Average duration of the FP8 global-layer decode-attention launch through the C ABI, HIP events on the launch
     stream.  The launches come as they do in the workload: one per global layer of the model (each on that layer's
     cache, so every launch streams from HBM), timed as a group, with a replay of the whole decode step between groups.
     (A hundred launches back to back measure something else: at 6 TB/s the device reaches its power limit within
-    milliseconds and the launch time climbs from 44 to 54 us.)"""
+    milliseconds and the launch time climbs from 44 to 54 us.)
+    ``front``: the launch the decode step itself uses, which also does the step in front of the attention (QK norm,
+    rotary embedding, cache append: lyra_decode_attention_qkv) from the unsummed slices of the q/k/v projection."""
     import torch
 
     from lyra_amd import _lib
+    from lyra_amd.model import _rope_tables
 
     dev = weights.emb.device
     L = _lib.lib
@@ -93,12 +96,27 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13):
     out = torch.empty_like(q)
     pos = torch.full((1,), ctx - 1, dtype=torch.int32, device=dev)
     layers = [c for i, c in enumerate(cache.layers) if i % 2 == 1]
-    sinks = weights.layers[1].attn.sinks
+    attn_w = weights.layers[1].attn
+    sinks = attn_w.sinks
     need = L.lyra_decode_attention_workspace(batch, N, K, ctx, H, 0)
     ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
+    if front:
+        width = (N + 2 * K) * H
+        splits = max(1, L.lyra_decode_gemm_splits(batch, cfg.n_embd, width, cfg.n_embd))
+        part = torch.randn(splits, batch, width, device=dev) * 0.5
+        cos_t, sin_t = _rope_tables(cfg, dev)
+        qn, kn = attn_w.qnorm_scale, attn_w.knorm_scale
 
     def launch(c):
+        if front:
+            rc = L.lyra_decode_attention_qkv(
+                None, part.data_ptr(), splits, qn.data_ptr() if qn is not None else None, kn.data_ptr() if kn is not None else None,
+                cos_t.data_ptr(), sin_t.data_ptr(), cos_t.shape[0], cfg.norm_eps, c.k.qval.data_ptr(), c.v.qval.data_ptr(),
+                c.k.scale.data_ptr(), c.v.scale.data_ptr(), sinks.data_ptr(), pos.data_ptr(), 0, None, out.data_ptr(), ws.data_ptr(),
+                ws.numel(), batch, N, K, ctx, H, H**-0.5, 0, _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, stream.cuda_stream)
+            _lib.check(rc, "lyra_decode_attention_qkv")
+            return
         rc = L.lyra_decode_attention(
             q.data_ptr(), c.k.qval.data_ptr(), c.v.qval.data_ptr(), c.k.scale.data_ptr(), c.v.scale.data_ptr(), sinks.data_ptr(),
             pos.data_ptr(), 0, None, out.data_ptr(), ws.data_ptr(), ws.numel(), batch, N, K, ctx, H, H**-0.5, 0,
@@ -490,6 +508,9 @@ def main():
     step_bytes = step_algorithmic_bytes(cfg, weights, args.batch, args.ctx, touched)
 
     t_attn = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step)
+    t_attn_front = None
+    if weights.layers[1].attn.xsa_alpha is None and args.batch * cfg.n_kv_heads <= 256:  # the launch the step itself uses
+        t_attn_front = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step, front=True)
     gemm_rows = time_expert_matmuls(dev, one_step, torch.cuda.current_stream(dev)) if not args.no_gemm_roofline else None
     attn_bytes = attention_algorithmic_bytes(args.batch, cfg.n_kv_heads, args.ctx, cfg.head_dim, fp8=True)
     achieved = attn_bytes / t_attn / 1e9
@@ -536,6 +557,14 @@ def main():
             "us_per_launch": t_attn * 1e6,
         },
     }
+    if t_attn_front is not None:
+        # the same launch with the step in front of it fused in (what the decode step runs): same cache bytes, more to do
+        result["roofline"]["with_front_step"] = {
+            "kernel": "decode_attention_kernel<128, fp8, QK norm + RoPE + cache append> (global layer)",
+            "us_per_launch": t_attn_front * 1e6,
+            "achieved": attn_bytes / t_attn_front / 1e9,
+            "frac": attn_bytes / t_attn_front / 1e9 / HBM_PEAK_GBS,
+        }
     if gemm_rows is not None:
         result["roofline"]["gemm"] = gemm_rows
     if args.traffic_probe:
