@@ -444,6 +444,9 @@ def test_sample_token_draws_from_the_topk_softmax():
     (4, 32, 2, 700, 128, False, False, 33, False, "ragged"),    # 16 query heads per kv head, bf16 cache
     (10, 6, 2, 1000, 128, True, True, 0, True, "edges"),        # tile and chunk boundaries, first row, outside the cache
     (70, 4, 4, 200, 64, True, True, 0, True, "ragged"),         # 280 pairs, one position per row: the whole-row kernel's case, refused
+    (64, 32, 8, 4096, 128, True, True, 0, True, "full"),        # lyra-medium: 512 pairs, two workgroups per compute unit
+    (64, 64, 8, 4096, 64, True, False, 0, False, "full"),       # gpt-oss shape: 8 query heads per kv head, head width 64
+    (64, 64, 8, 4096, 64, True, False, 128, False, "full"),
 ])
 def test_attention_with_the_front_step_equals_the_two_launches(B, N, K, S, H, fp8, qknorm, sw, unsummed, positions):
     """lyra_decode_attention_qkv against lyra_qkv_post(_sum) followed by lyra_decode_attention on copies of the same

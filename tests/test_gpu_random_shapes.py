@@ -154,3 +154,29 @@ def test_fused_step_kernels_at_drawn_shapes(seed):
     kk, temperature = int(rng.integers(1, 9)), float(rng.choice([0.3, 0.8, 1.0, 1.5]))
     _note(f"fused draw {seed}: sample_topk rows={rows} cols={cols} ld={ld} k={kk} T={temperature}")
     TF.test_sample_topk_matches_oracle(rows, cols, ld, kk, temperature)
+
+
+def _draw_front_step(seed):
+    rng = np.random.default_rng(seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    H, K, G = pick([64, 128]), pick([1, 2, 4, 8]), pick([1, 2, 3, 4, 8, 16])
+    B, S = int(rng.integers(1, 71)), int(rng.integers(2, 1500))
+    positions = pick(["full", "ragged", "short", "edges"])
+    if positions == "edges":
+        B = min(B, 10)
+    if positions != "full":
+        B = min(B, 256 // K)  # more pairs than compute units with one position per row is the whole-row kernel's case
+    return dict(B=B, N=K * G, K=K, S=S, H=H, fp8=bool(rng.integers(0, 2)), qknorm=bool(rng.integers(0, 2)),
+                sw=pick([0, 0, 1, 33, 128, 1000]), unsummed=bool(rng.integers(0, 2)), positions=positions)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_attention_front_step_at_drawn_shapes(seed):
+    """The attention launch that also does QK norm, rotary embedding and cache append, against the two separate launches
+    (outputs and cache bytes identical; tests/test_gpu_fused.py), at drawn head counts, cache lengths and positions."""
+    from tests import test_gpu_fused as TF
+
+    d = _draw_front_step(13000 + seed)
+    _note(f"front step draw {seed}: {d}")
+    TF.test_attention_with_the_front_step_equals_the_two_launches(
+        d["B"], d["N"], d["K"], d["S"], d["H"], d["fp8"], d["qknorm"], d["sw"], d["unsummed"], d["positions"])
