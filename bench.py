@@ -30,13 +30,16 @@ def attention_algorithmic_bytes(batch, kv_heads, visible, head_dim, fp8=True):
     return 2 * batch * kv_heads * visible * per_row
 
 
-def build_model(batch, ctx, device, variant="lyra-small"):
+def build_model(batch, ctx, device, variant="lyra-small", layout="headline"):
     import torch
 
     from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights
     from lyra_amd.nn.quant import QArray
 
-    cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True, fp8_attn=True, per_channel=True)
+    if layout == "reference-fp8":  # what the reference's serve path sets with --fp8 (generate.py:31-38), nothing more
+        cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True)
+    else:
+        cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True, fp8_attn=True, per_channel=True)
     weights = init_weights(cfg, device)
     cache = init_cache(cfg, batch, ctx, device)
     g = torch.Generator(device=device)
@@ -471,6 +474,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm-roofline", action="store_true", help="skip the stand-alone expert matmul timings")
+    ap.add_argument("--layout", default="headline", choices=["headline", "reference-fp8"],
+                    help="headline: FP8 cache, every projection and MLP weight FP8 with one scale per output channel; "
+                         "reference-fp8: FP8 cache and MLP weights with (256, 256) scale blocks, attention projections bf16")
     ap.add_argument("--model", default="lyra-small", help="model variant of the decode step (the headline figure is lyra-small)")
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
@@ -494,7 +500,7 @@ def main():
                   f"{100 * r['cold_frac_of_peak']:.1f} | {r['hot_us']:.1f} |", file=sys.stderr)
         print(json.dumps({"metric": "operator launch time at model shapes", "unit": "us", "peak_GBs": HBM_PEAK_GBS, "kernels": rows}))
         return
-    cfg, weights, cache = build_model(args.batch, args.ctx, dev, args.model)
+    cfg, weights, cache = build_model(args.batch, args.ctx, dev, args.model, args.layout)
     elapsed, one_step = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
     tokens_per_s = args.batch * args.steps / elapsed
 
@@ -536,14 +542,16 @@ def main():
         "config": {
             "workload": f"full {args.model} decode step ({cfg.n_layers} layers, {cfg.n_attn_heads}Q/{cfg.n_kv_heads}KV heads, "
                         f"H={cfg.head_dim}, {cfg.n_routed_experts}+{cfg.n_shared_experts} experts, LM head {cfg.padded_vocab_size}), "
-                        f"B={args.batch}, ctx {args.ctx}, FP8 KV cache, FP8 per-output-channel weights, greedy sampling",
+                        f"B={args.batch}, ctx {args.ctx}, FP8 KV cache, " + ("FP8 per-output-channel weights" if args.layout == "headline" else
+                        "FP8 MLP weights with (256, 256) scale blocks, bf16 attention projections") + ", greedy sampling",
             "batch": args.batch,
             "ctx": args.ctx,
             "us_per_layer": elapsed / args.steps / cfg.n_layers * 1e6,
             "step_algorithmic_bytes": step_bytes,
             "step_frac": step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,  # of the 8 TB/s roofline, whole step
             "experts_with_rows_per_moe_layer": touched,
-            "projections": "q/k/v and output projections FP8 as well (quantize_attn; the reference's --fp8 leaves them bf16)",
+            "projections": ("q/k/v and output projections FP8 as well (quantize_attn; the reference's --fp8 leaves them bf16)"
+                            if args.layout == "headline" else "q/k/v and output projections bf16, as the reference's --fp8 leaves them"),
         },
         "roofline": {
             "kernel": "decode_attention_kernel<128, fp8> (global layer)",
