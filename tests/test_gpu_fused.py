@@ -20,11 +20,18 @@ def _say(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def _bf16_close(got, want, what):
-    """Equal up to one bf16 step of a float32 oracle value rounded to bf16."""
+def _bf16_close(got, want, what, update=None):
+    """Equal up to one bf16 step of a float32 oracle value rounded to bf16.
+
+    `update`: where the value is residual + update and the update went through two bf16 roundings of its own (the
+    weighted sum, then the sum times the residual scale), a different order of the float32 additions behind the sum can
+    move the first rounding by one step and with it the second by up to two steps of the update - more than a step of
+    the result where residual and update nearly cancel.  That much is allowed on top."""
     got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
     err = np.abs(got - O.bf16_round(want.copy()))
     bound = np.abs(want) * 2.0**-7 + 1e-30
+    if update is not None:
+        bound = bound + np.abs(np.asarray(update, np.float32)) * 2.0**-6
     assert (err <= bound).all(), f"{what}: {int((err > bound).sum())} values off by more than one bf16 step, max {err.max()}"
     assert (err == 0).mean() > 0.97, f"{what}: only {(err == 0).mean():.3f} bit-identical"
 
@@ -215,7 +222,7 @@ def test_moe_combine(T, topk, C):
     t = O.bf16_round(O.combine(rows, scores, dest))
     t = O.bf16_round(t * np.float32(rs))
     want = x + t
-    _bf16_close(U.to_np(out), want, "combine")
+    _bf16_close(U.to_np(out), want, "combine", update=t)
 
 
 @pytest.mark.parametrize("fp8", [False, True])
@@ -375,7 +382,7 @@ def test_uncombined_moe_layer_end_equals_combine_then_norm(T, topk, C, n, gate):
     assert torch.equal(x1, x2) and torch.equal(h1, h2)
     assert (y1 is None and y2 is None) or torch.equal(y1, y2)
     t = O.bf16_round(O.bf16_round(O.combine(rows_np, scores_np, dest_np)) * np.float32(rs))
-    _bf16_close(U.to_np(x1), x_np + t, "combined row")
+    _bf16_close(U.to_np(x1), x_np + t, "combined row", update=t)
 
 
 @pytest.mark.parametrize("rows,cols,ld,k,temperature", [(64, 201088, 204800, 4, 0.8), (3, 1000, 1024, 8, 1.5), (130, 5000, 5000, 1, 0.3),
