@@ -56,6 +56,11 @@ def test_argument_validation_needs_no_gpu():
     assert L.lyra_decode_attention(one, one, one, None, None, one, one, 0, None, one, None, 0, 1, 16, 5, 512, 128, 0.1, 0, 0, 0, None) == -1  # N % K
     assert L.lyra_decode_attention(one, one, one, None, None, one, one, 0, None, one, None, 0, 1, 16, 4, 512, 96, 0.1, 0, 0, 0, None) == -2  # head dim
     assert L.lyra_decode_gemm(None, None, None, 0, 0, None, None, None, None, 0, 4, 1, 64, 128, 0, 0, 0, 1.702, 7.0, None) == -1
+    # the attention launch with the front step: neither form of the projection given; a head width it does not cover
+    assert L.lyra_decode_attention_qkv(None, None, 0, None, None, one, one, 512, 1e-5, one, one, None, None, one, one, 0, None, one, None, 0,
+                                       1, 16, 4, 512, 128, 0.1, 0, 0, 0, None) == -1
+    assert L.lyra_decode_attention_qkv(one, None, 0, None, None, one, one, 512, 1e-5, one, one, None, None, one, one, 0, None, one, None, 0,
+                                       1, 16, 4, 512, 96, 0.1, 0, 0, 0, None) == -2
     assert L.lyra_decode_gemm(one, one, None, 0, 0, one, None, one, None, 0, 4, 1, 48, 128, 0, 0, 0, 1.702, 7.0, None) == -2  # K % 32
     assert L.lyra_decode_gemm(one, one, None, 0, 0, one, None, one, None, 0, 4, 1, 64, 128, 1, 0, 0, 1.702, 7.0, None) == -1  # fp8 without scales
     assert L.lyra_rmsnorm_proj(None, None, None, None, None, None, 1, 64, 0, 2, 1e-5, None) == -1
