@@ -180,3 +180,31 @@ def test_attention_front_step_at_drawn_shapes(seed):
     _note(f"front step draw {seed}: {d}")
     TF.test_attention_with_the_front_step_equals_the_two_launches(
         d["B"], d["N"], d["K"], d["S"], d["H"], d["fp8"], d["qknorm"], d["sw"], d["unsummed"], d["positions"])
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_variants_of_the_matmul_and_the_norm_at_drawn_shapes(seed):
+    """The equalities of tests/test_gpu_fused.py - row gather and residual epilogue inside the matmul, K slices summed by
+    the consumer, the MoE combine left to the norm behind it - bit for bit at drawn sizes."""
+    from tests import test_gpu_fused as TF
+
+    rng = np.random.default_rng(15000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    fp8, swiglu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    G, K, N = pick([1, 1, 2, 3, 8, 16, 40]), 32 * pick([1, 2, 4, 8, 16, 32, 64]), (256 if swiglu else 128) * pick([1, 2, 3, 8, 16])
+    while G * K * N > (1 << 24):
+        G = max(1, G // 2)
+    M = int(rng.integers(1, 321))
+    _note(f"variants draw {seed}: row map / residual fp8={fp8} M={M} G={G} K={K} N={N} swiglu={swiglu}")
+    TF.test_gemm_row_map_and_residual_epilogue(fp8, M, G, K, N, swiglu)
+
+    H, Kh, Gq = pick([64, 128]), pick([1, 2, 4]), pick([1, 2, 4])
+    if Kh * Gq * H % 256 == 0:  # (the output projection's scale blocks are (256, 256))
+        fp8, B, C = bool(rng.integers(0, 2)), int(rng.integers(1, 131)), pick([256, 512, 1024, 2048, 4096])
+        _note(f"variants draw {seed}: unsummed fp8={fp8} B={B} C={C} N={Kh * Gq} K={Kh} H={H}")
+        TF.test_unsummed_projection_consumers_equal_summed_path(fp8, B, C, Kh * Gq, Kh, H)
+
+    T, topk, gate = int(rng.integers(1, 131)), int(rng.integers(1, 17)), bool(rng.integers(0, 2))
+    C, n = 8 * int(rng.integers(8, 600)), pick([1, 7, 15, 16, 32, 64]) if gate else pick([0, 1, 7, 15, 16, 63])
+    _note(f"variants draw {seed}: uncombined T={T} topk={topk} C={C} n={n} gate={gate}")
+    TF.test_uncombined_moe_layer_end_equals_combine_then_norm(T, topk, C, n, gate)

@@ -74,3 +74,22 @@ def test_static_scratch_rejects_what_does_not_fit():
     assert L.lyra_decode_attention_static(one, one, one, None, None, one, one, 1, None, one, 255, 16, 1, 8192, 128, 0.1, 0, 0, 0, None) == -5
     assert L.lyra_decode_attention_workspace(128, 16, 1, 8192, 128, 0) <= limit
     assert b"static scratch" in L.lyra_strerror(-5)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_static_scratch_entry_point_at_drawn_shapes(seed):
+    """Few rows, long caches, one position per row (rows that see no key included): mostly chunked launches, whose partial
+    results and counters then live in the static array; bit-identical to the workspace entry point, call after call."""
+    from lyra_amd import _lib
+
+    rng = np.random.default_rng(50000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    H, K, G = pick([64, 128]), pick([1, 2, 4, 8]), pick([1, 2, 4, 8])
+    B, S, sw = int(rng.integers(1, 13)), int(rng.integers(300, 6000)), pick([0, 0, 0, 128, 700])
+    pos = rng.integers(-1, S, B).tolist()
+    print(f"static scratch draw {seed}: B={B} N={K * G} K={K} S={S} H={H} sw={sw} pos={pos}", file=sys.stderr, flush=True)
+    assert _lib.lib.lyra_decode_attention_workspace(B, K * G, K, S, H, sw) <= 4 << 20
+    case = U.attention_case(seed, B, K * G, K, S, H, fp8=True)
+    ref = _call(case, B, K * G, K, S, H, pos, sw, static=False)
+    got = _call(case, B, K * G, K, S, H, pos, sw, static=True)
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
