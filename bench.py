@@ -509,7 +509,7 @@ def main():
     from lyra_amd.model import model_apply
 
     cache.pos.fill_(args.ctx - 1)
-    model_apply(torch.arange(args.batch, device=dev) % cfg.vocab_size, weights, cache, cfg, groups_out=groups)
+    model_apply(torch.arange(args.batch, device=dev) % cfg.vocab_size, weights, cache, cfg, groups_out=groups, advance=False)
     touched = [int((g > 0).sum().item()) for g in groups]
     step_bytes = step_algorithmic_bytes(cfg, weights, args.batch, args.ctx, touched)
 

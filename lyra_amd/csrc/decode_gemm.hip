@@ -237,7 +237,7 @@ void decode_gemm_kernel(GemmParams p) {
     // which 128-column span this wavefront owns: 4 per workgroup, or (p.even_spans, one workgroup per compute unit)
     // workgroup i of n takes spans [i * total / n, (i + 1) * total / n), so that every compute unit has the same number
     // of spans to within one - 1600 spans as 400 workgroups of 4 leave 144 compute units with 8 spans and 112 with 4
-    const int total_spans = p.swiglu ? (p.N >> 1) / 64 : p.N / 128;
+    const int total_spans = p.swiglu ? ((p.N >> 1) + 63) / 64 : (p.N + 127) / 128;  // (the last span may be partly filled)
     const int first_span = p.even_spans ? (int)((long)blockIdx.x * total_spans / gridDim.x) : (int)blockIdx.x * kGemmWaves;
     const int end_span = p.even_spans ? (int)((long)(blockIdx.x + 1) * total_spans / gridDim.x) : total_spans;
     const int span = first_span + wave;
@@ -251,20 +251,20 @@ void decode_gemm_kernel(GemmParams p) {
     const int pad_from = (g == p.G - 1 && rpar == 0 && p.ksplit == 1 && ks == 0) ? off + cnt : p.M;  // rows past the last group
     if (cnt <= rpar * 16 * MT && pad_from >= p.M) return;  // no rows for this workgroup: its weights are never touched
 
-    // columns of this lane
+    // columns of this lane (span_ok: they exist - N need not be a multiple of the span, only of 8 columns)
     int ncol, out_col;
     bool span_ok;
     const bool is_lin_lane = p.swiglu && x >= 8;
     if (p.swiglu) {
         const int half = p.N >> 1;
-        span_ok = span < end_span && span * 64 < half;
         out_col = span * 64 + 8 * (x & 7);
+        span_ok = span < end_span && out_col + 8 <= half;
         ncol = is_lin_lane ? half + out_col : out_col;
     } else {
-        span_ok = span < end_span && span * 128 < p.N;
         ncol = out_col = span * 128 + 8 * x;
+        span_ok = span < end_span && ncol + 8 <= p.N;
     }
-    if (!span_ok) ncol = out_col = 0;  // idle wavefront of the last workgroup: keeps pace, stores nothing
+    if (!span_ok) ncol = out_col = 0;  // idle wavefront of the last workgroup, lanes past the last column: keep pace, store nothing
 
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
     const int row_bytes = p.N * ES;
@@ -1453,7 +1453,9 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
     static const bool no_split_k = getenv("LYRA_GEMM_NO_SPLIT_K") != nullptr;
     pl.one_pass = false;
     static const bool no_grouped = getenv("LYRA_GEMM_NO_GROUPED") != nullptr;
-    pl.grouped = G > 1 && G <= kMaxStreamGroups && G + M / (16 * kGroupTiles) <= kMaxRowBlocks && !no_grouped;
+    // the kernels built on whole 128-column spans; any other width (a multiple of 8) goes to the general kernel
+    const bool whole_spans = N % 128 == 0 && (!fused_swiglu || N % 256 == 0);
+    pl.grouped = G > 1 && G <= kMaxStreamGroups && G + M / (16 * kGroupTiles) <= kMaxRowBlocks && whole_spans && !no_grouped;
     if (pl.grouped) {
         pl.mt = 4;
         pl.row_par = 1;
@@ -1465,7 +1467,7 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
         pl.split_k = false;
         return pl;
     }
-    pl.split_k = allow_split_k && G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && !no_split_k;
+    pl.split_k = allow_split_k && G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && whole_spans && !no_split_k;
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
         pl.mt = 4;
@@ -1498,7 +1500,7 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
         pl.ksplit = (K + kpart - 1) / kpart;
         if (pl.split_k) return pl;
     }
-    pl.one_pass = G == 1 && weight_bytes <= 48e6 && !no_one_pass;
+    pl.one_pass = G == 1 && weight_bytes <= 48e6 && whole_spans && !no_one_pass;
     if (pl.one_pass) {
         pl.mt = 1;
         pl.row_par = (M + 15) / 16;
@@ -1625,7 +1627,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
-    if (K % 32 || N % 128 || (fused_swiglu && N % 256) || G > 8191) return LYRA_E_UNSUPPORTED;
+    if (K % 32 || N % 8 || (fused_swiglu && N % 16) || G > 8191) return LYRA_E_UNSUPPORTED;  // (a lane holds 8 columns)
     if ((size_t)M * N * 4 >= (1ull << 31)) return LYRA_E_UNSUPPORTED;  // results are stored through 31-bit buffer offsets
 
     GemmParams p;

@@ -42,7 +42,7 @@ def select_decode_gemm_config(m: int, groups: int, k: int, n: int, quant_dtype=N
     if min(m, groups, k, n) <= 0 or groups > _MAX_GROUPS:
         return None
     quant_dtype = quant_dtype if quant_dtype is not None and is_scaled(quant_dtype) else None
-    if k % 32 or n % 128 or (fused_swiglu and n % 256):
+    if k % 32 or n % 8 or (fused_swiglu and n % 16):  # (whole 128-column spans get the streaming kernels, other widths the general one)
         return None
     if quant_dtype is not None:
         if quant_dtype != torch.float8_e4m3fn:
@@ -208,7 +208,7 @@ def decode_gemm(
             swiglu_beta=swiglu_beta, swiglu_limit=swiglu_limit, out_dtype=out_dtype,
         )
 
-    tiling = None if config is None else f"n128/k32 dtype={'fp8' if config.fwd_dtype else 'bf16'}"
+    tiling = None if config is None else f"n8/k32 dtype={'fp8' if config.fwd_dtype else 'bf16'}"
     op_shape = f"m{M} g{G} k{K} n{N}"
     return dispatch_kernel(
         "decode_gemm", implementation=implementation, shape=op_shape, config=config, tiling=tiling, kernel=kernel, reference=reference

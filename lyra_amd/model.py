@@ -315,15 +315,25 @@ def init_cache(cfg: ModelConfig, batch: int, length: int, device) -> ModelCache:
 
 
 def cache_update(cache: LayerCache, k: torch.Tensor, v: torch.Tensor, pos: torch.Tensor) -> LayerCache:
-    """lyra/model.py:204-212 / quant.py:89-98 for one new token, written in place at ``pos`` (device scalar)."""
-    idx = pos.to(torch.int64).reshape(1)
+    """lyra/model.py:204-212 / quant.py:89-98 for one new token, written in place at ``pos`` (device scalar).
+
+    A position outside the cache writes nothing, as in the HIP kernels that append (the index lives on the device and
+    ``index_copy_`` does not check it: the row at the clamped index is read and written back unchanged instead)."""
+    S = (cache.k.qval if isinstance(cache.k, QArray) else cache.k).shape[2]
+    p64 = pos.to(torch.int64).reshape(1)
+    inside = (p64 >= 0) & (p64 < S)
+    idx = p64.clamp(0, S - 1)
+
+    def put(dst: torch.Tensor, new: torch.Tensor):
+        dst.index_copy_(2, idx, torch.where(inside, new, dst.index_select(2, idx)))
+
     for dst, new in ((cache.k, k), (cache.v, v)):
         if isinstance(dst, QArray):
             q = quantize(new, dst.dtype, dst.block, dst.stype)
-            dst.qval.view(torch.uint8).index_copy_(2, idx, q.qval.view(torch.uint8))
-            dst.scale.index_copy_(2, idx, q.scale)
+            put(dst.qval.view(torch.uint8), q.qval.view(torch.uint8))
+            put(dst.scale, q.scale)
         else:
-            dst.index_copy_(2, idx, new.to(dst.dtype))
+            put(dst, new.to(dst.dtype))
     return cache
 
 
@@ -398,12 +408,14 @@ def bpermute(expert_ids: torch.Tensor):
     return permutation, destinations
 
 
-def moe_apply(x, w: MoEWeights, cfg: ModelConfig):
+def moe_apply(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None = None):
     """lyra/model.py:498-567 without expert parallelism."""
     B, C = x.shape
     gmm = gmm_op(cfg.mode, cfg.implementation)
     xn = rms_norm(x, w.norm_scale, cfg.norm_eps)
     scores, active_map, groups = route_tokens(xn, w, cfg)
+    if groups_out is not None:
+        groups_out.append(groups)
     topk = cfg.n_active_experts
     permute_map, unpermute_map = bpermute(active_map)
     t = xn[permute_map // topk]
@@ -567,7 +579,7 @@ def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cf
                 groups_out: list | None = None, advance: bool = True):
     """lyra/model.py:734-793 in decode mode: tokens [B] int -> (logits [B, V_padded] f32, cache advanced by one).
     ``hidden_out``: optional list that receives the residual stream after the last layer [B, C] (for parity checks);
-    ``groups_out``: optional list that receives the rows-per-expert tensor of every MoE layer (fused driver only);
+    ``groups_out``: optional list that receives the rows-per-expert tensor of every MoE layer;
     ``advance=False`` leaves ``cache.pos`` where it is (the caller's sampler advances it, or nobody does)."""
     if _fused_supported(model, cfg):
         return model_apply_fused(tokens, model, cache, cfg, hidden_out, groups_out, advance)
@@ -577,7 +589,7 @@ def model_apply(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cf
     cos, sin = cos_t.index_select(0, pos.to(torch.int64).reshape(1))[0], sin_t.index_select(0, pos.to(torch.int64).reshape(1))[0]
     for idx, layer in enumerate(model.layers):
         h, _ = attention_apply(h, layer.attn, idx, pos, cos, sin, cache.layers[idx], cfg)
-        h = moe_apply(h, layer.mlp, cfg) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply(h, layer.mlp, cfg)
+        h = moe_apply(h, layer.mlp, cfg, groups_out) if isinstance(layer.mlp, MoEWeights) else dense_mlp_apply(h, layer.mlp, cfg)
     if hidden_out is not None:
         hidden_out.append(h)
     h = rms_norm(h, model.norm_scale, cfg.norm_eps)

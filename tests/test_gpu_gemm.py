@@ -42,11 +42,12 @@ def _case(seed, M, G, K, N, sizes, *, kind, block=(256, 256), bias=False, w_std=
     return c
 
 
-def _want(c, swiglu, big=False):
-    # Several groups with scale blocks shorter than K: the kernel dequantises like the reference, f32(code) * scale rounded
-    # to bf16 (lyra/nn/quant.py:82-85), so that is the operand the float32 product is taken on.  Everywhere else the
-    # scales factor out of the product and are applied to the float32 sums.
-    like_reference = c["kind"] == "fp8" and len(c["sizes"]) > 1 and c["block"][0] < c["lhs"].shape[1]
+def _want(c, swiglu, big=False, general_kernel=False):
+    # Several groups with scale blocks shorter than K: the expert kernel dequantises like the reference, f32(code) * scale
+    # rounded to bf16 (lyra/nn/quant.py:82-85), so that is the operand the float32 product is taken on.  Everywhere else -
+    # and in the general kernel, which takes the widths that are not whole spans - the scales factor out of the product
+    # and are applied to the float32 sums.
+    like_reference = c["kind"] == "fp8" and len(c["sizes"]) > 1 and c["block"][0] < c["lhs"].shape[1] and not general_kernel
     if big:  # the C restatement (same arithmetic, threaded) for shapes numpy would take minutes on
         if c["kind"] == "fp8":
             q, s = c["w"]
@@ -390,3 +391,35 @@ def test_zero_and_extreme_block_scales(G, M):
     got = _run(c, False)
     assert np.isfinite(got).all()
     U.assert_close(got, want, atol=2e-2 * max(1.0, float(np.abs(want).max()) / 50), what="zero / extreme scales")
+
+
+@pytest.mark.parametrize("M,G,K,N,kind,block,swiglu,bias", [
+    (64, 1, 4096, 2880, "bf16", None, False, True),          # gpt-oss-20b: output projection (64 heads of 64 -> width 2880)
+    (64, 1, 2880, 5120, "fp8", (2880, 1), False, True),      # ... its q/k/v projection (whole spans, K = 2880)
+    (64, 8, 2880, 5760, "fp8", (2880, 1), True, True),       # ... expert up projection with SwiGLU: 2880 output columns
+    (64, 8, 2880, 2880, "fp8", (2880, 1), False, True),      # ... expert down projection
+    (64, 8, 2880, 2880, "bf16", None, False, False),
+    (300, 8, 2880, 2880, "fp8", (96, 64), False, True),      # several row blocks per expert, scale blocks along K
+    (40, 3, 96, 8, "bf16", None, False, False),              # one lane of columns
+    (40, 3, 96, 16, "fp8", (32, 8), True, True),             # SwiGLU down to 8 output columns
+    (70, 5, 256, 200, "fp8", (64, 8), False, False),
+    (33, 1, 512, 72, "fp8", (512, 8), False, True),
+    (16, 1, 8192, 8200, "fp8", (8192, 1), False, False),     # large enough for K slices across workgroups + the finish kernel
+])
+def test_widths_that_are_not_whole_spans(M, G, K, N, kind, block, swiglu, bias):
+    """N % 8 == 0 (N % 16 == 0 with SwiGLU) is enough: widths that do not fill their last 128-column span take the general
+    kernel, whose lanes past the last column compute along and store nothing (the reference's kernel needs n % 128 == 0,
+    decode_gemm.py:88, and runs such shapes - all of gpt-oss-20b's, width 2880 - on its XLA path)."""
+    rng = np.random.default_rng(M + G + N)
+    cuts = np.sort(rng.integers(0, M + 1, G - 1)) if G > 1 else np.zeros(0, np.int64)
+    sizes = np.diff(np.concatenate([[0], cuts, [M]])).astype(np.int32)
+    if G > 2:
+        sizes[1] = 0  # an expert without rows
+    _note(f"gemm ragged width M={M} G={G} K={K} N={N} {kind} block={block} swiglu={swiglu} bias={bias} sizes={sizes.tolist()}")
+    c = _case(N, M, G, K, N, sizes, kind=kind, block=block, bias=bias, w_std=0.03)
+    want = _want(c, swiglu, big=True, general_kernel=N % (256 if swiglu else 128) != 0)
+    got = _run(c, swiglu)
+    assert got.shape == want.shape == (M, N // 2 if swiglu else N)
+    U.assert_close(got, want, what=f"ragged width N={N}")
+    got32 = _run(c, swiglu, out_f32=True)
+    U.assert_close(got32, want, atol=4e-3, rtol=4e-3, what=f"ragged width N={N}, float32 out")

@@ -208,3 +208,33 @@ def test_fused_variants_of_the_matmul_and_the_norm_at_drawn_shapes(seed):
     C, n = 8 * int(rng.integers(8, 600)), pick([1, 7, 15, 16, 32, 64]) if gate else pick([0, 1, 7, 15, 16, 63])
     _note(f"variants draw {seed}: uncombined T={T} topk={topk} C={C} n={n} gate={gate}")
     TF.test_uncombined_moe_layer_end_equals_combine_then_norm(T, topk, C, n, gate)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_decode_gemm_at_drawn_widths_that_are_not_whole_spans(seed):
+    """As test_decode_gemm_at_drawn_shapes, with N any multiple of 8 (16 with SwiGLU) up to 1500."""
+    rng = np.random.default_rng(17000 + seed)
+    swiglu = bool(rng.integers(0, 2))
+    G = int(rng.choice([1, 1, 2, 3, 5, 8, 17]))
+    K = 32 * int(rng.choice([1, 2, 3, 5, 8, 9, 16, 23, 32, 64, 90]))
+    step = 16 if swiglu else 8
+    N = step * int(rng.integers(1, 1500 // step))
+    while G * K * N > (1 << 23):
+        G, K = max(1, G // 2), (K if G > 1 else max(32, K // 2 // 32 * 32))
+    M = int(rng.choice([1, 2, 7, 16, 17, 33, 64, 65, 130, 300]))
+    cuts = np.sort(rng.integers(0, M + 1, G - 1)) if G > 1 else np.zeros(0, np.int64)
+    sizes = np.diff(np.concatenate([[0], cuts, [M]])).astype(np.int32)
+    if G > 1:
+        sizes[rng.integers(0, G)] = 0
+    kind = "fp8" if rng.integers(0, 4) else "bf16"
+    block = None
+    if kind == "fp8":
+        bks = [K] + [b for b in (32, 64, 96, 128, 256, 512) if K % b == 0 and b < K]
+        bk = int(rng.choice(bks))
+        bns = [b for b in (1, 8, 16, 64, 128, 256) if N % b == 0 and (bk == K or b % 8 == 0)]
+        block = (bk, int(rng.choice(bns)))
+    bias = bool(rng.integers(0, 2))
+    _note(f"gemm width draw {seed}: M={M} G={G} K={K} N={N} sizes={sizes.tolist()} {kind} block={block} bias={bias} swiglu={swiglu}")
+    c = gemm_case(seed, M, G, K, N, sizes.tolist(), kind=kind, block=block, bias=bias, w_std=0.05)
+    want = gemm_want(c, swiglu, general_kernel=N % (256 if swiglu else 128) != 0)
+    U.assert_close(run_gemm(c, swiglu), want, what=f"width draw {seed}")

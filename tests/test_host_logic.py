@@ -286,3 +286,38 @@ def test_sampling():
     draws = torch.stack([sample_token(logits, cfg, g) for _ in range(200)])
     assert set(draws[:, 0].tolist()) <= {1, 2} and set(draws[:, 1].tolist()) <= {0, 3}
     assert len(set(draws[:, 0].tolist())) == 2
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_cache_append_outside_the_cache_writes_nothing(fp8):
+    """cache_update with the position on the device: a row inside the cache is written (quantised for an FP8 cache), a
+    position at or beyond its length, or below zero, leaves every byte as it was (the HIP kernels that append do the same)."""
+    from lyra_amd.model import LayerCache, cache_update
+    from lyra_amd.nn.quant import QArray, dequantize, quantize
+
+    B, K, S, H = 2, 3, 8, 16
+    g = torch.Generator().manual_seed(5)
+    hist = [torch.randn(B, K, S, H, generator=g).to(torch.bfloat16) for _ in range(2)]
+    new = [torch.randn(B, K, 1, H, generator=g).to(torch.bfloat16) for _ in range(2)]
+
+    def fresh():
+        if fp8:
+            return LayerCache(*(quantize(h, torch.float8_e4m3fn, (1, H)) for h in hist))
+        return LayerCache(*(h.clone() for h in hist))
+
+    def raw(c):
+        return [(a.qval.view(torch.uint8).clone(), a.scale.clone()) if isinstance(a, QArray) else (a.clone(),) for a in (c.k, c.v)]
+
+    before = raw(fresh())
+    for pos in (-1, S, S + 100):
+        c = cache_update(fresh(), new[0], new[1], torch.tensor(pos, dtype=torch.int32))
+        for got, want in zip(raw(c), before):
+            assert all(torch.equal(a, b) for a, b in zip(got, want)), f"position {pos} changed the cache"
+    for pos in (0, 5, S - 1):
+        c = cache_update(fresh(), new[0], new[1], torch.tensor(pos, dtype=torch.int32))
+        for arr, n, (old, *_) in zip((c.k, c.v), new, before):
+            row = dequantize(arr, torch.float32)[:, :, pos] if isinstance(arr, QArray) else arr[:, :, pos].float()
+            assert torch.allclose(row, n[:, :, 0].float(), atol=0.08 if fp8 else 0, rtol=0.07 if fp8 else 0)
+            now = arr.qval.view(torch.uint8) if isinstance(arr, QArray) else arr
+            keep = [i for i in range(S) if i != pos]
+            assert torch.equal(now[:, :, keep], old[:, :, keep])
