@@ -987,7 +987,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     int spans, kw, wslot, half, span_cols, tile_cols, n_my, trips;
     auto set_layout = [&](bool w) {
         wide = w;
-        spans = p.swiglu ? (p.N >> 1) / 128 : (w ? p.N / 256 : p.N / 128);
+        spans = p.swiglu ? ((p.N >> 1) + 127) / 128 : (w ? p.N / 256 : (p.N + 127) / 128);  // (the last span may be partly filled)
         kw = w ? 2 : kSplitWaves;
         wslot = w ? (wave & 1) : wave, half = w ? (wave >> 1) : 0;
         span_cols = p.swiglu || !w ? 128 : 256;
@@ -1115,10 +1115,13 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         row0 = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][1] : 0);
         rows = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][2] : 0);
         ncol = half * half_stride + span * span_cols + 8 * x;
+        // (N need not fill the last span: lanes past the last column - of the gate or linear half with SwiGLU - load
+        // nothing, accumulate zeros and are left out of the epilogue)
+        const bool cols = span * span_cols + (wide && !p.swiglu ? 128 * half : 0) + 8 * x < NO;
         wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
                                                   (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-        wvoff = valid ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
-        if constexpr (STEP_SCALES) sc_voff = valid ? (g * p.KB * p.NB + (ncol >> p.bn_shift)) * 4 : kNoLoad;
+        wvoff = valid && cols ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
+        if constexpr (STEP_SCALES) sc_voff = valid && cols ? (g * p.KB * p.NB + (ncol >> p.bn_shift)) * 4 : kNoLoad;
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) {
             const int r = mt * 16 + x;
@@ -1368,6 +1371,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             // operand is read with an offset outside its descriptor and yields zeros), rows two at a time
             const int oc = cur_span * span_cols + 4 * q;
             const int oc2 = p.swiglu ? NO + oc : oc + 128;  // second set of columns of a wide unit: linear columns, or the next span
+            const bool oc_live = oc < NO, oc2_live = oc + 128 < NO;  // (a last span that N does not fill: nothing is stored past N)
             const f32x4 bias_v = load_f32x4(bias_rsrc, p.bias ? (cur_g * p.N + oc) * 4 : kNoLoad);
             const f32x4 bias_l = load_f32x4(bias_rsrc, (p.bias && wide) ? (cur_g * p.N + oc2) * 4 : kNoLoad);
             const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1393,13 +1397,13 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         }
                     }
                     if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
-                        finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
-                        finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
+                        if (oc_live) finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
+                        if (oc2_live) finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
                         if (two) {
-                            finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
-                            finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
+                            if (oc_live) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
+                            if (oc2_live) finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
                         }
-                    } else {
+                    } else if (oc_live) {
                         finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, oa);
                         if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, ob);
                     }
@@ -1415,10 +1419,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
     const int total = total_rows;
     const int pad_rows = p.M - min(total, p.M);
-    const int pad_spans = p.swiglu ? spans : p.N / 128;
+    const int pad_spans = p.swiglu ? spans : (p.N + 127) / 128;
     for (int i = blockIdx.x; i < pad_rows * pad_spans; i += gridDim.x) {
-        if (threadIdx.x < 32) {
-            const int row = min(total, p.M) + i / pad_spans, sp = i % pad_spans;
+        const int sp = i % pad_spans;
+        if (threadIdx.x < 32 && sp * 128 + 4 * q < NO) {
+            const int row = min(total, p.M) + i / pad_spans;
             float vg[4] = {0.f, 0.f, 0.f, 0.f}, vl[4] = {0.f, 0.f, 0.f, 0.f};
             group_epilogue(p, vg, vl, p.G - 1, row, sp * 128 + 4 * q, NO);
         }
@@ -1455,13 +1460,13 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
     static const bool no_grouped = getenv("LYRA_GEMM_NO_GROUPED") != nullptr;
     // the kernels built on whole 128-column spans; any other width (a multiple of 8) goes to the general kernel
     const bool whole_spans = N % 128 == 0 && (!fused_swiglu || N % 256 == 0);
-    pl.grouped = G > 1 && G <= kMaxStreamGroups && G + M / (16 * kGroupTiles) <= kMaxRowBlocks && whole_spans && !no_grouped;
+    pl.grouped = G > 1 && G <= kMaxStreamGroups && G + M / (16 * kGroupTiles) <= kMaxRowBlocks && !no_grouped;  // (any width)
     if (pl.grouped) {
         pl.mt = 4;
         pl.row_par = 1;
         static const bool want_wide = getenv("LYRA_GEMM_WIDE") != nullptr;  // tuning override: 256-column units whatever their number
         pl.wide = !fused_swiglu && N % 256 == 0 && want_wide;
-        pl.spans = (fused_swiglu || pl.wide) ? N / 256 : N / 128;
+        pl.spans = fused_swiglu ? (N / 2 + 127) / 128 : (pl.wide ? N / 256 : (N + 127) / 128);
         pl.ksplit = 1;
         pl.kpart = K;
         pl.split_k = false;

@@ -477,9 +477,11 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
     B = x.shape[0]
     one = _one_group(B, x.device)
-    qkv = F.gemm_unsummed(h, w.qkv, one)
+    qkv = F.gemm_unsummed(h, w.qkv, one) if w.qkv_bias is None else None
     if qkv is None:
         qkv = F.gemm(h, w.qkv, one)
+        if w.qkv_bias is not None:  # :310-313: added to the projection's bf16 result, in bf16
+            qkv = qkv + w.qkv_bias.to(qkv.dtype)
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     t = None
     if w.xsa_alpha is None and not _SEPARATE_QKV_POST:  # QK norm + RoPE + cache append inside the attention launch
@@ -494,6 +496,9 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         attn = attn_op(cfg.mode, cfg.implementation)
         t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
                  xsa_alpha=w.xsa_alpha).reshape(B, N * H)
+    if w.out_bias is not None:  # :366-373: projection, + bias, * residual scale, + residual, each a bf16 result
+        t = (F.gemm(t, w.out, one) + w.out_bias.to(t.dtype)) * cfg.residual_scale
+        return (x + t).to(x.dtype), cache
     out = F.gemm_unsummed(t, w.out, one)
     if out is None:
         return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache
@@ -515,9 +520,10 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None 
     scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
     if groups_out is not None:
         groups_out.append(groups)
+    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32).reshape(bias.shape[0], -1).contiguous()  # :527-528
     t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
-               swiglu_limit=cfg.swiglu_limit)
-    t = F.gemm(t, w.mlp_down, groups)
+               swiglu_limit=cfg.swiglu_limit, bias=bf(w.mlp_up_bias))
+    t = F.gemm(t, w.mlp_down, groups, bias=bf(w.mlp_down_bias))
     if topk <= 16 and not _SEPARATE_COMBINE:  # the combine step is left to the norm that follows (the next layer's, or the final one)
         return F.Uncombined(t, scores, dest, x, cfg.residual_scale)
     return F.moe_combine(t, scores, dest, x, cfg.residual_scale)
@@ -531,7 +537,11 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     else:
         t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     one = _one_group(x.shape[0], x.device)
-    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit)
+    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32).reshape(1, -1).contiguous()
+    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, bias=bf(w.mlp_up_bias))
+    if w.mlp_down_bias is not None:  # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result
+        t = (F.gemm(t, w.mlp_down, one) + w.mlp_down_bias[0].to(t.dtype)) * cfg.dense_residual_scale
+        return (x + t).to(x.dtype)
     down = F.gemm_unsummed(t, w.mlp_down, one)
     if down is None:
         return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)
@@ -540,16 +550,16 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
 
 
 def _fused_supported(model: ModelWeights, cfg: ModelConfig) -> bool:
-    """Shapes the fused launches cover (the matmul kernel's: K % 32, N % 128, N % 256 with SwiGLU)."""
+    """Shapes the fused launches cover (the matmul kernel's: K % 32, N % 8; the norm kernels': width % 4; the
+    attention's: head width 64 or 128).  Projections whose widths are whole 128-column spans also run split over K with
+    the sum left to their consumer; the others, and those followed by a bias, are summed by the matmul itself."""
     if not (cfg.fused_glue and cfg.implementation != "xla" and model.emb.is_cuda):
         return False
-    if cfg.use_qkv_bias or cfg.use_attn_out_bias or cfg.use_mlp_bias:  # the fused launches between the operators carry no biases
-        return False
     C, H = cfg.n_embd, cfg.head_dim
-    widths_ok = C % 128 == 0 and ((cfg.n_attn_heads + 2 * cfg.n_kv_heads) * H) % 128 == 0 and (cfg.n_attn_heads * H) % 32 == 0
+    widths_ok = C % 32 == 0 and (cfg.n_attn_heads * H) % 32 == 0
     hidden = [cfg.dense_hidden] + ([cfg.expert_hidden] if "moe" in cfg.mlp_map else [])
-    return (widths_ok and H in (64, 128) and all(h % 128 == 0 for h in hidden) and cfg.n_routed_experts <= 128
-            and cfg.n_active_routed_experts <= 8 and cfg.padded_vocab_size % 128 == 0)
+    return (widths_ok and H in (64, 128) and all(h % 32 == 0 for h in hidden) and cfg.n_routed_experts <= 128
+            and cfg.n_active_routed_experts <= 8 and cfg.padded_vocab_size % 8 == 0)
 
 
 def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, hidden_out: list | None = None,

@@ -42,12 +42,11 @@ def _case(seed, M, G, K, N, sizes, *, kind, block=(256, 256), bias=False, w_std=
     return c
 
 
-def _want(c, swiglu, big=False, general_kernel=False):
-    # Several groups with scale blocks shorter than K: the expert kernel dequantises like the reference, f32(code) * scale
-    # rounded to bf16 (lyra/nn/quant.py:82-85), so that is the operand the float32 product is taken on.  Everywhere else -
-    # and in the general kernel, which takes the widths that are not whole spans - the scales factor out of the product
-    # and are applied to the float32 sums.
-    like_reference = c["kind"] == "fp8" and len(c["sizes"]) > 1 and c["block"][0] < c["lhs"].shape[1] and not general_kernel
+def _want(c, swiglu, big=False):
+    # Several groups with scale blocks shorter than K: the kernel dequantises like the reference, f32(code) * scale rounded
+    # to bf16 (lyra/nn/quant.py:82-85), so that is the operand the float32 product is taken on.  Everywhere else the
+    # scales factor out of the product and are applied to the float32 sums.
+    like_reference = c["kind"] == "fp8" and len(c["sizes"]) > 1 and c["block"][0] < c["lhs"].shape[1]
     if big:  # the C restatement (same arithmetic, threaded) for shapes numpy would take minutes on
         if c["kind"] == "fp8":
             q, s = c["w"]
@@ -242,12 +241,12 @@ def test_quantize_on_the_fly_and_dispatch_contract():
     rhs = QArray(U.t_fp8(q), U.t_f32(s), (256, 256))
     out = decode_gemm(U.t_bf16(lhs), rhs, gs, implementation="pallas")
     U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, (q, s), sizes, block=(256, 256), mode="ref"), what="dequantised")
-    # unsupported N: "pallas" raises, "auto" takes the plain path
-    w2 = U.t_bf16(w[:, :, :200])
+    # unsupported N (not a multiple of 8): "pallas" raises, "auto" takes the plain path
+    w2 = U.t_bf16(w[:, :, :204])
     with pytest.raises(ValueError, match="no HIP kernel configuration"):
         decode_gemm(U.t_bf16(lhs), w2, gs, implementation="pallas")
     out = decode_gemm(U.t_bf16(lhs), w2, gs, implementation="auto")
-    U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, O.bf16_round(w[:, :, :200]), sizes), what="fallback")
+    U.assert_close(U.to_np(out), O.decode_gemm_reference(lhs, O.bf16_round(w[:, :, :204]), sizes), what="fallback")
     with pytest.raises(ValueError, match="Unsupported bias shape"):
         decode_gemm(U.t_bf16(lhs), U.t_bf16(w), gs, bias=torch.zeros(3, N, device=U.dev()))
 
@@ -407,9 +406,9 @@ def test_zero_and_extreme_block_scales(G, M):
     (16, 1, 8192, 8200, "fp8", (8192, 1), False, False),     # large enough for K slices across workgroups + the finish kernel
 ])
 def test_widths_that_are_not_whole_spans(M, G, K, N, kind, block, swiglu, bias):
-    """N % 8 == 0 (N % 16 == 0 with SwiGLU) is enough: widths that do not fill their last 128-column span take the general
-    kernel, whose lanes past the last column compute along and store nothing (the reference's kernel needs n % 128 == 0,
-    decode_gemm.py:88, and runs such shapes - all of gpt-oss-20b's, width 2880 - on its XLA path)."""
+    """N % 8 == 0 (N % 16 == 0 with SwiGLU) is enough: in the expert kernel and in the general kernel the lanes past the
+    last column of a partly filled 128-column span load nothing and store nothing (the reference's kernel needs
+    n % 128 == 0, decode_gemm.py:88, and runs such shapes - all of gpt-oss-20b's, width 2880 - on its XLA path)."""
     rng = np.random.default_rng(M + G + N)
     cuts = np.sort(rng.integers(0, M + 1, G - 1)) if G > 1 else np.zeros(0, np.int64)
     sizes = np.diff(np.concatenate([[0], cuts, [M]])).astype(np.int32)
@@ -417,7 +416,7 @@ def test_widths_that_are_not_whole_spans(M, G, K, N, kind, block, swiglu, bias):
         sizes[1] = 0  # an expert without rows
     _note(f"gemm ragged width M={M} G={G} K={K} N={N} {kind} block={block} swiglu={swiglu} bias={bias} sizes={sizes.tolist()}")
     c = _case(N, M, G, K, N, sizes, kind=kind, block=block, bias=bias, w_std=0.03)
-    want = _want(c, swiglu, big=True, general_kernel=N % (256 if swiglu else 128) != 0)
+    want = _want(c, swiglu, big=True)
     got = _run(c, swiglu)
     assert got.shape == want.shape == (M, N // 2 if swiglu else N)
     U.assert_close(got, want, what=f"ragged width N={N}")

@@ -352,3 +352,50 @@ def test_graphed_decoder_samples_inside_the_graph():
         assert (nxt.long()[:, None] == top4).any(-1).all()
         draws.append(U.to_np(nxt).copy())
     assert len({d.tobytes() for d in draws}) > 1
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_gpt_oss_like_variant_width_not_a_multiple_of_128_with_biases(fp8):
+    """The options of gpt-oss-20b (lyra/variants.py:62-80: biases on q/k/v, the output projection and the MLPs, no shared
+    expert, no QK norm, YaRN tables) at a width that is not a multiple of 128 (320; gpt-oss-20b's is 2880): the fused driver
+    takes such a model too - its matmuls through the general kernel, the biases the reference adds to a bf16 result added
+    the same way - and must match the oracle step by step, match the plain-operator driver, and replay from a HIP graph."""
+    from lyra_amd.generate import GraphedDecoder
+    from lyra_amd.model import MODEL_VARIANTS, _fused_supported, apply_inference_overrides, init_cache, init_weights, model_apply
+
+    cfg = replace(MODEL_VARIANTS["dev"], implementation="pallas", n_embd=320, n_attn_heads=4, n_kv_heads=2, seq_len=128,
+                  sliding_window=32, use_qk_norm=False, use_qkv_bias=True, use_attn_out_bias=True, use_mlp_bias=True,
+                  n_shared_experts=0, n_active_experts=2, rope_scale=4.0, mlp_map=("moe", "dense", "moe", "moe"),
+                  sample_temperature=0.0)
+    if fp8:
+        cfg = apply_inference_overrides(cfg, fp8=True, fp8_attn=True, per_channel=True)
+    dev = U.dev()
+    assert _fused_supported(init_weights(cfg, dev, seed=3), cfg)
+    _run_steps(cfg, B=5, S=128, steps=3, start=40)
+
+    # fused driver against the plain-operator driver on the same weights and history (both on the HIP operators)
+    w = init_weights(cfg, dev, seed=3)
+    tok = torch.tensor([3, 900, 17, 5, 4], device=dev)
+    outs = []
+    for fused in (True, False):
+        c = replace(cfg, fused_glue=fused)
+        cache = init_cache(c, 5, 128, dev)
+        cache.pos.fill_(0)
+        steps, t = [], tok
+        for _ in range(3):
+            logits, _ = model_apply(t, w, cache, c)
+            steps.append(U.to_np(logits[:, : cfg.vocab_size]))
+            t = logits.argmax(-1)
+        outs.append(steps)
+    for a, b in zip(*outs):
+        U.assert_close(a, b, atol=3e-2, rtol=2e-2, what="fused vs plain-operator logits")
+
+    # ... and the captured step chains tokens like the eager one
+    cache = init_cache(cfg, 5, 128, dev)
+    cache.pos.fill_(0)
+    dec = GraphedDecoder(w, cache, cfg, batch=5)
+    dec.tokens.copy_(tok.to(torch.int32))
+    got = dec.decode(3)
+    torch.cuda.synchronize()
+    assert got.shape == (3, 5) and int(cache.pos.item()) == 3
+    assert torch.equal(got[0].cpu(), torch.from_numpy(outs[0][0].argmax(-1)).to(torch.int32))

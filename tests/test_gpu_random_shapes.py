@@ -236,5 +236,4 @@ def test_decode_gemm_at_drawn_widths_that_are_not_whole_spans(seed):
     bias = bool(rng.integers(0, 2))
     _note(f"gemm width draw {seed}: M={M} G={G} K={K} N={N} sizes={sizes.tolist()} {kind} block={block} bias={bias} swiglu={swiglu}")
     c = gemm_case(seed, M, G, K, N, sizes.tolist(), kind=kind, block=block, bias=bias, w_std=0.05)
-    want = gemm_want(c, swiglu, general_kernel=N % (256 if swiglu else 128) != 0)
-    U.assert_close(run_gemm(c, swiglu), want, what=f"width draw {seed}")
+    U.assert_close(run_gemm(c, swiglu), gemm_want(c, swiglu), what=f"width draw {seed}")
