@@ -399,3 +399,17 @@ def test_gpt_oss_like_variant_width_not_a_multiple_of_128_with_biases(fp8):
     torch.cuda.synchronize()
     assert got.shape == (3, 5) and int(cache.pos.item()) == 3
     assert torch.equal(got[0].cpu(), torch.from_numpy(outs[0][0].argmax(-1)).to(torch.int32))
+
+
+def test_width_2880_step_of_gpt_oss_20b_with_biases_32_experts_b64():
+    """The widths and options of gpt-oss-20b (lyra/variants.py:62-80: C=2880, 64Q/8KV heads of 64, 32 routed experts of
+    hidden 2880 and no shared one, 4 per token, biases on every projection, no QK norm, YaRN tables) at B=64 on two layers
+    with a small vocabulary: every projection width but q/k/v's is 22.5 spans of 128 columns.  The fused driver against the
+    CPU restatement, layer by layer and end to end."""
+    from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides
+
+    cfg = replace(MODEL_VARIANTS["gpt-oss-20b"], implementation="pallas", n_layers=2, mlp_map=("moe", "moe"), vocab_size=4000,
+                  padded_vocab_size=4096, seq_len=1024)
+    assert cfg.n_embd == 2880 and cfg.expert_hidden == 2880 and cfg.use_qkv_bias and cfg.use_mlp_bias and cfg.n_shared_experts == 0
+    cfg = apply_inference_overrides(cfg, fp8=True, fp8_attn=True, per_channel=True)
+    _full_width_parity(cfg, B=64, S=1024, start=700, steps=2, min_clear=40, moe_layers=2, hidden_tol=0.03)
