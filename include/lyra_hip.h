@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 10
+#define LYRA_ABI_VERSION 11
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -179,9 +179,13 @@ size_t lyra_decode_gemm_workspace_for(int M, int G, int K, int N, int bk, int fu
  *   lhs_row_map [M] int32 or NULL: sorted row r reads lhs[lhs_row_map[r], :] - the token gather that feeds the
  *               expert up-projection (x[permute_map // topk], model.py:536-540); lhs then has as many rows as
  *               the map addresses.
- *   post_scale  != 0: out = bf16(residual + bf16(bf16(t) * out_scale)), t the plain result - a projection's
+ *   post_scale  bit 0: out = bf16(residual + bf16(bf16(t) * out_scale)), t the plain result - a projection's
  *               output scaled in bf16 and added to the residual stream; residual [M,N] bf16 or NULL (scale only).
- *               residual requires post_scale and a bf16 output.
+ *               residual requires bit 0 and a bf16 output.
+ *               bit 1 (one group, no fused_swiglu, bf16 output, bias given): the bias is added after the cast,
+ *               t = bf16(bf16(product) + bias), as the model does for the q/k/v, output and dense down
+ *               projections (model.py:310-313, 367-368, 629-630: a bf16 bias added to the operator's bf16
+ *               result); without it the bias is added to the float32 product (gemm.py:1600-1605).
  */
 int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
                         int bn, const int32_t* group_sizes, const float* bias, const void* residual, float out_scale,

@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 10
+ABI_VERSION = 11
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 
 _c = ctypes

@@ -40,6 +40,7 @@ struct GemmParams {
     int ksplit, kpart;  // kpart: rows of K per split, multiple of 32 (and of bk when bk < K)
     int row_par;        // row blocks of a group that run as separate workgroups (grid.z = G * row_par)
     int wide;           // grouped kernel without SwiGLU: units of 256 columns (two wavefront pairs)
+    int bias_post;      // one group, no SwiGLU: the bias is added to the bf16-rounded product, in bf16 (then scale / residual)
     int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
     int snake;          // grouped kernel: odd rounds of units run over the workgroups in the opposite direction (-1: if >= 4 rounds)
     int even_spans;     // plain kernel: spans dealt out evenly over one workgroup per compute unit
@@ -193,7 +194,7 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
     if (p.bias) {
         const float* bp = p.bias + (size_t)g * p.N + ncol;
 #pragma unroll
-        for (int c = 0; c < 8; ++c) t[c] += bp[c];
+        for (int c = 0; c < 8; ++c) t[c] = p.bias_post ? round_bf16(round_bf16(t[c]) + bp[c]) : t[c] + bp[c];
     }
     int NO = p.N;
     if (p.swiglu) {
@@ -438,7 +439,8 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
     if (p.bias) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            a[c] += p.bias[(size_t)g * p.N + col + c];
+            const float bv = p.bias[(size_t)g * p.N + col + c];
+            a[c] = p.bias_post ? round_bf16(round_bf16(a[c]) + bv) : a[c] + bv;
             if (p.swiglu) b[c] += p.bias[(size_t)g * p.N + NO + col + c];
         }
     }
@@ -639,7 +641,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(Gem
     }
     if (!e_ok) return;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] += ebias[c];
+    for (int c = 0; c < 4; ++c) v[c] = p.bias_post ? round_bf16(round_bf16(v[c]) + ebias[c]) : v[c] + ebias[c];
     if (p.swiglu) {
         float o[2] = {swiglu_one(v[0], v[2], p.beta, p.limit), swiglu_one(v[1], v[3], p.beta, p.limit)};
         if (p.post_scale) {
@@ -1625,7 +1627,11 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
                                    int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
                                    lyra_stream_t stream) {
     using namespace lyra;
+    const bool bias_post = (post_scale & 2) != 0;  // post_scale: bit 0 the scale / residual epilogue, bit 1 the bias after the cast
+    post_scale &= 1;
     if (residual && (!post_scale || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
+    if (bias_post && (!bias || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
+    if (bias_post && (G != 1 || fused_swiglu)) return LYRA_E_UNSUPPORTED;
     if (!lhs || !rhs || !group_sizes || !out) return LYRA_E_BADARG;
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
     if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
@@ -1684,6 +1690,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
     p.post_scale = post_scale != 0;
+    p.bias_post = bias_post ? 1 : 0;
     p.arrivals = nullptr;
     if (pl.ksplit > 1 || pl.split_k || pl.grouped) {
         // the first kGemmCounterBytes belong to the grouped kernel's arrival counters, whichever kernel runs

@@ -249,9 +249,12 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
 def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,
          residual: torch.Tensor | None = None, out_scale: float | None = None, fused_swiglu: bool = False,
          swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False,
-         bias: torch.Tensor | None = None) -> torch.Tensor:
+         bias: torch.Tensor | None = None, bias_after_cast: bool = False) -> torch.Tensor:
     """lyra_decode_gemm_ex: the decode grouped matmul with an optional row gather on the input and an optional
-    ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray."""
+    ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray.
+    ``bias`` [G, N] float32 is added to the float32 product (lyra/kernels/gemm.py:1600-1605), or with ``bias_after_cast``
+    (one group, no SwiGLU) to the product rounded to bf16, in bf16, as a caller does that adds a bias to the operator's
+    result (lyra/model.py:310-313, 367-368)."""
     dev = lhs.device
     G, K, N = rhs.shape
     M = rows if rows is not None else lhs.shape[0]
@@ -277,7 +280,8 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     need = _L.lyra_decode_gemm_workspace(M, G, K, N, int(fused_swiglu))
     ws = _lib.workspace("gemm", dev, stream, need)
     rc = _L.lyra_decode_gemm_ex(lhs.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
-                                _ptr(residual), 1.0 if out_scale is None else float(out_scale), int(out_scale is not None),
+                                _ptr(residual), 1.0 if out_scale is None else float(out_scale),
+                                int(out_scale is not None) | (2 if bias_after_cast else 0),
                                 out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
                                 _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
                                 float(swiglu_limit), stream)

@@ -462,6 +462,19 @@ class TokenRows:
     tokens: torch.Tensor  # [B] int32
 
 
+def _bf16_bias(bias, groups: int = 1):
+    """A bias as the matmul epilogue takes it: [groups, N] float32 holding the values rounded to bf16 (None stays None;
+    lyra/model.py:527-528 casts the biases to the compute dtype).  Converted once and kept on the bias tensor itself, so
+    that a decode step does not spend launches on its own weights (an in-place change of the bias converts it again)."""
+    if bias is None:
+        return None
+    kept = getattr(bias, "_lyra_bf16_as_f32", None)
+    if kept is None or kept[0] != (bias._version, groups):
+        kept = ((bias._version, groups), bias.to(torch.bfloat16).to(torch.float32).reshape(groups, -1).contiguous())
+        bias._lyra_bf16_as_f32 = kept
+    return kept[1]
+
+
 def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, cache: LayerCache, cfg: ModelConfig):
     """attention_apply as 4 launches: norm(+gate) | qkv matmul | QK norm + RoPE + cache append + attention | output matmul.
     ``x`` is the residual stream or an ``Unsummed`` projection that still has to be added to it; the return value likewise
@@ -479,9 +492,8 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     one = _one_group(B, x.device)
     qkv = F.gemm_unsummed(h, w.qkv, one) if w.qkv_bias is None else None
     if qkv is None:
-        qkv = F.gemm(h, w.qkv, one)
-        if w.qkv_bias is not None:  # :310-313: added to the projection's bf16 result, in bf16
-            qkv = qkv + w.qkv_bias.to(qkv.dtype)
+        # (:310-313: a bias is added to the projection's bf16 result, in bf16 - inside the matmul's epilogue)
+        qkv = F.gemm(h, w.qkv, one, bias=_bf16_bias(w.qkv_bias), bias_after_cast=w.qkv_bias is not None)
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     t = None
     if w.xsa_alpha is None and not _SEPARATE_QKV_POST:  # QK norm + RoPE + cache append inside the attention launch
@@ -497,8 +509,7 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
                  xsa_alpha=w.xsa_alpha).reshape(B, N * H)
     if w.out_bias is not None:  # :366-373: projection, + bias, * residual scale, + residual, each a bf16 result
-        t = (F.gemm(t, w.out, one) + w.out_bias.to(t.dtype)) * cfg.residual_scale
-        return (x + t).to(x.dtype), cache
+        return F.gemm(t, w.out, one, bias=_bf16_bias(w.out_bias), bias_after_cast=True, residual=x, out_scale=cfg.residual_scale), cache
     out = F.gemm_unsummed(t, w.out, one)
     if out is None:
         return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache
@@ -520,10 +531,10 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None 
     scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
     if groups_out is not None:
         groups_out.append(groups)
-    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32).reshape(bias.shape[0], -1).contiguous()  # :527-528
+    G = cfg.n_experts
     t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
-               swiglu_limit=cfg.swiglu_limit, bias=bf(w.mlp_up_bias))
-    t = F.gemm(t, w.mlp_down, groups, bias=bf(w.mlp_down_bias))
+               swiglu_limit=cfg.swiglu_limit, bias=_bf16_bias(w.mlp_up_bias, G))
+    t = F.gemm(t, w.mlp_down, groups, bias=_bf16_bias(w.mlp_down_bias, G))
     if topk <= 16 and not _SEPARATE_COMBINE:  # the combine step is left to the norm that follows (the next layer's, or the final one)
         return F.Uncombined(t, scores, dest, x, cfg.residual_scale)
     return F.moe_combine(t, scores, dest, x, cfg.residual_scale)
@@ -537,11 +548,11 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     else:
         t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     one = _one_group(x.shape[0], x.device)
-    bf = lambda bias: None if bias is None else bias.to(x.dtype).to(torch.float32).reshape(1, -1).contiguous()
-    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, bias=bf(w.mlp_up_bias))
+    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
+               bias=_bf16_bias(w.mlp_up_bias))
     if w.mlp_down_bias is not None:  # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result
-        t = (F.gemm(t, w.mlp_down, one) + w.mlp_down_bias[0].to(t.dtype)) * cfg.dense_residual_scale
-        return (x + t).to(x.dtype)
+        return F.gemm(t, w.mlp_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=True, residual=x,
+                      out_scale=cfg.dense_residual_scale)
     down = F.gemm_unsummed(t, w.mlp_down, one)
     if down is None:
         return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)

@@ -521,3 +521,39 @@ def test_attention_with_the_front_step_equals_the_two_launches(B, N, K, S, H, fp
     # a second call on the same caches (the row is appended again, identically) must give the same result
     got2 = F.attention_qkv(qkv_a, qn, kn, cos_t, sin_t, pos, ka, va, sinks, H**-0.5, sw, N, K, H, 1e-5, gate=gate)
     assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("M,K,N", [(64, 2048, 2048),    # K-split kernel + finish kernel
+                                    (64, 2880, 5120),    # one-pass kernel (K not a multiple of 128)
+                                    (64, 4096, 2880),    # general kernel (a width that is not whole spans)
+                                    (5, 8192, 8200),     # general kernel, K split across workgroups + finish kernel
+                                    (130, 512, 136)])
+def test_gemm_bias_after_the_cast(fp8, M, K, N):
+    """bias_after_cast: bf16(bf16(x @ w) + bias), then the scale / residual epilogue - bit for bit what the plain matmul
+    followed by the bf16 torch ops of lyra/model.py:366-373 gives."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import quantize
+
+    _say(f"gemm bias after cast fp8={fp8} M{M} K{K} N{N}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(M + N)
+    x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(1, K, N, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    if fp8:
+        w = quantize(w, torch.float8_e4m3fn, (K, 1))
+    one = torch.full((1,), M, dtype=torch.int32, device=dev)
+    bias = torch.randn(N, generator=g, device=dev).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g, device=dev).to(torch.bfloat16)
+    b32 = bias.to(torch.float32).reshape(1, N).contiguous()
+    plain = F.gemm(x, w, one)
+    got = F.gemm(x, w, one, bias=b32, bias_after_cast=True)
+    assert torch.equal(got, plain + bias)
+    scale = 0.1767766952966369
+    got = F.gemm(x, w, one, bias=b32, bias_after_cast=True, residual=res, out_scale=scale)
+    assert torch.equal(got, res + (plain + bias) * scale)
+    # and the float32 bias of the operator itself is something else: added before the cast
+    pre = F.gemm(x, w, one, bias=b32)
+    assert not torch.equal(pre, plain + bias)
+    U.assert_close(U.to_np(pre), U.to_np(plain).astype(np.float32) + U.to_np(bias), atol=2e-2, rtol=1e-2, what="bias in float32")
