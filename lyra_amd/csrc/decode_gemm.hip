@@ -691,7 +691,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
     const int span = blockIdx.x, ks = blockIdx.y, row0 = blockIdx.z * p.row_block;
-    const int ncol = span * 128 + 8 * x;
+    const bool cols = span * 128 + 8 * x < p.N;    // (N need not fill the last span: lanes past it load nothing, store nothing)
+    const int ncol = cols ? span * 128 + 8 * x : 0;
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
     const int steps = (k1 - k0) >> 5;
     // steps wave, wave + 4, ... of the slice (<= DEPTH), or steps wave * DEPTH ... when scales change along K
@@ -701,7 +702,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int row_bytes = p.N * ES;
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-    const int wvoff = 8 * kb * row_bytes + ncol * ES;
+    const int wvoff = cols ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
     int avoff[MT];
 #pragma unroll
@@ -844,7 +845,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
             const f32x4 t = *(const f32x4*)(sm_part + wv * (64 * kSplitPitch) + r * kSplitPitch + 4 * q);
             v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
         }
-        store_through(p.part, (((size_t)ks * p.M + row) * p.N + span * 128 + 4 * q) * 4, v);
+        if (span * 128 + 4 * q < p.N) store_through(p.part, (((size_t)ks * p.M + row) * p.N + span * 128 + 4 * q) * 4, v);
     }
 }
 
@@ -1474,7 +1475,9 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
         pl.split_k = false;
         return pl;
     }
-    pl.split_k = allow_split_k && G == 1 && weight_bytes <= 160e6 && M <= 256 && K % 128 == 0 && whole_spans && !no_split_k;
+    // (a K that is not a multiple of 128 leaves the last slice's wavefronts unequal shares, which is fine; scale blocks
+    // along K are only lined up with the slices for K % 128 == 0)
+    pl.split_k = allow_split_k && G == 1 && weight_bytes <= 160e6 && M <= 256 && (K % 128 == 0 || bk <= 0 || bk >= K) && !no_split_k;
     if (pl.split_k) {
         // ~256 workgroups; a slice is a multiple of 128 rows (4 wavefronts x 32) and of the scale block, at most 512 rows
         pl.mt = 4;
