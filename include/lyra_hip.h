@@ -157,8 +157,7 @@ int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t s
  *               (lyra_workspace_init); every call leaves the counters at zero.  Float32 partial products follow.
  * Supported: K % 32 == 0, N % 8 == 0 (N % 16 == 0 with fused_swiglu), G <= 8191; fp8 blocks with bn a
  * power of two, and either (bn % 8 == 0 and (bk % 32 == 0 or bk == K)) or bk == K.  N need not fill its last
- * 128-column span (the reference's kernel wants n % 128 == 0, decode_gemm.py:88, and otherwise takes its XLA path);
- * with one group such a width takes the general kernel instead of the K-split one.
+ * 128-column span (the reference's kernel wants n % 128 == 0, decode_gemm.py:88, and otherwise takes its XLA path).
  */
 int lyra_decode_gemm(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
                      const int32_t* group_sizes, const float* bias, void* out, void* workspace,
