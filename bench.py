@@ -253,6 +253,7 @@ def benchmark_routing():
     r["small_B8"] = zipf_group_sizes(rng, 8, 15, 3, 1)
     r["small_B64"] = zipf_group_sizes(rng, 64, 15, 3, 1)
     r["probe"] = zipf_group_sizes(rng, 64, 15, 3, 1)
+    r["gptoss_B64"] = zipf_group_sizes(rng, 64, 32, 4, 0)  # gpt-oss-20b: 4 of 32 routed experts per token, no shared expert
     return r
 
 
@@ -407,6 +408,12 @@ def kernel_table(dev, only=""):
                            ("dense down", 3072, 2048, False)):
         gemm(f"lyra-small {name} projection B=64 ({K}x{N} fp8)", 64, 1, K, N, [64], sw, (K, 1))
     gemm("lyra-medium dense up+SwiGLU B=64 (4096x12288 fp8)", 64, 1, 4096, 12288, [64], True, (4096, 1))
+    # gpt-oss-20b: width 2880 = 22.5 spans of 128 columns
+    s = routing["gptoss_B64"]
+    gemm("gpt-oss-20b expert up+SwiGLU B=64 (32x2880x5760 fp8)", int(s.sum()), 32, 2880, 5760, s, True, (2880, 1))
+    gemm("gpt-oss-20b expert down B=64 (32x2880x2880 fp8)", int(s.sum()), 32, 2880, 2880, s, False, (2880, 1))
+    gemm("gpt-oss-20b q/k/v projection B=64 (2880x5120 fp8)", 64, 1, 2880, 5120, [64], False, (2880, 1))
+    gemm("gpt-oss-20b out projection B=64 (4096x2880 fp8)", 64, 1, 4096, 2880, [64], False, (4096, 1))
     gemm("lyra-small LM head B=64 (2048x204800 bf16, f32 logits)", 64, 1, 2048, 204800, [64], False, None, fp8=False, out_f32=True)
     for r in rows:
         r["cold_GBs"] = r["bytes"] / r["cold_us"] / 1e3

@@ -181,7 +181,7 @@ __device__ __forceinline__ void convert_colpair(const RawW<FP8>& t, int cp, Pack
 // Writes 8 consecutive result columns of one row: fused epilogue (ksplit == 1) or float32 partials.
 // Must be called by all lanes of the wavefront (SwiGLU exchanges gate and linear halves by shuffle);
 // `store` says whether this lane's row exists.
-__device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], int g, int row, int ncol, int out_col,
+__device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], const float (&bias8)[8], int row, int ncol, int out_col,
                                            int ks, bool store, bool is_lin_lane) {
     if (p.ksplit > 1) {
         if (store) {
@@ -191,10 +191,12 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], i
         }
         return;
     }
-    if (p.bias) {
-        const float* bp = p.bias + (size_t)g * p.N + ncol;
+    if (p.bias_post) {  // (the lane's 8 bias values were loaded once, by the caller)
 #pragma unroll
-        for (int c = 0; c < 8; ++c) t[c] = p.bias_post ? round_bf16(round_bf16(t[c]) + bp[c]) : t[c] + bp[c];
+        for (int c = 0; c < 8; ++c) t[c] = round_bf16(round_bf16(t[c]) + bias8[c]);
+    } else if (p.bias) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) t[c] += bias8[c];
     }
     int NO = p.N;
     if (p.swiglu) {
@@ -362,7 +364,9 @@ void decode_gemm_kernel(GemmParams p) {
             }
         }
 
-        float colscale[8];
+        float colscale[8], bias8[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) bias8[c] = (p.bias && p.ksplit == 1) ? p.bias[(size_t)g * p.N + ncol + c] : 0.f;
 #pragma unroll
         for (int c = 0; c < 8; ++c) colscale[c] = s_cur;
         if (FP8 && p.scale_mode == 2) {
@@ -378,18 +382,21 @@ void decode_gemm_kernel(GemmParams p) {
                     float t[8];
 #pragma unroll
                     for (int c = 0; c < 8; ++c) t[c] = acc[mt][c][r] * colscale[c];
-                    finish_row(p, t, g, rowbase + lr, ncol, out_col, ks, span_ok && lr < rows_here, is_lin_lane);
+                    finish_row(p, t, bias8, rowbase + lr, ncol, out_col, ks, span_ok && lr < rows_here, is_lin_lane);
                 }
             }
         }
     }
 
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
+    float pad_bias8[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) pad_bias8[c] = (p.bias && p.ksplit == 1 && pad_from < p.M) ? p.bias[(size_t)g * p.N + ncol + c] : 0.f;
     for (int row0 = pad_from; row0 < p.M; row0 += 4) {
         float t[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) t[c] = 0.f;
-        finish_row(p, t, g, row0 + kb, ncol, out_col, ks, span_ok && row0 + kb < p.M, is_lin_lane);
+        finish_row(p, t, pad_bias8, row0 + kb, ncol, out_col, ks, span_ok && row0 + kb < p.M, is_lin_lane);
     }
 }
 
