@@ -230,7 +230,9 @@ int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, cons
  * computes): x_out = bf16(residual + bf16(bf16(sum_k scores[b,k] * rows[dest[b*topk+k]]) * out_scale)), rows [B*topk, C]
  * bf16 in sorted order, scores [B, topk] float32, dest [B*topk] int32, topk <= 16.  Same aliasing rule. */
 /* Same for the first layer of a step: row b is the embedding row table[tokens[b]] (the gather of lyra/model.py:752; table
- * [table_rows, C] bf16, tokens [B] int32 in [0, table_rows)), also copied to x_out [B,C] as the residual stream. */
+ * [table_rows, C] bf16, tokens [B] int32), also copied to x_out [B,C] as the residual stream.  A token id outside
+ * [0, table_rows) is clamped into the range (jnp.take's "clip" mode; the reference's default mode fills such rows with NaN,
+ * lyra/model.py:747): the kernel never reads outside the table. */
 int lyra_rmsnorm_proj_embed(const void* table, const int32_t* tokens, int table_rows, void* x_out, const float* scale, void* h,
                             const float* proj_t, const float* bias, void* y, int B, int C, int n, int mode, float eps,
                             lyra_stream_t stream);

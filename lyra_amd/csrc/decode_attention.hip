@@ -629,7 +629,12 @@ void decode_attention_kernel(AttnParams p) {
             rope_sn = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(make_rsrc(p.sin_t, rope_bytes), roff, 0, 0));
         }
         for (int t = wave; t < G; t += WAVES) {
-            if (t != wave) request_head<H>(p, part_rsrc, qkv_rsrc, b, kh * G + t, true, lane, hq);  // (more than WAVES query heads per kv head)
+            if (t != wave) {  // (more than WAVES query heads per kv head)
+                // both requests, in this order: the first one clears the slots the second one fills (which it leaves
+                // at zero, without memory traffic, when the projection has no more than kFirstSlices slices)
+                request_head<H>(p, part_rsrc, qkv_rsrc, b, kh * G + t, true, lane, hq);
+                request_head<H, kFirstSlices>(p, part_rsrc, qkv_rsrc, b, kh * G + t, true, lane, hq);
+            }
             float a, c;
             sum_head<H>(p, part_rsrc, b, kh * G + t, lane, hq, a, c);
             head_norm_rope(a, c, p.qnorm != nullptr, qn_a, qn_c, rope_cs, rope_sn, p.norm_eps, H);

@@ -50,6 +50,8 @@ struct NormProjParams {
     int comb_topk;              // <= 16
     // or: row b is row row_index[b] of x (the embedding table: the token gather of lyra/model.py:752), copied to x_out
     const int32_t* row_index;   // [B] or null
+    int row_limit;              // rows of x when row_index is set: an index outside [0, row_limit) is clamped into it, so a
+                                // bad token id (padding such as -1, a stale buffer) reads a valid row instead of faulting
 };
 
 constexpr int kNormThreads = 1024;
@@ -75,7 +77,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
 #pragma unroll
         for (int i = 0; i < 8; ++i) w_first[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (i * 256 + (int)(threadIdx.x & 63) * 4) * 4, 0, 0);
     }
-    const uint16_t* xr = p.x + (size_t)(p.row_index ? p.row_index[b] : b) * p.C;
+    const uint16_t* xr = p.x + (size_t)(p.row_index ? min(max(p.row_index[b], 0), p.row_limit - 1) : b) * p.C;
     // (the norm weights of this thread's first 4 columns, likewise requested ahead of the row)
     const int c_first = min((int)threadIdx.x * 4, p.C - 4);
     const f32x4 sc_first = *(const f32x4*)(p.scale + c_first);
@@ -748,7 +750,7 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
-                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr};
+                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr, 0};
     return launch_rmsnorm_proj(p, B, stream);
 }
 
@@ -761,7 +763,7 @@ extern "C" int lyra_rmsnorm_proj_embed(const void* table, const int32_t* tokens,
     if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)table, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
-                     nullptr, 0, B, nullptr, 1.0f, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, tokens};
+                     nullptr, 0, B, nullptr, 1.0f, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, tokens, table_rows};
     return launch_rmsnorm_proj(p, B, stream);
 }
 
@@ -775,7 +777,7 @@ extern "C" int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, 
     if (C % 4 || C > 32768 || topk > 16) return LYRA_E_UNSUPPORTED;
     NormProjParams p{nullptr, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      nullptr, 0, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out,
-                     (const uint16_t*)rows, scores, dest, topk, nullptr};
+                     (const uint16_t*)rows, scores, dest, topk, nullptr, 0};
     return launch_rmsnorm_proj(p, B, stream);
 }
 

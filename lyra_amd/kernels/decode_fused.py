@@ -200,13 +200,16 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
 
 
 def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v, sinks,
-                  sm_scale: float, sliding_window: int, n_heads: int, n_kv_heads: int, head_dim: int, eps: float, gate=None):
+                  sm_scale: float, sliding_window: int, n_heads: int, n_kv_heads: int, head_dim: int, eps: float, gate=None,
+                  out_dtype: torch.dtype = torch.bfloat16):
     """``qkv_post`` and the decode attention in one launch (lyra/model.py:309-347): the attention kernel's workgroups sum
     the projection's slices, apply QK norm and the rotary embedding, append the new key and value rows to the caches (in
     place) and attend.  Results and cache contents are bit-identical to the two launches.  Returns [B, N*H] bf16, or None
     when the launch does not exist for this shape (a ragged batch of more than 256 (row, kv head) pairs, which the
-    whole-row kernel takes): the caller then runs the two launches."""
+    whole-row kernel takes): the caller then runs the two launches.  ``out_dtype``: bfloat16 (what the decode step
+    uses) or float32 (the attention's ``dtype`` argument, lyra/kernels/decode_attention.py:373)."""
     N, K, H = n_heads, n_kv_heads, head_dim
+    assert out_dtype in (torch.bfloat16, torch.float32)
     unsummed = isinstance(qkv, Unsummed)
     if unsummed:
         part = qkv.partials
@@ -230,7 +233,7 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
     assert sinks.dtype == torch.float32 and sinks.numel() == N and sinks.is_contiguous()
     if gate is not None:
         assert gate.dtype == torch.bfloat16 and gate.is_contiguous() and gate.numel() == B * N
-    out = torch.empty((B, N * H), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((B, N * H), dtype=out_dtype, device=dev)
     stream = _stream(dev)
     need = _L.lyra_decode_attention_workspace(B, N, K, S, H, int(sliding_window))
     ws = _lib.workspace("attention", dev, stream, need)
@@ -239,7 +242,8 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
                                       _f32(sin_t).data_ptr(), cos_t.shape[0], float(eps), kq.data_ptr(), vq.data_ptr(), _ptr(ks),
                                       _ptr(vs), sinks.data_ptr(), pos.data_ptr(), 0 if pos.numel() == 1 else 1, _ptr(gate),
                                       out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, float(sm_scale),
-                                      int(sliding_window), _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_BF16, stream)
+                                      int(sliding_window), _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16,
+                                      _lib.DTYPE_F32 if out_dtype == torch.float32 else _lib.DTYPE_BF16, stream)
     if rc == _lib.E_UNSUPPORTED:
         return None
     _lib.check(rc, "lyra_decode_attention_qkv")

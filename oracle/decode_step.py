@@ -134,8 +134,15 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
             t = R(t * np.float32(cfg.residual_scale))
             h = R(h + t)
         else:
-            t = _gemm(xn, m["mlp_up"], one, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
-                      bias=_bias(m.get("mlp_up_bias")), inner=inner)
+            if ref and m.get("mlp_up_bias") is not None:
+                # model.py:613-616: the product is a bf16 array, the bias is added to it in bf16, SwiGLU follows
+                # (inner="fp32", like the kernels, adds the bias to the float32 product inside the fused epilogue)
+                t = _gemm(xn, m["mlp_up"], one, use_c=use_c, inner=inner)
+                t = R(t + _bias(m["mlp_up_bias"])[0])
+                t = R(O.swiglu(t, cfg.swiglu_beta, cfg.swiglu_limit))
+            else:
+                t = _gemm(xn, m["mlp_up"], one, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
+                          bias=_bias(m.get("mlp_up_bias")), inner=inner)
             t = _gemm(R(t), m["mlp_down"], one, use_c=use_c, inner=inner)
             if m.get("mlp_down_bias") is not None:  # model.py:629-630
                 t = R(t + _bias(m["mlp_down_bias"])[0])

@@ -62,6 +62,31 @@ def test_rmsnorm_proj(B, C, n, mode):
         assert y is None
 
 
+@pytest.mark.parametrize("B,V,C,n", [(64, 1000, 2048, 16), (7, 33, 256, 0), (5, 204800, 2048, 16)])
+def test_embedding_gather_inside_the_first_norm(B, V, C, n):
+    """lyra_rmsnorm_proj_embed: rows table[tokens] (lyra/model.py:747) normalised like lyra_rmsnorm_proj's, bit for bit;
+    token ids outside [0, V) are clamped into the table (the rule stated in the header) instead of being read."""
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"embed B{B} V{V} C{C} n{n}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(V + B)
+    table = torch.randn(V, C, generator=g, device=dev).to(torch.bfloat16)
+    scale = 1 + 0.1 * torch.randn(C, generator=g, device=dev)
+    proj = torch.randn(C, n, generator=g, device=dev) / C**0.5 if n else None
+    ids = torch.randint(0, V, (B,), generator=g, device=dev, dtype=torch.int32)
+    ids[0], ids[-1] = 0, V - 1
+    bad = ids.clone()
+    bad[1], bad[2], bad[3] = -1, V, 2**31 - 1  # padding, one past the end, garbage
+    for tokens in (ids, bad):
+        h, y, x = F.embed_rmsnorm_proj(table, tokens, scale, 1e-5, proj, None, gate=True)
+        rows = table[tokens.long().clamp(0, V - 1)]
+        h2, y2 = F.rmsnorm_proj(rows, scale, 1e-5, proj, None, gate=True)
+        assert torch.equal(x, rows) and torch.equal(h, h2)
+        assert (y is None and y2 is None) or torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("B,N,K,S,H,fp8,qknorm,per_row", [
     (64, 16, 4, 512, 128, True, True, False),
     (3, 2, 1, 256, 64, True, True, True),
@@ -454,10 +479,19 @@ def test_sample_token_draws_from_the_topk_softmax():
     (64, 32, 8, 4096, 128, True, True, 0, True, "full"),        # lyra-medium: 512 pairs, two workgroups per compute unit
     (64, 64, 8, 4096, 64, True, False, 0, False, "full"),       # gpt-oss shape: 8 query heads per kv head, head width 64
     (64, 64, 8, 4096, 64, True, False, 128, False, "full"),
+    # more query heads per kv head than wavefronts AND more slices than one request holds: every head needs both requests
+    (4, 16, 2, 300, 64, True, True, 0, 5, "short"),
+    (3, 32, 2, 515, 128, True, True, 0, 8, "ragged"),
+    (2, 16, 1, 200, 128, False, True, 33, 12, "ragged"),
+    (6, 24, 3, 400, 64, True, False, 128, 8, "edges"),
+    (5, 32, 2, 1000, 64, False, False, 0, 12, "ragged"),
+    (9, 8, 1, 260, 128, True, True, 0, 5, "short"),
+    (8, 16, 4, 4096, 128, True, True, 0, 8, "ragged"),          # lyra-small at a small batch: the planner's 8 slices
 ])
 def test_attention_with_the_front_step_equals_the_two_launches(B, N, K, S, H, fp8, qknorm, sw, unsummed, positions):
     """lyra_decode_attention_qkv against lyra_qkv_post(_sum) followed by lyra_decode_attention on copies of the same
-    caches: outputs and every byte of the caches must be identical."""
+    caches: outputs and every byte of the caches must be identical.  `unsummed`: False = the summed bf16 projection,
+    True = 3 float32 slices, a number = that many slices."""
     from lyra_amd.kernels import decode_fused as F
     from lyra_amd.kernels.decode_attention import decode_attention
     from lyra_amd.nn.quant import QArray, quantize
@@ -469,7 +503,8 @@ def test_attention_with_the_front_step_equals_the_two_launches(B, N, K, S, H, fp
     gen.manual_seed(S + B)
     width = (N + 2 * K) * H
     if unsummed:
-        part = torch.randn(3, B, width, device=dev, generator=gen) * 0.8
+        n_slices = 3 if unsummed is True else int(unsummed)
+        part = torch.randn(n_slices, B, width, device=dev, generator=gen) * (1.4 / n_slices**0.5)
         qkv_a, qkv_b = F.Unsummed(part, None, 1.0), F.Unsummed(part.clone(), None, 1.0)
     else:
         t = (torch.randn(B, width, device=dev, generator=gen) * 2).to(torch.bfloat16)

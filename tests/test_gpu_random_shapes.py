@@ -167,7 +167,8 @@ def _draw_front_step(seed):
     if positions != "full":
         B = min(B, 256 // K)  # more pairs than compute units with one position per row is the whole-row kernel's case
     return dict(B=B, N=K * G, K=K, S=S, H=H, fp8=bool(rng.integers(0, 2)), qknorm=bool(rng.integers(0, 2)),
-                sw=pick([0, 0, 1, 33, 128, 1000]), unsummed=bool(rng.integers(0, 2)), positions=positions)
+                sw=pick([0, 0, 1, 33, 128, 1000]), unsummed=pick([False, False, 1, 2, 3, 4, 5, 7, 8, 9, 12, 16]),
+                positions=positions)
 
 
 @pytest.mark.parametrize("seed", range(32))
