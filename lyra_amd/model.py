@@ -20,7 +20,7 @@ import torch
 
 from lyra_amd.kernels.common import Implementation
 from lyra_amd.kernels.op import Mode, attn_op, gmm_op
-from lyra_amd.nn.quant import QArray, quantize
+from lyra_amd.nn.quant import QArray, dot, quantize
 
 PADDED_VOCAB_SIZE = 204800  # lyra/tokenizer.py:3
 
@@ -339,7 +339,11 @@ def cache_update(cache: LayerCache, k: torch.Tensor, v: torch.Tensor, pos: torch
 
 # ---- layers ------------------------------------------------------------------------------------------
 def _dense(x: torch.Tensor, w, cfg: ModelConfig, *, fused_swiglu=False, out_f32=False, bias=None) -> torch.Tensor:
-    """quant.dot for a [B, C] activation (lyra/nn/quant.py:106-108) = the one-group decode matmul."""
+    """quant.dot for a [B, C] activation (lyra/nn/quant.py:106-108) = the one-group decode matmul.  With a SwiGLU or a
+    float32 bias behind it the operator's fused epilogue does both (the decode_gemm operator itself)."""
+    if not fused_swiglu and bias is None:
+        w2 = QArray(w.qval[0], w.scale[0], w.block) if isinstance(w, QArray) else w[0]
+        return dot(x, w2, preferred_element_type=torch.float32 if out_f32 else None, implementation=cfg.implementation)
     gmm = gmm_op(cfg.mode, cfg.implementation)
     sizes = torch.full((1,), x.shape[0], dtype=torch.int32, device=x.device)
     lhs = x.to(torch.float32) if out_f32 else x

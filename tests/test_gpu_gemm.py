@@ -130,6 +130,50 @@ def test_dense_projection_is_the_one_group_case(K, N):
             U.assert_close(_run(c, swiglu), _want(c, swiglu, big=True), what=f"dense M={M}")
 
 
+@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", "channel"), ("fp8", (256, 1, 256))])
+def test_quant_dot_takes_the_projections_of_a_decode_step_to_the_kernel(kind, block):
+    """lyra_amd.nn.quant.dot with the reference's call shapes (lyra/model.py:307-309, 366, 614, 628: [B, 1, C] . [C, N] and
+    the [C, 2, Hd] up projection under NN_INNER) against the float32 oracle on the same dequantised weights; "pallas" and
+    "auto" must be the HIP kernel (bit-identical to the one-group decode_gemm call), "xla" the torch path."""
+    from lyra_amd.kernels.decode_gemm import decode_gemm
+    from lyra_amd.nn.quant import QArray, dot, einsum
+
+    NN_INNER = (((2,), (0,)), ((), ()))
+    B, C, Hd = 64, 2048, 3072
+    rng = np.random.default_rng(61)
+    x = O.bf16_round(rng.standard_normal((B, 1, C), dtype=np.float32))
+    for shape in ((C, 2560), (C, 2, Hd)):
+        w = (rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)).astype(np.float32)
+        N = int(np.prod(shape[1:]))
+        _note(f"quant.dot {kind} block={block} rhs={shape}")
+        if kind == "fp8":
+            blk = (C,) + (1,) * (len(shape) - 1) if block == "channel" else ((256, 256) if len(shape) == 2 else block)
+            flat_blk = (blk[0], blk[-1])
+            q, sc = clib.quantize_blocks(w.reshape(1, C, N), flat_blk)
+            rhs = QArray(U.t_fp8(q.reshape(shape)), U.t_f32(sc.reshape((C // blk[0],) + shape[1:-1] + (shape[-1] // blk[-1],))), blk)
+            rhs_flat = QArray(rhs.qval.reshape(1, C, N), rhs.scale.reshape(1, C // blk[0], -1), flat_blk)
+            want = clib.decode_gemm(O.bf16_bits(x[:, 0]), q, sc, flat_blk, np.array([B], np.int32), None)
+        else:
+            rhs = U.t_bf16(w)
+            rhs_flat = rhs.reshape(1, C, N)
+            want = clib.decode_gemm(O.bf16_bits(x[:, 0]), O.bf16_bits(O.bf16_round(w).reshape(1, C, N)), None, None,
+                                    np.array([B], np.int32), None)
+        xt = U.t_bf16(x)
+        got = dot(xt, rhs, dimension_numbers=NN_INNER, implementation="pallas")
+        assert tuple(got.shape) == (B, 1) + shape[1:] and got.dtype == torch.bfloat16
+        U.assert_close(U.to_np(got).reshape(B, N), want, what="dot bf16")
+        got32 = dot(xt, rhs, dimension_numbers=NN_INNER, preferred_element_type=torch.float32, implementation="pallas")
+        assert got32.dtype == torch.float32
+        U.assert_close(U.to_np(got32).reshape(B, N), want, atol=2e-3, rtol=2e-3, what="dot f32")
+        sizes = torch.full((1,), B, dtype=torch.int32, device=U.dev())
+        direct = decode_gemm(xt[:, 0], rhs_flat, sizes, quant_dtype=torch.float8_e4m3fn if kind == "fp8" else None, implementation="pallas")
+        assert torch.equal(got.reshape(B, N), direct)
+        assert torch.equal(dot(xt, rhs, dimension_numbers=NN_INNER), got)  # auto = the kernel
+        assert torch.equal(einsum("btc,c" + "jh"[: len(shape) - 1] + "->bt" + "jh"[: len(shape) - 1], xt, rhs), got)
+        plain = dot(xt, rhs, dimension_numbers=NN_INNER, implementation="xla")
+        U.assert_close(U.to_np(plain).reshape(B, N), want, what="dot plain path")
+
+
 def _zipf_routing(rng, T, n_routed, k, n_shared):
     p = 1.0 / np.arange(1, n_routed + 1) ** 1.1
     p /= p.sum()

@@ -321,3 +321,41 @@ def test_cache_append_outside_the_cache_writes_nothing(fp8):
             now = arr.qval.view(torch.uint8) if isinstance(arr, QArray) else arr
             keep = [i for i in range(S) if i != pos]
             assert torch.equal(now[:, :, keep], old[:, :, keep])
+
+
+def test_quant_dot_and_einsum_on_the_plain_path():
+    """lyra/nn/quant.py:106-113 on CPU tensors (the torch path): dequantise-if-QArray, then the contraction lax.dot_general
+    describes; output axes are batch, lhs free, rhs free; output dtype is preferred_element_type or lhs.dtype."""
+    from lyra_amd.nn.quant import dequantize, dot, einsum, quantize
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 1, 64, generator=g).to(torch.bfloat16)
+    w = (torch.randn(64, 2, 48, generator=g) * 0.1).to(torch.bfloat16)
+    nn_inner = (((2,), (0,)), ((), ()))
+    want = torch.einsum("btc,cjh->btjh", x.float(), w.float())
+    got = dot(x, w, dimension_numbers=nn_inner)
+    assert got.shape == (3, 1, 2, 48) and got.dtype == torch.bfloat16
+    assert (got.float() - want).abs().max() <= 2e-2
+    got32 = dot(x, w, dimension_numbers=nn_inner, preferred_element_type=torch.float32)
+    assert got32.dtype == torch.float32 and (got32 - want).abs().max() <= 1e-5
+    # a QArray weight is dequantised to the activation dtype first (quant.py:101-103)
+    qw = quantize(w, torch.float8_e4m3fn, (32, 1, 16))
+    assert qw.scale.shape == (2, 2, 3)
+    want_q = torch.einsum("btc,cjh->btjh", x.float(), dequantize(qw, torch.bfloat16).float())
+    assert (dot(x, qw, dimension_numbers=nn_inner, preferred_element_type=torch.float32) - want_q).abs().max() <= 1e-5
+    assert torch.equal(dot(x[:, 0], qw.__class__(qw.qval[:, 0], qw.scale[:, 0], (32, 16))), dot(x, qw)[:, 0, 0])
+    # default dimension numbers: last axis of lhs with first axis of rhs
+    assert torch.equal(dot(x, w), got)
+    # a contraction with a batch axis: [b, t, c] . [b, c, n] over c, batched over b
+    wb = torch.randn(3, 64, 5, generator=g).to(torch.bfloat16)
+    got_b = dot(x, wb, dimension_numbers=(((2,), (1,)), ((0,), (0,))), preferred_element_type=torch.float32)
+    assert got_b.shape == (3, 1, 5)
+    assert (got_b - torch.einsum("btc,bcn->btn", x.float(), wb.float())).abs().max() <= 1e-5
+    # einsum: the projection pattern is dot; anything else is torch.einsum on the dequantised weight
+    assert torch.equal(einsum("btc,cjh->btjh", x, qw), dot(x, qw))
+    sc = torch.rand(3, 2, generator=g)
+    rows = torch.randn(3, 2, 7, generator=g)
+    assert torch.allclose(einsum("fkc,fk->fc", rows, sc), (rows * sc[:, :, None]).sum(1))  # lyra/model.py:557
+    # the kernel cannot be asked for on CPU tensors
+    with pytest.raises(ValueError, match="no HIP kernel"):
+        dot(x, w, implementation="pallas")
