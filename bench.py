@@ -269,7 +269,7 @@ def zipf_group_sizes(rng, tokens, n_routed, k_routed, n_shared):
     return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
 
 
-def kernel_table(dev, only=""):
+def kernel_table(dev, only="", span_major=False):
     """Stand-alone timings of the two operators through the C ABI at the shapes of the named model variants: HIP events
     over back-to-back launches, once rotating over enough distinct caches / weight sets that every launch streams from
     HBM ("cold") and once re-using one set ("hot", which the 256 MB last-level cache may serve in part)."""
@@ -347,13 +347,26 @@ def kernel_table(dev, only=""):
         touched = int((np.asarray(sizes) > 0).sum())
         nbytes = touched * K * N * es + (touched * (K // bk) * (N // bn) * 4 if fp8 else 0) + M * K * 2 + M * NO * out.element_size()
 
+        dt = _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16
+        flag = 0
+        if span_major and N < 100000:  # the weights in the span-major copy lyra_gemm_pack makes (not for the LM head's kernel)
+            layout = 2 if (swiglu and G > 1) else 1
+            flag = _lib.RHS_SPAN_MAJOR if layout == 1 else _lib.RHS_SPAN_MAJOR_GLU
+            packed = []
+            for w in weights:
+                buf = torch.empty(L.lyra_gemm_packed_bytes(G, K, N, dt, layout), dtype=torch.uint8, device=dev)
+                _lib.check(L.lyra_gemm_pack(w.data_ptr(), buf.data_ptr(), G, K, N, dt, layout, stream.cuda_stream), "lyra_gemm_pack")
+                packed.append(buf)
+            stream.synchronize()
+            weights = packed
+            label += " [span-major]"
+
         def launch(i, hot=False):
-            rc = L.lyra_decode_gemm(
-                lhs.data_ptr(), weights[0 if hot else i % nbuf].data_ptr(), scale.data_ptr() if fp8 else None, bk, bn,
-                gs.data_ptr(), None, out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N,
-                _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(swiglu),
-                1.702, 7.0, stream.cuda_stream)
-            _lib.check(rc, "lyra_decode_gemm")
+            rc = L.lyra_decode_gemm_ex(
+                lhs.data_ptr(), None, weights[0 if hot else i % nbuf].data_ptr(), scale.data_ptr() if fp8 else None, bk, bn,
+                gs.data_ptr(), None, None, 1.0, 0, out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N,
+                dt | flag, _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(swiglu), 1.702, 7.0, stream.cuda_stream)
+            _lib.check(rc, "lyra_decode_gemm_ex")
 
         cold = _time_launches(launch, stream)
         hot = _time_launches(lambda i: launch(i, True), stream)
@@ -488,6 +501,8 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
     ap.add_argument("--only", default="", help="with --kernels: only the cases whose name contains this text")
+    ap.add_argument("--span-major", action="store_true",
+                    help="with --kernels: the matmuls read the span-major copy of their weights (lyra_gemm_pack)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a copy-like kernel of known size (reference point for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -499,7 +514,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.kernels:
-        rows = kernel_table(dev, args.only)
+        rows = kernel_table(dev, args.only, args.span_major)
         if args.traffic_probe:
             traffic_probe(dev)
         for r in rows:

@@ -18,12 +18,16 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 11
+#define LYRA_ABI_VERSION 12
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
 #define LYRA_DTYPE_E4M3FN 1 /* OCP FP8 E4M3 (finite, max 448), 1 byte; needs scales */
 #define LYRA_DTYPE_F32 2    /* float32 (outputs only) */
+/* OR-ed into rhs_dtype of lyra_decode_gemm_ex / lyra_decode_gemm_partials: rhs is not the reference's [G,K,N] array but
+ * the span-major copy of it that lyra_gemm_pack writes (layout 1 or 2 below). */
+#define LYRA_RHS_SPAN_MAJOR 0x100     /* layout 1: spans of 128 consecutive columns */
+#define LYRA_RHS_SPAN_MAJOR_GLU 0x200 /* layout 2: spans of 64 gate columns + their 64 linear columns (fused_swiglu) */
 
 #define LYRA_OK 0
 #define LYRA_E_BADARG (-1)      /* null pointer, non-positive size, N % K != 0 ... */
@@ -191,6 +195,28 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
                         int post_scale, void* out, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
                         int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
                         lyra_stream_t stream);
+
+/*
+ * Span-major weights (no counterpart in the reference, whose kernels read [G,K,N] as it is: lyra/kernels/decode_gemm.py:
+ * 145-298).  A decode matmul streams, per workgroup, one 128-column span of a weight matrix from its first K row to its
+ * last; in the row-major [G,K,N] array those are 128-byte pieces N bytes apart - and pieces that straddle two cache
+ * lines whenever N (or N/2, where the linear half of a SwiGLU projection starts) is not a multiple of 128 bytes, as
+ * with gpt-oss-20b's width 2880.  lyra_gemm_pack copies the weights once, at load time, so that every span is one
+ * contiguous, 128-byte aligned run of K rows of 128 elements:
+ *   layout 1 (LYRA_RHS_SPAN_MAJOR):      packed[g][s][k][c] = rhs[g][k][128 s + c],           s < ceil(N / 128)
+ *   layout 2 (LYRA_RHS_SPAN_MAJOR_GLU):  packed[g][s][k][c] = rhs[g][k][64 s + c]             (c < 64: gate column)
+ *                                                          = rhs[g][k][N/2 + 64 s + c - 64]   (c >= 64: its linear column),
+ *                                                                                            s < ceil(N / 2 / 64)
+ * with zeros where the column does not exist (a last span that N does not fill).  Scales, biases and outputs keep the
+ * reference's column order.  lyra_decode_gemm_ex takes layout 2 for several groups with fused_swiglu, layout 1 for
+ * several groups without and for the K-split projections of one group (with or without fused_swiglu), and answers
+ * LYRA_E_UNSUPPORTED for any other combination; lyra_decode_gemm_partials takes layout 1.  Results are the same
+ * function of the same weights; the float32 summation order over K may differ from the row-major call's.
+ *   lyra_gemm_packed_bytes  size of the packed copy (0 for bad arguments)
+ *   lyra_gemm_pack          rhs [G,K,N] (rhs_dtype bf16 or e4m3fn) -> packed; layout 1 or 2; N % 8 == 0 (16 for layout 2)
+ */
+size_t lyra_gemm_packed_bytes(int G, int K, int N, int rhs_dtype, int layout);
+int lyra_gemm_pack(const void* rhs, void* packed, int G, int K, int N, int rhs_dtype, int layout, lyra_stream_t stream);
 
 /*
  * A dense projection (one group, a few MB of weights) runs split over K across all compute units; the float32

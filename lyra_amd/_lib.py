@@ -8,7 +8,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
-ABI_VERSION = 11
+RHS_SPAN_MAJOR, RHS_SPAN_MAJOR_GLU = 0x100, 0x200  # LYRA_RHS_SPAN_MAJOR(_GLU): OR-ed into a matmul's rhs_dtype
+ABI_VERSION = 12
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 
 _c = ctypes
@@ -53,6 +54,8 @@ SIGNATURES = {
     "lyra_moe_route": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 4 + [_c.c_void_p]),
     "lyra_moe_combine": (_c.c_int, [_c.c_void_p] * 5 + [_c.c_int] * 3 + [_c.c_float, _c.c_void_p]),
     "lyra_decode_gemm_splits": (_c.c_int, [_c.c_int] * 4),
+    "lyra_gemm_packed_bytes": (_c.c_size_t, [_c.c_int] * 5),
+    "lyra_gemm_pack": (_c.c_int, [_c.c_void_p] * 2 + [_c.c_int] * 5 + [_c.c_void_p]),
     "lyra_decode_gemm_partials": (
         _c.c_int,
         [_c.c_void_p] * 3 + [_c.c_int] * 2 + [_c.c_void_p] * 2 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_void_p],

@@ -49,6 +49,10 @@ struct GemmParams {
     const uint16_t* residual;  // bf16 [M, NO] added after scaling, or null
     float out_scale;           // epilogue: out = bf16(residual + bf16(bf16(t) * out_scale)) when post_scale is set
     int post_scale;
+    // span-major weights (lyra_gemm_pack): 0 = rhs is [G,K,N]; 1 = [G][pspans][K][128], span s = columns 128 s ...;
+    // 2 = the same with span s = gate columns 64 s ... followed by their linear columns N/2 + 64 s ...
+    int packed;
+    int pspans;
 };
 
 // Results go out with plain stores; only the float32 K slices that the next kernel sums are written through at agent
@@ -706,10 +710,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     const int n_my = (STEP_SCALES && !LOOP) ? max(0, min(DEPTH, steps - wave * DEPTH)) : (steps - wave + kSplitWaves - 1) / kSplitWaves;
     auto step_row = [&](int d) { return k0 + (((STEP_SCALES && !LOOP) ? wave * DEPTH + d : wave + kSplitWaves * d) << 5); };
 
-    const int row_bytes = p.N * ES;
+    // (span-major weights: this workgroup's span is a contiguous run of K rows of 128 weights)
+    const int row_bytes = p.packed ? 128 * ES : p.N * ES;
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.rhs), 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-    const int wvoff = cols ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
+        const_cast<uint8_t*>(p.rhs) + (p.packed ? (size_t)span * p.K * row_bytes : (size_t)0), 0, (uint32_t)p.K * (uint32_t)row_bytes,
+        0x00020000);
+    const int wvoff = cols ? 8 * kb * row_bytes + (p.packed ? 8 * x : ncol) * ES : kNoLoad;
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.lhs), 0, 0x7FFFFFFFu, 0x00020000);
     int avoff[MT];
 #pragma unroll
@@ -971,7 +977,11 @@ __device__ __forceinline__ unsigned long long wg_scan_exclusive4(unsigned long l
 
 // WIDE_DYN: an instantiation for launches without SwiGLU that may have enough units for the wider ones (decided below,
 // once the unit list is known; the other instantiations know their layout from the start).
-template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false>
+// PACKED: the weights are span-major (GemmParams::packed): every unit streams one or two contiguous runs of K rows of 128
+// weights.  With SwiGLU a span then holds 64 gate columns and their 64 linear columns, so a unit of one span is half as
+// wide as without the copy and a launch has twice the units to deal out; whether wavefront pairs take two spans (as many
+// rounds as before) or all four wavefronts one span (short lists: finer shares) is decided once the unit list is known.
+template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false, bool PACKED = false>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int DEPTH = FP8 ? 4 : 2;
@@ -990,22 +1000,23 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     // which streams ~14 % faster); otherwise one set of 128 columns and all 4 wavefronts interleave.
     const int NO = p.swiglu ? p.N >> 1 : p.N;
     const int q = threadIdx.x & 31;
-    const int row_bytes = p.N * ES;
+    const int row_bytes = PACKED ? 128 * ES : p.N * ES;
     const int steps = p.K >> 5;
     const int half_stride = p.swiglu ? (p.N >> 1) : 128;
     bool wide;
     int spans, kw, wslot, half, span_cols, tile_cols, n_my, trips;
     auto set_layout = [&](bool w) {
         wide = w;
-        spans = p.swiglu ? ((p.N >> 1) + 127) / 128 : (w ? p.N / 256 : (p.N + 127) / 128);  // (the last span may be partly filled)
+        if constexpr (PACKED) spans = w ? (p.pspans + 1) >> 1 : p.pspans;
+        else spans = p.swiglu ? ((p.N >> 1) + 127) / 128 : (w ? p.N / 256 : (p.N + 127) / 128);  // (the last span may be partly filled)
         kw = w ? 2 : kSplitWaves;
         wslot = w ? (wave & 1) : wave, half = w ? (wave >> 1) : 0;
-        span_cols = p.swiglu || !w ? 128 : 256;
+        span_cols = PACKED ? (p.swiglu ? (w ? 128 : 64) : (w ? 256 : 128)) : (p.swiglu || !w ? 128 : 256);  // output columns of a unit
         tile_cols = w ? 256 : 128;                                  // floats per row of a workspace slot
         n_my = (steps - wslot + kw - 1) / kw;                       // steps of this wavefront in a whole unit
         trips = ((steps + kw - 1) / kw + TRIP - 1) / TRIP;          // trips of a whole unit (same for every wavefront)
     };
-    if constexpr (!WIDE_DYN) set_layout(p.swiglu || p.wide);
+    if constexpr (!WIDE_DYN) set_layout(PACKED ? false : (p.swiglu || p.wide));
 
     // ---- unit list: thread t looks at group G-1-t ----
     const int t = threadIdx.x;
@@ -1038,7 +1049,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             sm_blk[j][2] = min(16 * MTM, my_cnt - i * 16 * MTM);
         }
     }
-    if (n_blocks_all * (p.N >> 8) > (int)gridDim.x) {
+    if (n_blocks_all * (PACKED ? p.pspans : (p.N >> 8)) > (int)gridDim.x) {
         // More than one round of units: the list is put in the order of cost, in four classes by the number of 16-row
         // tiles a block fills - all blocks of 49-64 rows (in group order from the last group down), then those of 33-48,
         // 17-32 and 1-16 rows - so that, whatever the order of the groups, the units at the end of the list are the light
@@ -1066,7 +1077,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     const int nwg = gridDim.x;
     // Without SwiGLU the wider units are taken when they still fill 1.75 rounds of workgroups (lyra-max down projection at
     // batch 128: -8 %); with fewer, their coarser rounds cost more than the access pattern gains.
-    if constexpr (WIDE_DYN) set_layout(p.swiglu || p.wide || 4 * n_blocks * (p.N / 256) >= 7 * nwg);
+    if constexpr (WIDE_DYN) {
+        if constexpr (PACKED) set_layout(p.wide || 4 * n_blocks * ((p.pspans + 1) >> 1) >= 7 * nwg);
+        else set_layout(p.swiglu || p.wide || 4 * n_blocks * (p.N / 256) >= 7 * nwg);
+    }
     const int n_units = __builtin_amdgcn_readfirstlane(n_blocks * spans);  // (same in every lane: tell the compiler)
     // whole units in full rounds of nwg; when there is not even one full round, the units are cut into `slices` K slices each
     // (a power of two that divides trips).  After a full round slicing the rest was measured to cost as much as it saves:
@@ -1083,6 +1097,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     bool seg_valid = false;
     int seg_u = 0, seg_r0 = 0, seg_r1 = 0;  // its unit and trips [r0, r1) of it
     int g = 0, row0 = 0, rows = 0, span = 0, ncol = 0, wvoff = kNoLoad, avoff[MTM];
+    bool seg_cols = false;  // the lane's columns exist (scales of absent columns are not read)
     __amdgpu_buffer_rsrc_t wrsrc;
     constexpr int ADEPTH = 2;  // activation steps in flight (they come from the caches; the weights, from memory, need DEPTH)
     u32x4 a[ADEPTH][MTM];
@@ -1124,13 +1139,33 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         g = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][0] : 0);
         row0 = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][1] : 0);
         rows = __builtin_amdgcn_readfirstlane(valid ? sm_blk[blk][2] : 0);
-        ncol = half * half_stride + span * span_cols + 8 * x;
-        // (N need not fill the last span: lanes past the last column - of the gate or linear half with SwiGLU - load
-        // nothing, accumulate zeros and are left out of the epilogue)
-        const bool cols = span * span_cols + (wide && !p.swiglu ? 128 * half : 0) + 8 * x < NO;
-        wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
-                                                  (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-        wvoff = valid && cols ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
+        bool cols;
+        if constexpr (PACKED) {
+            // this wavefront's span of the packed copy: K rows of 128 weights, contiguous.  ncol is the column (of the
+            // reference's array) that the lane's first weight belongs to: scales and biases keep that order.
+            const int ps = wide ? 2 * span + half : span;
+            const bool ps_ok = ps < p.pspans;
+            if (p.swiglu) {
+                ncol = (x < 8 ? 0 : (p.N >> 1)) + 64 * ps + 8 * (x & 7);
+                cols = ps_ok && 64 * ps + 8 * (x & 7) < NO;
+            } else {
+                ncol = 128 * ps + 8 * x;
+                cols = ps_ok && ncol < NO;
+            }
+            wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint8_t*>(p.rhs) + ((size_t)g * p.pspans + (ps_ok ? ps : 0)) * p.K * row_bytes, 0,
+                (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+            wvoff = valid && ps_ok ? 8 * kb * row_bytes + 8 * x * ES : kNoLoad;  // (columns N does not have hold zeros)
+        } else {
+            ncol = half * half_stride + span * span_cols + 8 * x;
+            // (N need not fill the last span: lanes past the last column - of the gate or linear half with SwiGLU - load
+            // nothing, accumulate zeros and are left out of the epilogue)
+            cols = span * span_cols + (wide && !p.swiglu ? 128 * half : 0) + 8 * x < NO;
+            wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0,
+                                                      (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+            wvoff = valid && cols ? 8 * kb * row_bytes + ncol * ES : kNoLoad;
+        }
+        seg_cols = cols;
         if constexpr (STEP_SCALES) sc_voff = valid && cols ? (g * p.KB * p.NB + (ncol >> p.bn_shift)) * 4 : kNoLoad;
 #pragma unroll
         for (int mt = 0; mt < MTM; ++mt) {
@@ -1169,6 +1204,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     while (seg_valid) {
         const int cur_u = seg_u, r0 = seg_r0, r1 = seg_r1;
         const int cur_g = g, cur_row0 = row0, cur_rows = rows, cur_span = span, cur_ncol = ncol;
+        const bool cur_cols = seg_cols;
         const int n_mt = (cur_rows + 15) >> 4;
         const __amdgpu_buffer_rsrc_t cur_wrsrc = wrsrc;
         const int cur_wvoff = wvoff;
@@ -1274,11 +1310,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         for (int c = 0; c < 8; ++c) {
             colscale[c] = 1.f;  // (scale blocks along K were applied to the weights)
             if (FP8 && p.scale_mode == 1 && !STEP_SCALES) {
-                const int off = (cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift)) * 4;
+                const int off = (!PACKED || cur_cols) ? (cur_g * p.KB * p.NB + (cur_ncol >> p.bn_shift)) * 4 : kNoLoad;
                 if (c == 0) colscale[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));
                 else colscale[c] = colscale[0];
             } else if (FP8 && p.scale_mode == 2) {
-                const int off = (cur_g * p.NB + ((cur_ncol + c) >> p.bn_shift)) * 4;
+                const int off = (!PACKED || cur_cols) ? (cur_g * p.NB + ((cur_ncol + c) >> p.bn_shift)) * 4 : kNoLoad;
                 colscale[c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scrsrc, off, 0, 0));
             }
         }
@@ -1376,7 +1412,43 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                 }
             }
         }
-        if (finish) {
+        if (finish && PACKED && p.swiglu) {
+            // A span's tile holds 64 gate columns followed by their 64 linear columns.  Thread (eq = q & 15) finishes 4 output
+            // columns of one row for each span of the unit; the 32 threads that share threadIdx.x >> 5 take two rows.
+            const int eq = q & 15;
+            const int oc_a = cur_span * span_cols + 4 * eq, oc_b = oc_a + 64;  // first output column in the unit's first / second span
+            const bool a_live = oc_a < NO, b_live = wide && oc_b < NO;
+            const f32x4 bias_ga = load_f32x4(bias_rsrc, (p.bias && a_live) ? (cur_g * p.N + oc_a) * 4 : kNoLoad);
+            const f32x4 bias_la = load_f32x4(bias_rsrc, (p.bias && a_live) ? (cur_g * p.N + NO + oc_a) * 4 : kNoLoad);
+            const f32x4 bias_gb = load_f32x4(bias_rsrc, (p.bias && b_live) ? (cur_g * p.N + oc_b) * 4 : kNoLoad);
+            const f32x4 bias_lb = load_f32x4(bias_rsrc, (p.bias && b_live) ? (cur_g * p.N + NO + oc_b) * 4 : kNoLoad);
+            const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int r = 2 * (int)(threadIdx.x >> 5) + (q >> 4); r < cur_rows; r += 16) {
+                const float* src = sm_part + r * kSplitPitch + 4 * eq;
+                const f32x4 g0 = *(const f32x4*)src, g1 = *(const f32x4*)(src + TS), g2 = *(const f32x4*)(src + 2 * TS),
+                            g3 = *(const f32x4*)(src + 3 * TS);
+                const f32x4 l0 = *(const f32x4*)(src + 64), l1 = *(const f32x4*)(src + 64 + TS),
+                            l2 = *(const f32x4*)(src + 64 + 2 * TS), l3 = *(const f32x4*)(src + 64 + 3 * TS);
+                f32x4 ga, la, gb = zero4, lb = zero4;
+                if (wide) {
+                    ga = g0 + g1;
+                    la = l0 + l1;
+                    gb = g2 + g3;
+                    lb = l2 + l3;
+                } else {
+                    ga = ((g0 + g1) + g2) + g3;
+                    la = ((l0 + l1) + l2) + l3;
+                }
+                const size_t oa = (size_t)(cur_row0 + r) * NO + oc_a;
+                f32x4 res_a = zero4, res_b = zero4;
+                if (p.residual) {
+                    res_a = load_bf16x4(res_rsrc, a_live ? (int)(oa * 2) : kNoLoad);
+                    res_b = load_bf16x4(res_rsrc, b_live ? (int)((oa + 64) * 2) : kNoLoad);
+                }
+                if (a_live) finish4(p, ga, la, bias_ga, bias_la, res_a, oa);
+                if (b_live) finish4(p, gb, lb, bias_gb, bias_lb, res_b, oa + 64);
+            }
+        } else if (finish) {
             // biases of this thread's columns once per unit; residual values per row; every load unconditional (a null
             // operand is read with an offset outside its descriptor and yields zeros), rows two at a time
             const int oc = cur_span * span_cols + 4 * q;
@@ -1429,7 +1501,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
     const int total = total_rows;
     const int pad_rows = p.M - min(total, p.M);
-    const int pad_spans = p.swiglu ? spans : (p.N + 127) / 128;
+    const int pad_spans = (NO + 127) / 128;
     for (int i = blockIdx.x; i < pad_rows * pad_spans; i += gridDim.x) {
         const int sp = i % pad_spans;
         if (threadIdx.x < 32 && sp * 128 + 4 * q < NO) {
@@ -1439,6 +1511,45 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         }
     }
 }
+
+// ---- span-major copy of a weight array (done once, when the weights are loaded) ---------------------------------------
+// One thread moves 8 consecutive elements of a packed row: they come from 8 consecutive columns of the reference's array
+// (widths are multiples of 8, or 16 with gate and linear halves) or are zeros where the span runs past the last column.
+struct PackParams {
+    const uint8_t* src;
+    uint8_t* dst;
+    int G, K, N, es, glu, pspans;
+};
+__global__ __launch_bounds__(256) void gemm_pack_kernel(PackParams p) {
+    const size_t total = (size_t)p.G * p.pspans * p.K * 16;  // pieces of 8 elements
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int piece = (int)(i & 15);
+        const size_t row = i >> 4;  // (g * pspans + s) * K + k
+        const int k = (int)(row % p.K);
+        const size_t gs = row / p.K;
+        const int s = (int)(gs % p.pspans), g = (int)(gs / p.pspans);
+        int col;  // first source column of the piece, or -1
+        if (p.glu) {
+            const int half = p.N >> 1, c = 64 * s + 8 * (piece & 7);
+            col = c < half ? (piece < 8 ? c : half + c) : -1;
+        } else {
+            const int c = 128 * s + 8 * piece;
+            col = c < p.N ? c : -1;
+        }
+        const size_t dst = i * 8 * p.es;
+        if (p.es == 1) {
+            u32x2 v = u32x2{0u, 0u};
+            if (col >= 0) v = *(const u32x2*)(p.src + ((size_t)g * p.K + k) * p.N + col);
+            *(u32x2*)(p.dst + dst) = v;
+        } else {
+            u32x4 v = u32x4{0u, 0u, 0u, 0u};
+            if (col >= 0) v = *(const u32x4*)(p.src + (((size_t)g * p.K + k) * p.N + col) * 2);
+            *(u32x4*)(p.dst + dst) = v;
+        }
+    }
+}
+
+static int packed_spans(int N, int layout) { return layout == 2 ? (N / 2 + 63) / 64 : (N + 127) / 128; }
 
 struct GemmPlan {
     int mt;       // 16-row tiles held in registers per pass
@@ -1607,6 +1718,26 @@ static size_t gemm_partial_bytes(const GemmPlan& pl, int M, int N) {
 }
 }  // namespace lyra
 
+extern "C" size_t lyra_gemm_packed_bytes(int G, int K, int N, int rhs_dtype, int layout) {
+    if (G <= 0 || K <= 0 || N <= 0 || (layout != 1 && layout != 2)) return 0;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return 0;
+    if (N % 8 || (layout == 2 && N % 16)) return 0;
+    return (size_t)G * lyra::packed_spans(N, layout) * K * 128 * (rhs_dtype == LYRA_DTYPE_E4M3FN ? 1 : 2);
+}
+
+extern "C" int lyra_gemm_pack(const void* rhs, void* packed, int G, int K, int N, int rhs_dtype, int layout, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!rhs || !packed || G <= 0 || K <= 0 || N <= 0 || (layout != 1 && layout != 2)) return LYRA_E_BADARG;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    if (N % 8 || (layout == 2 && N % 16)) return LYRA_E_UNSUPPORTED;
+    if (((uintptr_t)rhs | (uintptr_t)packed) % 16) return LYRA_E_BADARG;
+    PackParams p{(const uint8_t*)rhs, (uint8_t*)packed, G, K, N, rhs_dtype == LYRA_DTYPE_E4M3FN ? 1 : 2, layout == 2, packed_spans(N, layout)};
+    const size_t pieces = (size_t)G * p.pspans * K * 16;
+    const unsigned blocks = (unsigned)std::min<size_t>((pieces + 255) / 256, 65536);
+    hipLaunchKernelGGL(gemm_pack_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
 extern "C" size_t lyra_decode_gemm_workspace(int M, int G, int K, int N, int fused_swiglu) {
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return 0;
     // The scale block is not known here and decides both which kernel runs (a block that does not tile a K slice sends a
@@ -1639,6 +1770,10 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     using namespace lyra;
     const bool bias_post = (post_scale & 2) != 0;  // post_scale: bit 0 the scale / residual epilogue, bit 1 the bias after the cast
     post_scale &= 1;
+    // span-major weights (lyra_gemm_pack): the layout travels in the upper bits of rhs_dtype
+    const int layout = (rhs_dtype & LYRA_RHS_SPAN_MAJOR) ? 1 : ((rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU) ? 2 : 0);
+    if ((rhs_dtype & LYRA_RHS_SPAN_MAJOR) && (rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU)) return LYRA_E_BADARG;
+    rhs_dtype &= ~(LYRA_RHS_SPAN_MAJOR | LYRA_RHS_SPAN_MAJOR_GLU);
     if (residual && (!post_scale || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
     if (bias_post && (!bias || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
     if (bias_post && (G != 1 || fused_swiglu)) return LYRA_E_UNSUPPORTED;
@@ -1668,6 +1803,12 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         else return LYRA_E_UNSUPPORTED;
     }
     const GemmPlan pl = plan_gemm(M, G, K, N, fp8 ? bk : 0, fused_swiglu);
+    // the packed copy exists for the kernels that stream whole spans: several groups (layout 2 with SwiGLU, else 1) and
+    // the K-split projections of one group (layout 1)
+    if (layout && !((pl.grouped && layout == (fused_swiglu ? 2 : 1)) || (!pl.grouped && pl.split_k && layout == 1))) return LYRA_E_UNSUPPORTED;
+    if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
+    p.packed = layout;
+    p.pspans = layout ? packed_spans(N, layout) : 0;
     p.lhs = (const uint16_t*)lhs;
     p.rhs = (const uint8_t*)rhs;
     p.scale = rhs_scale;
@@ -1715,8 +1856,12 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     hipStream_t st = (hipStream_t)stream;
     if (pl.grouped) {
         // one workgroup per compute unit (more would only queue behind the LDS tiles), fewer when there is less work
-        const long most_units = (long)pl.spans * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
-        const int gkw = (fused_swiglu || pl.wide) ? 2 : kSplitWaves;
+        const long most_blocks = std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
+        // (packed: units of one span unless the list is long enough for units of two - the kernel's own rule, on the most
+        // row blocks the shapes allow)
+        const bool packed_wide = layout && 4 * most_blocks * ((p.pspans + 1) / 2) >= 7 * (long)kGroupMaxWgs;
+        const long most_units = (layout ? (long)p.pspans : (long)pl.spans) * most_blocks;
+        const int gkw = layout ? (packed_wide ? 2 : kSplitWaves) : ((fused_swiglu || pl.wide) ? 2 : kSplitWaves);
         const long trips_least = std::max(1, ((K / 32 + gkw - 1) / gkw + 7) / 8);  // trips per unit (at least)
         const dim3 ggrid((unsigned)std::max(1L, std::min((long)kGroupMaxWgs, most_units * trips_least))), gblock(kSplitWaves * 64);
         const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
@@ -1740,15 +1885,25 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
         hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, false, true>), ggrid, gblock, glds, st, p);             \
     } while (0)
+#define LYRA_GROUP_P(F, S, R, C, W)                                                                                   \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C, W, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C, W, true>), ggrid, gblock, glds, st, p);              \
+    } while (0)
 #define LYRA_GROUP_R(F, S, R)                                               \
     do {                                                                    \
-        if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
+        if (layout) {                                                       \
+            if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_P(F, S, R, true, false); \
+            else LYRA_GROUP_P(F, S, R, false, true);                        \
+        } else if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
         else if (wide_dyn) LYRA_GROUP_RSW(F, S, R);                         \
         else LYRA_GROUP_RS(F, S, R, false);                                 \
     } while (0)
 #define LYRA_GROUP(F, S, DEPTH_)                                                          \
     do {                                                                                  \
-        const int kw = (fused_swiglu || pl.wide) ? 2 : kSplitWaves;                       \
+        const int kw = gkw;                                                               \
         const int per_wave = (K / 32 + kw - 1) / kw;                                      \
         const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
         if (K % (kw * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);                 \
@@ -1759,6 +1914,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         else LYRA_GROUP(false, false, 2);
 #undef LYRA_GROUP
 #undef LYRA_GROUP_R
+#undef LYRA_GROUP_P
 #undef LYRA_GROUP_RSW
 #undef LYRA_GROUP_RS
         return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
@@ -1837,6 +1993,10 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
                                          int rhs_dtype, lyra_stream_t stream) {
     using namespace lyra;
     if (!lhs || !rhs || !group_sizes || !partials || M <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
+    if (rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU) return LYRA_E_UNSUPPORTED;
+    const int layout = (rhs_dtype & LYRA_RHS_SPAN_MAJOR) ? 1 : 0;
+    rhs_dtype &= ~LYRA_RHS_SPAN_MAJOR;
+    if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
     if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
@@ -1867,5 +2027,7 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     p.kpart = pl.kpart;
     p.row_par = pl.row_par;
     p.row_block = pl.row_block;
+    p.packed = layout;
+    p.pspans = layout ? packed_spans(N, layout) : 0;
     return launch_split_k(p, pl, fp8, (hipStream_t)stream);
 }

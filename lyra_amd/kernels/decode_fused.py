@@ -62,23 +62,93 @@ class Uncombined:
         self.rows, self.scores, self.dest, self.residual, self.scale = rows, scores, dest, residual, scale
 
 
+class SpanMajor:
+    """Weights [G, K, N] (bf16, or FP8 with their QArray scales) in the span-major copy ``lyra_gemm_pack`` makes once when a
+    model is loaded: every 128-column span of every matrix is one contiguous run of K rows.  ``layout`` 1: spans of 128
+    consecutive columns; 2: spans of 64 gate columns followed by their 64 linear columns (expert up projections, whose
+    SwiGLU is fused).  ``scale`` / ``block`` keep the reference's [G, K/bk, N/bn] layout.  Accepted by ``gemm`` and
+    ``gemm_unsummed`` wherever the reference array is; the array itself is no longer needed then."""
+
+    __slots__ = ("data", "shape", "dtype", "scale", "block", "layout", "fallback")
+
+    def __init__(self, data, shape, dtype, scale, block, layout, fallback=None):
+        self.data, self.shape, self.dtype, self.scale, self.block, self.layout = data, tuple(shape), dtype, scale, block, layout
+        self.fallback = fallback  # the reference array, when the caller kept it: used where no kernel reads this layout
+
+
+def pack_weights(rhs, glu: bool = False) -> SpanMajor:
+    """rhs: bf16 [G, K, N] tensor or FP8 QArray -> SpanMajor (layout 2 when ``glu``: gate and linear columns paired)."""
+    fp8 = isinstance(rhs, QArray)
+    rv = rhs.qval if fp8 else rhs
+    assert rv.is_contiguous() and rv.ndim == 3 and (fp8 or rv.dtype == torch.bfloat16)
+    G, K, N = rv.shape
+    layout = 2 if glu else 1
+    dt = _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16
+    nbytes = _L.lyra_gemm_packed_bytes(G, K, N, dt, layout)
+    if nbytes == 0:
+        raise ValueError(f"no span-major layout {layout} for weights {tuple(rv.shape)} {rv.dtype}")
+    data = torch.empty(nbytes, dtype=torch.uint8, device=rv.device)
+    _lib.check(_L.lyra_gemm_pack(rv.data_ptr(), data.data_ptr(), G, K, N, dt, layout, _stream(rv.device)), "lyra_gemm_pack")
+    return SpanMajor(data, (G, K, N), rv.dtype, _f32(rhs.scale) if fp8 else None, tuple(rhs.block) if fp8 else None, layout)
+
+
+_SPAN_MAJOR: dict = {}
+_SPAN_MAJOR_MODE = __import__("os").environ.get("LYRA_SPAN_MAJOR", "auto")  # tuning override: "0" never, "1" every weight
+
+
+def span_major(rhs, glu: bool = False):
+    """The weight operand a fused decode step should hand to ``gemm``: the span-major copy (made once per weight array and
+    kept) when the rows of the reference's array do not start on 128-byte lines - FP8 weights whose width, or whose linear
+    half under a fused SwiGLU, is not a multiple of 128 columns, as with gpt-oss-20b's 2880: every 128-byte piece a
+    workgroup reads from such an array straddles two lines and the launch fetches half as much again - else ``rhs``."""
+    if isinstance(rhs, SpanMajor) or _SPAN_MAJOR_MODE == "0":
+        return rhs
+    fp8 = isinstance(rhs, QArray)
+    rv = rhs.qval if fp8 else rhs
+    N = rv.shape[-1]
+    row = N * rv.element_size()
+    if _SPAN_MAJOR_MODE != "1" and row % 128 == 0 and not (glu and (row // 2) % 128):
+        return rhs
+    if N % (16 if glu else 8) or not rv.is_cuda:
+        return rhs
+    key = (rv.data_ptr(), tuple(rv.shape), glu)
+    hit = _SPAN_MAJOR.get(key)
+    if hit is None or hit[0] is not rv:
+        packed = pack_weights(rhs, glu)
+        packed.fallback = rhs
+        hit = (rv, packed)
+        _SPAN_MAJOR[key] = hit
+    return hit[1]
+
+
+def _rhs_args(rhs):
+    """(data tensor, scale tensor | None, bk, bn, rhs_dtype word of the C ABI, shape) of a weight operand."""
+    if isinstance(rhs, SpanMajor):
+        fp8 = rhs.scale is not None
+        flag = _lib.RHS_SPAN_MAJOR if rhs.layout == 1 else _lib.RHS_SPAN_MAJOR_GLU
+        bk, bn = rhs.block if fp8 else (0, 0)
+        return rhs.data, rhs.scale, bk, bn, (_lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16) | flag, rhs.shape
+    if isinstance(rhs, QArray):
+        bk, bn = rhs.block
+        assert rhs.qval.is_contiguous()
+        return rhs.qval, _f32(rhs.scale), bk, bn, _lib.DTYPE_E4M3FN, tuple(rhs.shape)
+    assert rhs.dtype == torch.bfloat16 and rhs.is_contiguous()
+    return rhs, None, 0, 0, _lib.DTYPE_BF16, tuple(rhs.shape)
+
+
 def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed | None:
     """lyra_decode_gemm_partials for a one-group projection; None when the shape does not run split over K."""
     M, K = lhs.shape
-    G, _, N = rhs.shape
-    fp8 = isinstance(rhs, QArray)
-    bk, bn = rhs.block if fp8 else (0, 0)
-    if G != 1 or K % 32 or N % 128:
+    rv, rs, bk, bn, rd, (G, _, N) = _rhs_args(rhs)
+    if G != 1 or K % 32 or N % 128 or (isinstance(rhs, SpanMajor) and rhs.layout != 1):
         return None
     splits = _L.lyra_decode_gemm_splits(M, K, N, bk)
     if splits <= 0:
         return None
     assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous()
     part = torch.empty((splits, M, N), dtype=torch.float32, device=lhs.device)
-    rv = rhs.qval if fp8 else rhs
-    rc = _L.lyra_decode_gemm_partials(lhs.data_ptr(), rv.data_ptr(), _f32(rhs.scale).data_ptr() if fp8 else None, bk, bn,
-                                      group_sizes.data_ptr(), part.data_ptr(), part.numel() * 4, M, K, N,
-                                      _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _stream(lhs.device))
+    rc = _L.lyra_decode_gemm_partials(lhs.data_ptr(), rv.data_ptr(), _ptr(rs), bk, bn,
+                                      group_sizes.data_ptr(), part.data_ptr(), part.numel() * 4, M, K, N, rd, _stream(lhs.device))
     _lib.check(rc, "lyra_decode_gemm_partials")
     return Unsummed(part)
 
@@ -256,22 +326,15 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
          bias: torch.Tensor | None = None, bias_after_cast: bool = False) -> torch.Tensor:
     """lyra_decode_gemm_ex: the decode grouped matmul with an optional row gather on the input and an optional
     ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray.
+    A ``SpanMajor`` rhs (``pack_weights``) is read in that layout.
     ``bias`` [G, N] float32 is added to the float32 product (lyra/kernels/gemm.py:1600-1605), or with ``bias_after_cast``
     (one group, no SwiGLU) to the product rounded to bf16, in bf16, as a caller does that adds a bias to the operator's
     result (lyra/model.py:310-313, 367-368)."""
     dev = lhs.device
-    G, K, N = rhs.shape
+    rv, rs, bk, bn, rd, (G, K, N) = _rhs_args(rhs)
     M = rows if rows is not None else lhs.shape[0]
     assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
     assert group_sizes.dtype == torch.int32 and group_sizes.numel() == G
-    if isinstance(rhs, QArray):
-        bk, bn = rhs.block
-        rv, rs, rd = rhs.qval, _f32(rhs.scale), _lib.DTYPE_E4M3FN
-    else:
-        assert rhs.dtype == torch.bfloat16
-        bk = bn = 0
-        rv, rs, rd = rhs, None, _lib.DTYPE_BF16
-    assert rv.is_contiguous()
     NO = N // 2 if fused_swiglu else N
     out = torch.empty((M, NO), dtype=torch.float32 if out_f32 else torch.bfloat16, device=dev)
     if residual is not None:
@@ -289,6 +352,11 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
                                 out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
                                 _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
                                 float(swiglu_limit), stream)
+    if rc == _lib.E_UNSUPPORTED and isinstance(rhs, SpanMajor) and rhs.fallback is not None:
+        # (a shape whose plan has no span-major kernel, e.g. one group with too many rows for the K-split kernel)
+        return gemm(lhs, rhs.fallback, group_sizes, rows=rows, row_map=row_map, residual=residual, out_scale=out_scale,
+                    fused_swiglu=fused_swiglu, swiglu_beta=swiglu_beta, swiglu_limit=swiglu_limit, out_f32=out_f32, bias=bias,
+                    bias_after_cast=bias_after_cast)
     _lib.check(rc, "lyra_decode_gemm_ex")
     return out
 

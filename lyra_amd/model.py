@@ -494,10 +494,11 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
     B = x.shape[0]
     one = _one_group(B, x.device)
-    qkv = F.gemm_unsummed(h, w.qkv, one) if w.qkv_bias is None else None
+    w_qkv, w_out = F.span_major(w.qkv), F.span_major(w.out)  # (the arrays themselves unless their rows straddle cache lines)
+    qkv = F.gemm_unsummed(h, w_qkv, one) if w.qkv_bias is None else None
     if qkv is None:
         # (:310-313: a bias is added to the projection's bf16 result, in bf16 - inside the matmul's epilogue)
-        qkv = F.gemm(h, w.qkv, one, bias=_bf16_bias(w.qkv_bias), bias_after_cast=w.qkv_bias is not None)
+        qkv = F.gemm(h, w_qkv, one, bias=_bf16_bias(w.qkv_bias), bias_after_cast=w.qkv_bias is not None)
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     t = None
     if w.xsa_alpha is None and not _SEPARATE_QKV_POST:  # QK norm + RoPE + cache append inside the attention launch
@@ -513,10 +514,10 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
                  xsa_alpha=w.xsa_alpha).reshape(B, N * H)
     if w.out_bias is not None:  # :366-373: projection, + bias, * residual scale, + residual, each a bf16 result
-        return F.gemm(t, w.out, one, bias=_bf16_bias(w.out_bias), bias_after_cast=True, residual=x, out_scale=cfg.residual_scale), cache
-    out = F.gemm_unsummed(t, w.out, one)
+        return F.gemm(t, w_out, one, bias=_bf16_bias(w.out_bias), bias_after_cast=True, residual=x, out_scale=cfg.residual_scale), cache
+    out = F.gemm_unsummed(t, w_out, one)
     if out is None:
-        return F.gemm(t, w.out, one, residual=x, out_scale=cfg.residual_scale), cache
+        return F.gemm(t, w_out, one, residual=x, out_scale=cfg.residual_scale), cache
     out.residual, out.scale = x, cfg.residual_scale
     return out, cache
 
@@ -536,9 +537,9 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None 
     if groups_out is not None:
         groups_out.append(groups)
     G = cfg.n_experts
-    t = F.gemm(xn, w.mlp_up, groups, rows=B * topk, row_map=row_map, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta,
-               swiglu_limit=cfg.swiglu_limit, bias=_bf16_bias(w.mlp_up_bias, G))
-    t = F.gemm(t, w.mlp_down, groups, bias=_bf16_bias(w.mlp_down_bias, G))
+    t = F.gemm(xn, F.span_major(w.mlp_up, glu=True), groups, rows=B * topk, row_map=row_map, fused_swiglu=True,
+               swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, bias=_bf16_bias(w.mlp_up_bias, G))
+    t = F.gemm(t, F.span_major(w.mlp_down), groups, bias=_bf16_bias(w.mlp_down_bias, G))
     if topk <= 16 and not _SEPARATE_COMBINE:  # the combine step is left to the norm that follows (the next layer's, or the final one)
         return F.Uncombined(t, scores, dest, x, cfg.residual_scale)
     return F.moe_combine(t, scores, dest, x, cfg.residual_scale)
@@ -552,14 +553,15 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     else:
         t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
     one = _one_group(x.shape[0], x.device)
-    t = F.gemm(t, w.mlp_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
+    w_up, w_down = F.span_major(w.mlp_up), F.span_major(w.mlp_down)
+    t = F.gemm(t, w_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
                bias=_bf16_bias(w.mlp_up_bias))
     if w.mlp_down_bias is not None:  # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result
-        return F.gemm(t, w.mlp_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=True, residual=x,
+        return F.gemm(t, w_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=True, residual=x,
                       out_scale=cfg.dense_residual_scale)
-    down = F.gemm_unsummed(t, w.mlp_down, one)
+    down = F.gemm_unsummed(t, w_down, one)
     if down is None:
-        return F.gemm(t, w.mlp_down, one, residual=x, out_scale=cfg.dense_residual_scale)
+        return F.gemm(t, w_down, one, residual=x, out_scale=cfg.dense_residual_scale)
     down.residual, down.scale = x, cfg.dense_residual_scale
     return down
 

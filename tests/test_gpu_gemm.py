@@ -466,3 +466,128 @@ def test_widths_that_are_not_whole_spans(M, G, K, N, kind, block, swiglu, bias):
     U.assert_close(got, want, what=f"ragged width N={N}")
     got32 = _run(c, swiglu, out_f32=True)
     U.assert_close(got32, want, atol=4e-3, rtol=4e-3, what=f"ragged width N={N}, float32 out")
+
+
+# ---- span-major weights (lyra_gemm_pack) -------------------------------------------------------------------------------
+def _run_packed(c, swiglu, *, out_f32=False, bias=True, row_map=None, rows=None):
+    """The case's weights through lyra_gemm_pack and lyra_decode_gemm_ex (the host wrapper lyra_amd.kernels.decode_fused.gemm)."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray
+
+    if c["kind"] == "fp8":
+        q, s = c["w"]
+        rhs = QArray(U.t_fp8(q), U.t_f32(s), tuple(c["block"]))
+    else:
+        rhs = U.t_bf16(c["w"])
+    G = len(c["sizes"])
+    packed = F.pack_weights(rhs, glu=swiglu and G > 1)
+    gs = torch.from_numpy(c["sizes"]).to(U.dev())
+    b = None if (c["bias"] is None or not bias) else U.t_f32(c["bias"])
+    out = F.gemm(U.t_bf16(c["lhs"]), packed, gs, fused_swiglu=swiglu, out_f32=out_f32, bias=b)
+    torch.cuda.synchronize()
+    return U.to_np(out)
+
+
+def test_span_major_copy_is_the_documented_permutation():
+    """lyra_gemm_pack against the layout written in the header, for both layouts, both element sizes and widths that do
+    not fill their last span (zeros there)."""
+    from lyra_amd.kernels import decode_fused as F
+
+    rng = np.random.default_rng(5)
+    for (G, K, N) in ((3, 64, 256), (2, 32, 360), (1, 96, 2880), (2, 32, 5760), (1, 32, 16)):
+        for es in (1, 2):
+            w = rng.integers(1, 250, (G, K, N)).astype(np.uint8) if es == 1 else rng.integers(1, 60000, (G, K, N)).astype(np.uint16)
+            t = torch.from_numpy(w.view(np.int16) if es == 2 else w).to(U.dev())
+            t = t.view(torch.bfloat16) if es == 2 else t.view(torch.float8_e4m3fn)
+            for glu in (False, True):
+                if glu and N % 16:
+                    continue
+                if es == 1:
+                    from lyra_amd.nn.quant import QArray
+                    rhs = QArray(t, torch.ones(G, 1, N, device=U.dev()), (K, 1))
+                else:
+                    rhs = t
+                pk = F.pack_weights(rhs, glu=glu)
+                torch.cuda.synchronize()
+                got = pk.data.cpu().numpy().view(np.uint8 if es == 1 else np.uint16)
+                if glu:
+                    S, half = (N // 2 + 63) // 64, N // 2
+                    want = np.zeros((G, S, K, 128), w.dtype)
+                    for s_ in range(S):
+                        n = min(64, half - 64 * s_)
+                        want[:, s_, :, :n] = w[:, :, 64 * s_ : 64 * s_ + n]
+                        want[:, s_, :, 64 : 64 + n] = w[:, :, half + 64 * s_ : half + 64 * s_ + n]
+                else:
+                    S = (N + 127) // 128
+                    want = np.zeros((G, S, K, 128), w.dtype)
+                    for s_ in range(S):
+                        n = min(128, N - 128 * s_)
+                        want[:, s_, :, :n] = w[:, :, 128 * s_ : 128 * s_ + n]
+                assert got.size == want.size, (G, K, N, es, glu)
+                np.testing.assert_array_equal(got.reshape(want.shape), want, err_msg=f"G{G} K{K} N{N} es{es} glu{glu}")
+
+
+@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", "channel"), ("fp8", (64, 64))])
+@pytest.mark.parametrize("swiglu", [False, True])
+@pytest.mark.parametrize("M,G,K,N,sizes", [
+    (11, 4, 512, 512, [3, 0, 7, 1]),                    # fewer units than workgroups: units cut into K slices
+    (80, 4, 256, 1024, [70, 1, 0, 9]),                  # two row blocks in one group
+    (300, 16, 512, 4096, None),                         # several rounds of units (units of two spans), cost-ordered list
+    (260, 16, 256, 2048, None),                         # about two rounds of single spans
+    (200, 40, 64, 4096, None),                          # 40 row blocks: units of two spans also without SwiGLU
+    (300, 16, 64, 8192, None),                          # ... and with it (64 spans of 64 + 64 columns)
+    (40, 3, 320, 2880, [20, 0, 20]),                    # a width that fills no whole number of spans (22.5)
+    (7, 5, 64, 48, [2, 1, 0, 3, 1]),                    # narrower than one span, padding rows (sum < M is drawn below)
+])
+def test_span_major_weights_match_oracle_and_row_major_call(kind, block, swiglu, M, G, K, N, sizes):
+    """Every grouped-matmul case through the span-major copy: against the oracle at the acceptance bound, float32 output at
+    2e-3, and against the row-major call of the same kernel (same products; only the float32 summation order over K may
+    differ, so the two agree to a few float32 roundings)."""
+    if swiglu and N % 32:
+        N = N // 32 * 32
+    rng = np.random.default_rng(M + G + N)
+    if sizes is None:
+        cuts = np.sort(rng.integers(0, M + 1, G - 1))
+        sizes = np.diff(np.concatenate([[0], cuts, [M]])).tolist()
+        sizes[-1] = min(sizes[-1] + 0, 64 * 3)
+        sizes[0] = 64  # a full block first in lhs order, last in the kernel's list
+        M = int(sum(sizes)) + 3  # three rows past the last group
+    blk = (K, 1) if block == "channel" else block
+    if kind == "fp8" and blk is not None and (K % blk[0] or N % blk[1]):
+        pytest.skip("block does not tile the shape")
+    c = _case(7, M, G, K, N, sizes, kind=kind, block=blk, bias=True, w_std=0.05)
+    _note(f"span-major kind={kind} block={blk} swiglu={swiglu} M={M} G={G} K={K} N={N}")
+    want = _want(c, swiglu, big=G * K * N > (1 << 22))
+    got = _run_packed(c, swiglu)
+    U.assert_close(got, want, what="span-major bf16 out")
+    got32 = _run_packed(c, swiglu, out_f32=True)
+    U.assert_close(got32, want, atol=2e-3, rtol=2e-3, what="span-major f32 out")
+    plain32 = _run(c, swiglu, out_f32=True)
+    assert np.abs(got32 - plain32).max() <= 1e-4 * max(1.0, np.abs(plain32).max()), np.abs(got32 - plain32).max()
+
+
+def test_span_major_untouched_experts_are_never_read():
+    M, G, K, N = 6, 8, 512, 256
+    sizes = [0, 4, 0, 0, 2, 0, 0, 0]
+    c = _case(3, M, G, K, N, sizes, kind="fp8", block=(256, 256))
+    want = _want(c, True)
+    q, s = c["w"]
+    q, s = q.copy(), s.copy()
+    for g, n in enumerate(sizes):
+        if n == 0:
+            q[g] = 0x7F
+            s[g] = np.nan
+    U.assert_close(_run_packed(dict(c, w=(q, s)), True), want, what="poisoned idle experts, span-major")
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8"])
+@pytest.mark.parametrize("M,K,N,swiglu", [(64, 2048, 2048, False), (64, 2048, 6144, True), (33, 4096, 2880, False), (8, 2880, 5120, False)])
+def test_span_major_dense_projection_runs_split_over_k(kind, M, K, N, swiglu):
+    """One group: the K-split kernel reads layout 1 (also under a fused SwiGLU, which its finish step applies); bit-identical
+    to the row-major call, whose slices hold the same sums."""
+    block = (K, 1) if kind == "fp8" else None
+    c = _case(9, M, 1, K, N, [M], kind=kind, block=block, bias=False)
+    _note(f"span-major dense kind={kind} M={M} K={K} N={N} swiglu={swiglu}")
+    got = _run_packed(c, swiglu, out_f32=True)
+    np.testing.assert_array_equal(got, _run(c, swiglu, out_f32=True))
+    U.assert_close(got, _want(c, swiglu, big=True), atol=2e-3, rtol=2e-3, what="span-major dense")
