@@ -284,7 +284,7 @@ def kernel_table(dev, only="", span_major=False):
     gen = torch.Generator(device=dev)
     gen.manual_seed(1000)
 
-    def attention(label, B, N, K, H, S, sw, fp8, lengths=None):
+    def attention(label, B, N, K, H, S, sw, fp8, lengths=None, ranked=False):
         if only not in label:
             return
         es = 1 if fp8 else 2
@@ -311,12 +311,18 @@ def kernel_table(dev, only="", span_major=False):
         need = L.lyra_decode_attention_workspace(B, N, K, S, H, sw)
         ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
 
+        order = None
+        if ranked:  # the rows ranked by length once (lyra_attention_rank), as a decode step would do it for all its layers
+            order = torch.empty(B, dtype=torch.int32, device=dev)
+            _lib.check(L.lyra_attention_rank(pos.data_ptr(), B, order.data_ptr(), stream.cuda_stream), "lyra_attention_rank")
+
         def launch(i, hot=False):
             (k, v), (ks, vs) = caches[0 if hot else i % nbuf]
-            rc = L.lyra_decode_attention(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), ks.data_ptr() if fp8 else None, vs.data_ptr() if fp8 else None,
-                sinks.data_ptr(), pos.data_ptr(), stride, None, out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H,
-                H**-0.5, sw, _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_BF16, stream.cuda_stream)
+            head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), ks.data_ptr() if fp8 else None, vs.data_ptr() if fp8 else None,
+                    sinks.data_ptr(), pos.data_ptr(), stride)
+            tail = (None, out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, H**-0.5, sw,
+                    _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, _lib.DTYPE_BF16, stream.cuda_stream)
+            rc = L.lyra_decode_attention_ranked(*head, order.data_ptr(), *tail) if ranked else L.lyra_decode_attention(*head, *tail)
             _lib.check(rc, "lyra_decode_attention")
 
         nbytes = 2 * K * visible * (H * es + (4 if fp8 else 0))
@@ -386,7 +392,9 @@ def kernel_table(dev, only="", span_major=False):
     attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged 256..4096 global", 64, 64, 8, 64, 4096, 0, True, lengths)
     attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged sliding 128", 64, 64, 8, 64, 4096, 128, True, lengths)
     attention("gpt-oss shape B=64 64Q/8KV H=64 ctx 4096 fp8 global", 64, 64, 8, 64, 4096, 0, True)
+    attention("gpt-oss shape B=64 64Q/8KV H=64 fp8 ragged 256..4096 global, rows ranked once", 64, 64, 8, 64, 4096, 0, True, lengths, ranked=True)
     attention("lyra-medium B=64 fp8 ragged 256..4096 global", 64, 32, 8, 128, 4096, 0, True, lengths)
+    attention("lyra-medium B=64 fp8 ragged 256..4096 global, rows ranked once", 64, 32, 8, 128, 4096, 0, True, lengths, ranked=True)
     attention("lyra-medium B=64 ctx 4096 fp8 global, one position per row", 64, 32, 8, 128, 4096, 0, True, np.full(64, 4096))
     attention("lyra-max B=128 ctx 4096 fp8 global, one position per row", 128, 32, 8, 128, 4096, 0, True, np.full(128, 4096))
     for T in (1, 16, 64):

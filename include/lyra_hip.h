@@ -114,6 +114,24 @@ int lyra_decode_attention_qkv(const void* qkv, const float* partials, int splits
                               int out_dtype, lyra_stream_t stream);
 
 /*
+ * Ragged batches, rows dealt out by length (an extension of the boundary, like position_stride 1: the reference passes one
+ * position for the whole batch, lyra/kernels/decode_attention.py:364-375).  With more (row, kv head) pairs than compute
+ * units, which workgroup takes which pair decides how long a launch lasts.  The order of the rows by length changes
+ * only when the batch does - every row grows by one token per step - so it is computed once per step, or once per
+ * batch, by lyra_attention_rank and handed to every layer's launch:
+ *   lyra_attention_rank           row_order[i] = the row with the i-th largest position (ties: lower row first); B <= 8192
+ *   lyra_decode_attention_ranked  lyra_decode_attention with that order: the unchunked global-layer launch (position_stride 1,
+ *                                 more than 256 pairs) gives the workgroups that share a compute unit the i-th longest and
+ *                                 the i-th shortest pair; every other launch ignores the order.  row_order must be a
+ *                                 permutation of 0..B-1 (it is not checked); any permutation gives the same results.
+ */
+int lyra_attention_rank(const int32_t* position, int B, int32_t* row_order, lyra_stream_t stream);
+int lyra_decode_attention_ranked(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                 const float* sinks, const int32_t* position, int position_stride, const int32_t* row_order,
+                                 const void* gate, void* out, void* workspace, size_t workspace_bytes, int B, int N, int K, int S,
+                                 int H, float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream);
+
+/*
  * lyra_decode_attention for callers that cannot allocate device memory or hand over a workspace (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same arguments, same kernels and bit-identical results as lyra_decode_attention, minus the workspace: split partials

@@ -21,6 +21,11 @@ SIGNATURES = {
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_workspace": (_c.c_size_t, [_c.c_int] * 6),
+    "lyra_attention_rank": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p]),
+    "lyra_decode_attention_ranked": (
+        _c.c_int,
+        [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
     "lyra_decode_attention_xsa": (
         _c.c_int,
         [_c.c_void_p] * 7 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],

@@ -62,6 +62,9 @@ struct AttnParams {
     const float* sin_t;
     int rope_rows;
     float norm_eps;
+    // lyra_decode_attention_ranked: batch rows from longest to shortest ([B]), or null.  With it the unchunked launch deals
+    // its (row, kv head) pairs out so that the workgroups that share a compute unit hold a long and a short row.
+    const int32_t* row_order;
 };
 
 constexpr int kTile = 32;
@@ -503,8 +506,20 @@ void decode_attention_kernel(AttnParams p) {
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = lane & 15, kb = lane >> 4;
-    const int c_idx = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
+    const int c_idx = blockIdx.x;
+    int kh = blockIdx.y, b = blockIdx.z;
     const int G = p.G;
+    if (p.row_order) {
+        // Workgroups are started in the order of their linear index (kv head fastest), 256 at a time, one per compute
+        // unit: workgroup L of a round shares its unit with workgroup L of the next.  Pairs are ranked by length (row
+        // order[r / K], kv head r % K); even rounds take them from the front of their stretch, odd rounds from the back.
+        const int L = (int)blockIdx.z * p.K + (int)blockIdx.y, n_pairs = p.B * p.K;
+        const int round = L >> 8, i = L & 255;
+        const int last = min(n_pairs, (round + 1) << 8) - 1;  // (last rank of this round's stretch)
+        const int r = (round & 1) ? last - i : (round << 8) + i;
+        kh = r % p.K;
+        b = __builtin_amdgcn_readfirstlane(p.row_order[r / p.K]);
+    }
 
     // The position first: loads return in the order they were issued, so requested behind the cache tiles and the
     // projection slices it would arrive last, and everything that follows from it (rotary row, window, the owner of the
@@ -1143,7 +1158,8 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
                          const float* sinks, const int32_t* position, int position_stride, const void* gate, void* out,
                          void* workspace, size_t workspace_bytes, int too_small, bool clear_counters, const void* xsa_v,
                          const float* xsa_alpha, int B, int N, int K, int S, int H, float sm_scale, int sliding_window,
-                         int kv_dtype, int out_dtype, lyra_stream_t stream, const QkvFront* front = nullptr) {
+                         int kv_dtype, int out_dtype, lyra_stream_t stream, const QkvFront* front = nullptr,
+                         const int32_t* row_order = nullptr) {
     if ((!q && !front) || !k || !v || !sinks || !position || !out) return LYRA_E_BADARG;
     if (front) {
         if ((front->partials ? front->splits <= 0 : !front->qkv) || !front->cos_t || !front->sin_t || front->rope_rows <= 0)
@@ -1165,8 +1181,16 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     if ((H != 64 && H != 128) || G > 16) return LYRA_E_UNSUPPORTED;
     if (K > 65535 || B > 65535) return LYRA_E_UNSUPPORTED;
 
-    const AttnPlan pl = plan_attention(B, K, S, sliding_window);
+    AttnPlan pl = plan_attention(B, K, S, sliding_window);
+    // ranked rows: only the unchunked global-layer launch with one position per row and more pairs than compute units deals
+    // pairs out by length; every other launch ignores the order
+    const bool ranked = row_order && position_stride == 1 && sliding_window == 0 && pl.n_chunks == 1 && (long)B * K > 256 && !front;
+    if (ranked) {
+        static const long ranked_waves_env = env_long("LYRA_ATTN_RANKED_WAVES");  // tuning override, read once
+        pl.waves = (ranked_waves_env == 4 || ranked_waves_env == 8) ? (int)ranked_waves_env : (H == 64 ? 8 : 4);
+    }
     AttnParams p;
+    p.row_order = ranked ? row_order : nullptr;
     p.q = (const uint16_t*)q;
     p.k = (const uint8_t*)k;
     p.v = (const uint8_t*)v;
@@ -1239,7 +1263,7 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     static const char* rows_env = getenv("LYRA_ATTN_ROWS");
     static const long rows_mode = rows_env ? atol(rows_env) : 1;
     static const long rows_waves_env = env_long("LYRA_ATTN_ROWS_WAVES");
-    const bool rows = rows_mode > 0 && (position_stride == 1 || rows_mode > 1) && sliding_window == 0 && pl.n_chunks == 1 &&
+    const bool rows = !ranked && rows_mode > 0 && (position_stride == 1 || rows_mode > 1) && sliding_window == 0 && pl.n_chunks == 1 &&
                       (long)B * K > 256 && B <= kMaxRankedRows;
     // the front step exists in the chunked kernel with 4 wavefronts only; the caller takes the two launches otherwise
     if (front && (rows || pl.waves != 4)) return LYRA_E_UNSUPPORTED;
@@ -1352,6 +1376,44 @@ extern "C" int lyra_decode_attention(const void* q, const void* k, const void* v
     return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes,
                                LYRA_E_WORKSPACE, false, nullptr, nullptr, B, N, K, S, H, sm_scale, sliding_window, kv_dtype,
                                out_dtype, stream);
+}
+
+namespace lyra {
+// rank[i] = the row with the i-th largest position (ties: the lower row first); one workgroup, thread t places row t
+__global__ __launch_bounds__(1024) void attention_rank_kernel(const int32_t* position, int B, int32_t* order) {
+    extern __shared__ int sm_rank_pos[];
+    for (int i = threadIdx.x; i < B; i += blockDim.x) sm_rank_pos[i] = position[i];
+    __syncthreads();
+    for (int t = threadIdx.x; t < B; t += blockDim.x) {
+        const int mine = sm_rank_pos[t];
+        int rank = 0;
+        for (int j = 0; j < B; ++j) {
+            const int other = sm_rank_pos[j];
+            rank += (other > mine) || (other == mine && j < t);
+        }
+        order[rank] = t;
+    }
+}
+}  // namespace lyra
+
+extern "C" int lyra_attention_rank(const int32_t* position, int B, int32_t* row_order, lyra_stream_t stream) {
+    if (!position || !row_order || B <= 0) return LYRA_E_BADARG;
+    if (B > 8192) return LYRA_E_UNSUPPORTED;
+    const int threads = std::min(1024, (B + 63) / 64 * 64);
+    hipLaunchKernelGGL(lyra::attention_rank_kernel, dim3(1), dim3(threads), (size_t)B * sizeof(int), (hipStream_t)stream, position, B,
+                       row_order);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" int lyra_decode_attention_ranked(const void* q, const void* k, const void* v, const float* k_scale,
+                                            const float* v_scale, const float* sinks, const int32_t* position,
+                                            int position_stride, const int32_t* row_order, const void* gate, void* out,
+                                            void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
+                                            float sm_scale, int sliding_window, int kv_dtype, int out_dtype, lyra_stream_t stream) {
+    if (!row_order) return LYRA_E_BADARG;
+    return lyra::run_attention(q, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes,
+                               LYRA_E_WORKSPACE, false, nullptr, nullptr, B, N, K, S, H, sm_scale, sliding_window, kv_dtype,
+                               out_dtype, stream, nullptr, row_order);
 }
 
 extern "C" int lyra_decode_attention_xsa(const void* q, const void* k, const void* v, const float* k_scale,

@@ -84,8 +84,19 @@ def _position_vector(position, batch: int, device) -> tuple[torch.Tensor, int]:
     return pos.reshape(batch).contiguous(), 1
 
 
+def rank_rows(position: torch.Tensor) -> torch.Tensor:
+    """lyra_attention_rank: the batch rows from the longest to the shortest (int32 [B], ties to the lower row) for a [B]
+    int32 device tensor of positions.  The order only changes when the batch does (every row grows by one token per step):
+    compute it once per step or per batch and hand it to every layer's ``decode_attention(..., row_order=...)``."""
+    pos = position.to(torch.int32).reshape(-1).contiguous()
+    order = torch.empty_like(pos)
+    rc = _lib.lib.lyra_attention_rank(pos.data_ptr(), pos.numel(), order.data_ptr(), torch.cuda.current_stream(pos.device).cuda_stream)
+    _lib.check(rc, "lyra_attention_rank")
+    return order
+
+
 def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config: DecodeAttentionConfig, dtype, gate=None,
-                      xsa_v=None, xsa_alpha=None):
+                      xsa_v=None, xsa_alpha=None, row_order=None):
     """Launch the HIP kernel (the counterpart of decode_attention.py:150-260)."""
     B, N, T, H = q.shape
     if T != 1:
@@ -132,6 +143,9 @@ def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config
             vn = xsa_v.to(device=dev, dtype=torch.bfloat16).reshape(B, K, H).contiguous()
             alpha = xsa_alpha.to(device=dev, dtype=torch.float32).reshape(N).contiguous()
             rc = _lib.lib.lyra_decode_attention_xsa(*head, vn.data_ptr(), alpha.data_ptr(), *tail)
+        elif row_order is not None:
+            order = row_order.to(device=dev, dtype=torch.int32).reshape(B).contiguous()
+            rc = _lib.lib.lyra_decode_attention_ranked(*head[:8], order.data_ptr(), head[8], *tail)
         else:
             rc = _lib.lib.lyra_decode_attention(*head, *tail)
     _lib.check(rc, "lyra_decode_attention")
@@ -221,8 +235,12 @@ def decode_attention(
     gate: torch.Tensor | None = None,
     xsa_v: torch.Tensor | None = None,
     xsa_alpha: torch.Tensor | None = None,
+    row_order: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """q [B,N,1,H]; k, v [B,K,S,H] tensors or QArray (e4m3fn, block (1,H)); sinks [N]; returns [B,N,1,H].
+
+    ``row_order`` (``rank_rows(position)``; ragged batches only): lets the kernel deal the rows out by length instead of
+    ranking them in every launch.  It changes which workgroup computes which row, never a result.
 
     ``xsa_v`` [B,K,H] (the new token's value rows at unit length) with ``xsa_alpha`` [N] fuses the learned exclusive
     self attention of lyra/model.py:351-363 behind the gate; both default to None (the reference operator).
@@ -255,7 +273,7 @@ def decode_attention(
     def kernel():
         assert config is not None
         return _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config, dtype, gate=gate,
-                                 xsa_v=xsa_v, xsa_alpha=xsa_alpha)
+                                 xsa_v=xsa_v, xsa_alpha=xsa_alpha, row_order=row_order)
 
     tiling = None if config is None else f"kv{config.tile_kv} buf{config.kv_buffer_count} {'fp8' if config.cache_dtype else 'bf16'}"
     op_shape = f"b{B} n{N} k{K} s{S} h{H} sw{sliding_window}"

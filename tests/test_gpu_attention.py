@@ -17,16 +17,18 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-def _run(case, sm_scale, sw, pos, *, dtype=torch.bfloat16, gate=None, implementation="pallas", xsa_v=None, xsa_alpha=None):
-    from lyra_amd.kernels.decode_attention import decode_attention
+def _run(case, sm_scale, sw, pos, *, dtype=torch.bfloat16, gate=None, implementation="pallas", xsa_v=None, xsa_alpha=None,
+         ranked=False):
+    from lyra_amd.kernels.decode_attention import decode_attention, rank_rows
 
     q, k, v, sinks = U.attention_torch_inputs(case)
     p = pos if np.ndim(pos) == 0 else torch.from_numpy(np.asarray(pos, dtype=np.int32)).to(U.dev())
     g = None if gate is None else U.t_bf16(gate)
     xv = None if xsa_v is None else U.t_bf16(xsa_v)
     xa = None if xsa_alpha is None else U.t_f32(xsa_alpha)
+    order = rank_rows(p) if ranked else None
     out = decode_attention(q, k, v, sinks, sm_scale, sw, p, dtype=dtype, implementation=implementation, gate=g, xsa_v=xv,
-                           xsa_alpha=xa)
+                           xsa_alpha=xa, row_order=order)
     torch.cuda.synchronize()
     return U.to_np(out)
 
@@ -295,6 +297,50 @@ def test_ragged_rows_longest_first_launch(fp8, H, N, K, B):
     got_g = _run(case, H**-0.5, 0, pos, gate=gate)
     want_g = want * gate[:, :, None, None]
     U.assert_close(got_g, want_g, what="ragged + gate")
+
+
+def test_rank_rows_is_the_stable_descending_order():
+    from lyra_amd.kernels.decode_attention import rank_rows
+
+    rng = np.random.default_rng(9)
+    for B in (1, 2, 63, 64, 65, 300, 1025, 4000):
+        pos = rng.integers(-1, 50, B).astype(np.int32)  # many ties
+        got = rank_rows(torch.from_numpy(pos).to(U.dev())).cpu().numpy()
+        want = np.argsort(-pos.astype(np.int64), kind="stable").astype(np.int32)
+        np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("fp8,H,N,K,B", [(True, 64, 16, 8, 37), (False, 128, 8, 4, 70), (True, 128, 4, 2, 200), (True, 64, 2, 1, 300),
+                                         (True, 64, 64, 8, 64), (True, 128, 32, 8, 64)])
+def test_ragged_rows_dealt_out_by_a_given_order(fp8, H, N, K, B):
+    """lyra_decode_attention_ranked: the same cases as the launch that ranks the rows itself, with the order computed
+    beforehand; any permutation must give the same output bit for bit (it only changes which workgroup takes which row),
+    and a launch the order does not apply to (a window, few pairs) ignores it."""
+    from lyra_amd.kernels.decode_attention import decode_attention
+
+    S = 384
+    case = U.attention_case(4100 + B, B, N, K, S, H, fp8=fp8)
+    rng = np.random.default_rng(B + 1)
+    pos = rng.integers(0, S, B).astype(np.int32)
+    pos[: B // 4] = pos[B // 2 : B // 2 + B // 4]
+    pos[1], pos[B - 1], pos[B // 3] = -1, S - 1, S - 1
+    gate = O.bf16_round((2.0 / (1.0 + np.exp(-rng.standard_normal((B, N))))).astype(np.float32))
+    _note(f"attn ranked fp8={fp8} H={H} N={N} K={K} B={B}")
+    want = O.decode_attention_reference(case["q"], case["k"], case["v"], case["sinks"], H**-0.5, 0, pos)
+    got = _run(case, H**-0.5, 0, pos, ranked=True)
+    U.assert_close(got, want, what="ranked")
+    assert np.all(got[1] == 0)
+    U.assert_close(_run(case, H**-0.5, 0, pos, gate=gate, ranked=True), want * gate[:, :, None, None], what="ranked + gate")
+    got32 = _run(case, H**-0.5, 0, pos, dtype=torch.float32, ranked=True)
+    U.assert_close(got32, want, atol=4e-3, rtol=4e-3, what="ranked f32")
+    # any other permutation: identical bits
+    q, k, v, sinks = U.attention_torch_inputs(case)
+    p = torch.from_numpy(pos).to(U.dev())
+    perm = torch.from_numpy(rng.permutation(B).astype(np.int32)).to(U.dev())
+    other = decode_attention(q, k, v, sinks, H**-0.5, 0, p, implementation="pallas", row_order=perm)
+    np.testing.assert_array_equal(U.to_np(other), got)
+    # a window: the order is ignored, the result is the plain launch's
+    np.testing.assert_array_equal(_run(case, H**-0.5, 128, pos, ranked=True), _run(case, H**-0.5, 128, pos))
 
 
 def test_ragged_launch_replays_in_a_hip_graph():
