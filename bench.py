@@ -30,7 +30,8 @@ def attention_algorithmic_bytes(batch, kv_heads, visible, head_dim, fp8=True):
     return 2 * batch * kv_heads * visible * per_row
 
 
-def build_model(batch, ctx, device, variant="lyra-small", layout="headline"):
+def build_model(batch, ctx, device, variant="lyra-small", layout="headline", weights=None):
+    """Random-init weights of the variant (or ``weights``, to run them at another batch) and caches with a synthetic history."""
     import torch
 
     from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights
@@ -40,7 +41,7 @@ def build_model(batch, ctx, device, variant="lyra-small", layout="headline"):
         cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True)
     else:
         cfg = apply_inference_overrides(MODEL_VARIANTS[variant], fp8=True, fp8_attn=True, per_channel=True)
-    weights = init_weights(cfg, device)
+    weights = init_weights(cfg, device) if weights is None else weights
     cache = init_cache(cfg, batch, ctx, device)
     g = torch.Generator(device=device)
     g.manual_seed(1002)
@@ -55,15 +56,17 @@ def build_model(batch, ctx, device, variant="lyra-small", layout="headline"):
     return cfg, weights, cache
 
 
-def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup):
-    """Wall time of `steps` replays of the captured decode step; also returns the function that runs one more step."""
+def time_decode_steps(cfg, weights, cache, batch, ctx, steps, warmup, greedy=False):
+    """Wall time of `steps` replays of the captured decode step; also returns the function that runs one more step.
+    ``greedy`` False: the reference's default sampler (temperature 0.8, top-k 4: lyra/model.py:107-108, generate.py:46-53)
+    through lyra_sample_topk, the uniform numbers drawn inside the captured step; True: arg-max through lyra_argmax."""
     import torch
 
     from lyra_amd.generate import GraphedDecoder
 
     # every timed step runs at full context: the captured step does not move the position (ctx - 1, the last cache row);
     # each step decodes the tokens the step before it drew
-    dec = GraphedDecoder(weights, cache, cfg, batch, advance=False)
+    dec = GraphedDecoder(weights, cache, cfg, batch, greedy=greedy, advance=False)
     dec.tokens.copy_(torch.randint(0, cfg.vocab_size, (batch,), device=dec.tokens.device).to(torch.int32))
     one_step = dec.step
 
@@ -138,6 +141,103 @@ def time_dominant_kernel(cfg, weights, cache, batch, ctx, one_step, rounds=13, f
             pairs.append((start, stop))
     stream.synchronize()
     return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / (len(pairs) * len(layers))  # seconds per launch
+
+
+def time_attention_sustained(cfg, weights, cache, batch, ctx, launches=104, warm=16):
+    """The launch of `time_dominant_kernel(front=True)` (or the plain one when the step does not use the front step) back
+    to back: `launches` launches in one HIP-event bracket, rotating over the caches of the model's global layers (8 x 277 MB
+    at the headline shape: every launch streams from HBM).  Under this sustained load the device reaches its power limit
+    within milliseconds, which the groups of 8 between step replays do not."""
+    import torch
+
+    from lyra_amd import _lib
+
+    dev = weights.emb.device
+    L = _lib.lib
+    N, K, H = cfg.n_attn_heads, cfg.n_kv_heads, cfg.head_dim
+    q = torch.randn(batch, N, H, device=dev, dtype=torch.bfloat16)
+    out = torch.empty_like(q)
+    pos = torch.full((1,), ctx - 1, dtype=torch.int32, device=dev)
+    layers = [c for i, c in enumerate(cache.layers) if i % 2 == 1]
+    sinks = weights.layers[1].attn.sinks
+    ws = torch.zeros(max(L.lyra_decode_attention_workspace(batch, N, K, ctx, H, 0), 256), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def launch(i):
+        c = layers[i % len(layers)]
+        rc = L.lyra_decode_attention(
+            q.data_ptr(), c.k.qval.data_ptr(), c.v.qval.data_ptr(), c.k.scale.data_ptr(), c.v.scale.data_ptr(), sinks.data_ptr(),
+            pos.data_ptr(), 0, None, out.data_ptr(), ws.data_ptr(), ws.numel(), batch, N, K, ctx, H, H**-0.5, 0,
+            _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, stream.cuda_stream)
+        _lib.check(rc, "lyra_decode_attention")
+
+    return _time_launches(launch, stream, warm=warm, iters=launches), launches
+
+
+def time_attention_ragged(dev, one_step, stream, rounds=10):
+    """Benchmark configuration 4: gpt-oss attention shape (64 query / 8 kv heads of width 64), B=64, cache 4096, FP8, one
+    length per row drawn uniformly from [256, 4096] (seeded), global layer, the rows ranked once by lyra_attention_rank as a
+    decode step would do for all its layers.  Timed like the other stand-alone launches: groups (one launch per cache set,
+    3 sets) between replays of the decode step."""
+    import numpy as np
+    import torch
+
+    from lyra_amd import _lib
+
+    L = _lib.lib
+    B, N, K, H, S = 64, 64, 8, 64, 4096
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1004)
+    lengths = np.random.default_rng(1004).integers(256, 4097, size=B)
+    sets = []
+    for _ in range(3):
+        kv = [torch.randint(0, 0x78, (B, K, S, H), generator=gen, device=dev, dtype=torch.uint8) for _ in range(2)]
+        sc = [torch.rand(B, K, S, generator=gen, device=dev) * 0.004 + 0.006 for _ in range(2)]
+        sets.append((kv, sc))
+    q = torch.randn(B, N, H, generator=gen, device=dev, dtype=torch.bfloat16)
+    out = torch.empty_like(q)
+    sinks = torch.randn(N, generator=gen, device=dev)
+    pos = torch.from_numpy(lengths.astype(np.int32) - 1).to(dev)
+    order = torch.empty(B, dtype=torch.int32, device=dev)
+    _lib.check(L.lyra_attention_rank(pos.data_ptr(), B, order.data_ptr(), stream.cuda_stream), "lyra_attention_rank")
+    ws = torch.zeros(max(L.lyra_decode_attention_workspace(B, N, K, S, H, 0), 256), dtype=torch.uint8, device=dev)
+
+    def launch(kv, sc):
+        rc = L.lyra_decode_attention_ranked(
+            q.data_ptr(), kv[0].data_ptr(), kv[1].data_ptr(), sc[0].data_ptr(), sc[1].data_ptr(), sinks.data_ptr(), pos.data_ptr(), 1,
+            order.data_ptr(), None, out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, H**-0.5, 0, _lib.DTYPE_E4M3FN,
+            _lib.DTYPE_BF16, stream.cuda_stream)
+        _lib.check(rc, "lyra_decode_attention_ranked")
+
+    pairs = []
+    for r in range(rounds + 2):
+        one_step()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for kv, sc in sets:
+            launch(kv, sc)
+        b.record(stream)
+        if r >= 2:
+            pairs.append((a, b))
+    stream.synchronize()
+    t = sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / (len(pairs) * len(sets))
+    nbytes = int(2 * K * lengths.sum() * (H + 4))
+    return {"kernel": "decode_attention_kernel<64, fp8, 8 wavefronts> (rows dealt out by lyra_attention_rank's order)",
+            "case": "gpt-oss attention shape, B=64, 64Q/8KV, H=64, cache 4096, lengths U[256, 4096] (seed 1004), global layer",
+            "bound": "hbm", "achieved": nbytes / t / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
+            "algorithmic_bytes": nbytes, "us_per_launch": t * 1e6}
+
+
+def source_fingerprint():
+    """Hash of the attention kernel's sources: hardware-counter figures kept in profiles/ are only quoted for the sources
+    they were collected on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for rel in ("lyra_amd/csrc/decode_attention.hip", "lyra_amd/csrc/lyra_device.h"):
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def _nbytes(w):
@@ -495,13 +595,16 @@ def cpu_baseline(cfg, weights, cache, ctx, sample_batch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-gemm-roofline", action="store_true", help="skip the stand-alone expert matmul timings")
+    ap.add_argument("--no-gemm-roofline", action="store_true", help="skip the stand-alone expert matmul and extra attention timings")
+    ap.add_argument("--no-variants", action="store_true", help="skip the step under other settings (other sampler, B=8, reference-fp8 layout)")
+    ap.add_argument("--sampler", default="default", choices=["default", "greedy"],
+                    help="default: temperature 0.8 over the top 4, the reference's setting (lyra/model.py:107-108); greedy: arg-max")
     ap.add_argument("--layout", default="headline", choices=["headline", "reference-fp8"],
                     help="headline: FP8 cache, every projection and MLP weight FP8 with one scale per output channel; "
                          "reference-fp8: FP8 cache and MLP weights with (256, 256) scale blocks, attention projections bf16")
@@ -530,32 +633,54 @@ def main():
                   f"{100 * r['cold_frac_of_peak']:.1f} | {r['hot_us']:.1f} |", file=sys.stderr)
         print(json.dumps({"metric": "operator launch time at model shapes", "unit": "us", "peak_GBs": HBM_PEAK_GBS, "kernels": rows}))
         return
+    greedy = args.sampler == "greedy"
     cfg, weights, cache = build_model(args.batch, args.ctx, dev, args.model, args.layout)
-    elapsed, one_step = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup)
+    elapsed, one_step = time_decode_steps(cfg, weights, cache, args.batch, args.ctx, args.steps, args.warmup, greedy=greedy)
     tokens_per_s = args.batch * args.steps / elapsed
 
-    # what the step's own routing touches (one eager step; the graph replays the same kernels on the same inputs)
-    groups = []
     from lyra_amd.model import model_apply
 
-    cache.pos.fill_(args.ctx - 1)
-    model_apply(torch.arange(args.batch, device=dev) % cfg.vocab_size, weights, cache, cfg, groups_out=groups, advance=False)
-    touched = [int((g > 0).sum().item()) for g in groups]
-    step_bytes = step_algorithmic_bytes(cfg, weights, args.batch, args.ctx, touched)
+    def algorithmic_bytes(cfg_, weights_, cache_, batch):
+        """(bytes one step must move, experts with rows per MoE layer), from the step's own routing: one eager step (the
+        graph replays the same kernels on the same inputs)."""
+        groups = []
+        cache_.pos.fill_(args.ctx - 1)
+        model_apply(torch.arange(batch, device=dev) % cfg_.vocab_size, weights_, cache_, cfg_, groups_out=groups, advance=False)
+        touched_ = [int((g > 0).sum().item()) for g in groups]
+        return step_algorithmic_bytes(cfg_, weights_, batch, args.ctx, touched_), touched_
+
+    step_bytes, touched = algorithmic_bytes(cfg, weights, cache, args.batch)
 
     t_attn = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step)
     t_attn_front = None
     if weights.layers[1].attn.xsa_alpha is None and args.batch * cfg.n_kv_heads <= 256:  # the launch the step itself uses
         t_attn_front = time_dominant_kernel(cfg, weights, cache, args.batch, args.ctx, one_step, front=True)
-    gemm_rows = time_expert_matmuls(dev, one_step, torch.cuda.current_stream(dev)) if not args.no_gemm_roofline else None
+    stream = torch.cuda.current_stream(dev)
+    gemm_rows = time_expert_matmuls(dev, one_step, stream) if not args.no_gemm_roofline else None
     attn_bytes = attention_algorithmic_bytes(args.batch, cfg.n_kv_heads, args.ctx, cfg.head_dim, fp8=True)
-    achieved = attn_bytes / t_attn / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "decode_attention_traffic.json")
-    if os.path.exists(tpath) and (args.model, args.batch, args.ctx) == ("lyra-small", 64, 4096):
-        with open(tpath) as f:  # counters were collected for the headline launch only
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+    headline_shape = (args.model, args.batch, args.ctx) == ("lyra-small", 64, 4096)
 
+    # HBM traffic per launch from hardware counters: collected in separate rocprofv3 --pmc runs and kept in profiles/; quoted
+    # only while the kernel's sources are the ones the counters were collected on
+    traffic, traffic_plain, traffic_note = None, None, "no counters file"
+    tpath = os.path.join(ROOT, "profiles", "decode_attention_traffic.json")
+    if os.path.exists(tpath) and headline_shape:
+        with open(tpath) as f:
+            tj = json.load(f)
+        if tj.get("source_sha256_16") == source_fingerprint():
+            traffic, traffic_plain = tj.get("hbm_bytes_per_launch_front_step"), tj.get("hbm_bytes_per_launch")
+            traffic_note = f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {tpath[len(ROOT) + 1:]} (sources {tj['source_sha256_16']})"
+        else:
+            traffic_note = "the counters in profiles/decode_attention_traffic.json were collected on other kernel sources: not quoted"
+
+    plain = {
+        "kernel": "decode_attention_kernel<128, fp8> (global layer; the operator on its own, lyra_decode_attention)",
+        "us_per_launch": t_attn * 1e6,
+        "achieved": attn_bytes / t_attn / 1e9,
+        "frac": attn_bytes / t_attn / 1e9 / HBM_PEAK_GBS,
+        "traffic": traffic_plain,
+    }
+    t_main = t_attn_front if t_attn_front is not None else t_attn
     result = {
         "metric": "decode tokens/s at B=64 ctx 4096 FP8 cache; achieved HBM GB/s (% peak)",
         "value": tokens_per_s,
@@ -573,7 +698,8 @@ def main():
             "workload": f"full {args.model} decode step ({cfg.n_layers} layers, {cfg.n_attn_heads}Q/{cfg.n_kv_heads}KV heads, "
                         f"H={cfg.head_dim}, {cfg.n_routed_experts}+{cfg.n_shared_experts} experts, LM head {cfg.padded_vocab_size}), "
                         f"B={args.batch}, ctx {args.ctx}, FP8 KV cache, " + ("FP8 per-output-channel weights" if args.layout == "headline" else
-                        "FP8 MLP weights with (256, 256) scale blocks, bf16 attention projections") + ", greedy sampling",
+                        "FP8 MLP weights with (256, 256) scale blocks, bf16 attention projections") +
+                        (", greedy sampling" if greedy else f", sampling at temperature {cfg.sample_temperature} over the top {cfg.sample_topk} (the reference's default)"),
             "batch": args.batch,
             "ctx": args.ctx,
             "us_per_layer": elapsed / args.steps / cfg.n_layers * 1e6,
@@ -584,30 +710,59 @@ def main():
                             if args.layout == "headline" else "q/k/v and output projections bf16, as the reference's --fp8 leaves them"),
         },
         "roofline": {
-            "kernel": "decode_attention_kernel<128, fp8> (global layer)",
+            # the launch the decode step runs: with the step in front of the attention (QK norm, rotary embedding, cache
+            # append) fused in when the model allows it; timed in groups of one launch per global layer between step replays
+            "kernel": ("decode_attention_kernel<128, fp8, QK norm + RoPE + cache append> (global layer; the launch of the decode step, "
+                       "lyra_decode_attention_qkv)" if t_attn_front is not None else plain["kernel"]),
             "bound": "hbm",
-            "achieved": achieved,
+            "achieved": attn_bytes / t_main / 1e9,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": traffic,
+            "frac": attn_bytes / t_main / 1e9 / HBM_PEAK_GBS,
+            "traffic": traffic if t_attn_front is not None else traffic_plain,
+            "traffic_source": traffic_note,
             "algorithmic_bytes": attn_bytes,
-            "us_per_launch": t_attn * 1e6,
+            "us_per_launch": t_main * 1e6,
+            "timing": "HIP events around groups of 8 launches (one per global layer's cache) between replays of the decode step",
         },
     }
     if t_attn_front is not None:
-        # the same launch with the step in front of it fused in (what the decode step runs): same cache bytes, more to do
-        result["roofline"]["with_front_step"] = {
-            "kernel": "decode_attention_kernel<128, fp8, QK norm + RoPE + cache append> (global layer)",
-            "us_per_launch": t_attn_front * 1e6,
-            "achieved": attn_bytes / t_attn_front / 1e9,
-            "frac": attn_bytes / t_attn_front / 1e9 / HBM_PEAK_GBS,
-        }
+        result["roofline"]["attention_operator"] = plain
+    if not args.no_gemm_roofline:
+        t_sus, n_sus = time_attention_sustained(cfg, weights, cache, args.batch, args.ctx)
+        result["roofline"]["attention_sustained"] = {
+            "kernel": plain["kernel"], "launches_back_to_back": n_sus, "us_per_launch": t_sus * 1e6,
+            "achieved": attn_bytes / t_sus / 1e9, "frac": attn_bytes / t_sus / 1e9 / HBM_PEAK_GBS,
+            "note": "one HIP-event bracket around all launches, rotating over the global layers' caches (every launch from HBM)"}
+        result["roofline"]["attention_ragged"] = time_attention_ragged(dev, one_step, stream)
     if gemm_rows is not None:
         result["roofline"]["gemm"] = gemm_rows
+    if not args.no_variants and headline_shape and args.layout == "headline":
+        # the same step under the other settings a reader may ask for; each is its own captured graph, timed like the headline
+        variants = []
+
+        def timed(name, cfg_, weights_, cache_, batch, greedy_):
+            el, _ = time_decode_steps(cfg_, weights_, cache_, batch, args.ctx, args.steps, args.warmup, greedy=greedy_)
+            nbytes, _ = algorithmic_bytes(cfg_, weights_, cache_, batch)
+            variants.append({"variant": name, "batch": batch, "ms_per_step": el / args.steps * 1e3, "tokens_per_s": batch * args.steps / el,
+                             "step_algorithmic_bytes": nbytes, "step_frac": nbytes / (el / args.steps) / 1e9 / HBM_PEAK_GBS})
+
+        timed("greedy sampling (arg-max)" if not greedy else "sampling at temperature 0.8 over the top 4", cfg, weights, cache, args.batch, not greedy)
+        cfg8, _, cache8 = build_model(8, args.ctx, dev, args.model, args.layout, weights=weights)
+        timed("B=8 (benchmark configuration 2)", cfg8, weights, cache8, 8, greedy)
+        del cache8
+        if not args.no_cpu_baseline:  # (the CPU baseline reads the headline model: take it before the model is replaced)
+            result["cpu_baseline"] = cpu_baseline(cfg, weights, cache, args.ctx, min(args.cpu_sample, args.batch))
+        del weights, cache, one_step
+        torch.cuda.empty_cache()
+        cfg_r, weights_r, cache_r = build_model(args.batch, args.ctx, dev, args.model, "reference-fp8")
+        timed("layout reference-fp8 (what the reference's --fp8 sets: FP8 MLP weights with (256, 256) scale blocks and an FP8 cache, "
+              "bf16 attention projections)", cfg_r, weights_r, cache_r, args.batch, greedy)
+        result["variants"] = variants
+        weights = cache = None
     if args.traffic_probe:
         result["traffic_probe"] = traffic_probe(dev)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and "cpu_baseline" not in result:
         result["cpu_baseline"] = cpu_baseline(cfg, weights, cache, args.ctx, min(args.cpu_sample, args.batch))
     print(json.dumps(result))
 

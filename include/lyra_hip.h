@@ -343,6 +343,16 @@ size_t lyra_argmax_workspace(int rows, int cols);
 int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
                      int cols, int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream);
 size_t lyra_sample_topk_workspace(int rows, int cols, int k);
+/*
+ * The same draw with the uniform numbers made inside the launch, so that a captured decode step needs no generator
+ * launches of its own: rng is a device array of two uint64, {seed, count}; row r takes
+ *   u = (splitmix64(seed ^ (count + 1) * 0x9E3779B97F4A7C15 ^ (r + 1) * 0xD1B54A32D192ED03) >> 40) * 2^-24
+ * (splitmix64(z): z = (z ^ z >> 30) * 0xBF58476D1CE4E5B9; z = (z ^ z >> 27) * 0x94D049BB133111EB; z ^ z >> 31), and the
+ * launch leaves count + 1 behind once every workgroup has read count.  Like the reference's key stream
+ * (lyra/generate.py:53, jax.random.categorical) this is a stream of its own: same distribution, other numbers.
+ */
+int lyra_sample_topk_rng(const float* x, uint64_t* rng, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols,
+                         int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream);
 
 
 /*

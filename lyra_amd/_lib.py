@@ -84,6 +84,7 @@ SIGNATURES = {
     "lyra_argmax": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_size_t] + [_c.c_int] * 3 + [_c.c_void_p] * 2),
     "lyra_argmax_workspace": (_c.c_size_t, [_c.c_int] * 2),
     "lyra_sample_topk": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p, _c.c_void_p]),
+    "lyra_sample_topk_rng": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p, _c.c_void_p]),
     "lyra_sample_topk_workspace": (_c.c_size_t, [_c.c_int] * 3),
     "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
 }

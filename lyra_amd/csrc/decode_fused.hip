@@ -583,16 +583,25 @@ struct SampleParams {
     int rows, cols, ld, chunks, chunk_len, k;
     float temperature;
     int32_t* advance;  // as in ArgmaxParams
+    unsigned long long* rng;  // {seed, count} or null (then uniforms)
+    int* arrivals_all;        // rng: counts every workgroup of the launch (zero on entry, zero again on exit)
 };
+
+__device__ __forceinline__ unsigned long long splitmix64(unsigned long long z) {
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
 
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
 
-// Keeps the k best pairs seen so far in (tv, ti), best first.
-__device__ __forceinline__ void topk_insert(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], int k, float v, int i) {
-    if (!better(v, i, tv[k - 1], ti[k - 1])) return;
+// Keeps the K best pairs seen so far in (tv, ti), best first.  K is a compile-time constant: with a run-time k the arrays
+// are indexed dynamically and leave the registers (the launch then took 81 us over 64 x 201088 logits, the arg-max 14.5).
+template <int K>
+__device__ __forceinline__ void topk_insert(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], float v, int i) {
+    if (!better(v, i, tv[K - 1], ti[K - 1])) return;
 #pragma unroll
-    for (int j = kMaxSampleK - 1; j >= 0; --j) {
-        if (j >= k) continue;
+    for (int j = K - 1; j >= 0; --j) {
         const bool here = better(v, i, tv[j], ti[j]);
         const bool above = j > 0 && better(v, i, tv[j > 0 ? j - 1 : 0], ti[j > 0 ? j - 1 : 0]);
         if (here && above) {  // the pair goes further up: move the entry above down into this slot
@@ -607,16 +616,17 @@ __device__ __forceinline__ void topk_insert(float (&tv)[kMaxSampleK], int (&ti)[
 
 // The k best pairs over all threads of a workgroup of `nthreads` (64 or 256) threads, each holding its own k best,
 // best first: k rounds of "best head wins, its owner moves on".  Result in sm_tv / sm_ti (valid after the call).
-__device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], int k, int nthreads, float* sm_wv,
+template <int K>
+__device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[kMaxSampleK], int nthreads, float* sm_wv,
                                            int* sm_wi, float* sm_tv, int* sm_ti) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = nthreads >> 6;
     int head = 0;
-    for (int r = 0; r < k; ++r) {
+    for (int r = 0; r < K; ++r) {
         float hv = -INFINITY;
         int hi = 0x7FFFFFFF;
 #pragma unroll
-        for (int j = 0; j < kMaxSampleK; ++j)
-            if (j == head && j < k) {
+        for (int j = 0; j < K; ++j)
+            if (j == head) {
                 hv = tv[j];
                 hi = ti[j];
             }
@@ -647,11 +657,15 @@ __device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[k
     }
 }
 
+template <int K>
 __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
     __shared__ float sm_wv[4], sm_tv[kMaxSampleK];
     __shared__ int sm_wi[4], sm_ti[kMaxSampleK];
     __shared__ int sm_last;
-    const int c = blockIdx.x, row = blockIdx.y, k = p.k;
+    const int c = blockIdx.x, row = blockIdx.y;
+    constexpr int k = K;
+    // (the draw count is read before this workgroup is counted as arrived, and replaced only after all have been)
+    const unsigned long long draw = (p.rng && threadIdx.x == 0) ? __hip_atomic_load(&p.rng[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
     const float* xr = p.x + (size_t)row * p.ld;
     const int lo = c * p.chunk_len, hi = min(lo + p.chunk_len, p.cols);
     float tv[kMaxSampleK];
@@ -661,16 +675,54 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
         tv[j] = -INFINITY;
         ti[j] = 0x7FFFFFFF;
     }
-    for (int i = lo + threadIdx.x * 4; i < hi; i += 1024) {  // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads
-        if (i + 4 <= hi) {
-            const f32x4 v = *(const f32x4*)(xr + i);
+    // chunk_len % 4 == 0, ld % 4 == 0: aligned 16-byte loads, four of them in flight per thread.
+    // Two passes over the chunk.  Keeping K best pairs per thread costs ~15 instructions per pair and element, and with 64
+    // lanes some lane nearly always has a new candidate, so the wavefront would run the insertion for nearly every element
+    // (60 us for 64 x 201088 logits, the arg-max takes 14.5).  The first pass therefore takes one maximum per thread; the
+    // K-th largest of the workgroup's 256 maxima is a lower bound `floor_v` of the chunk's K-th best value (K elements at
+    // least that large exist).  The second pass reads the chunk again (from the caches) and only looks closer at values
+    // >= floor_v - a handful per chunk unless many logits are equal, in which case it is merely slow.
+    const int n_vec = (hi - lo) >> 2;
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(xr + lo), 0, (uint32_t)n_vec * 16u, 0x00020000);
+    float mx = -INFINITY;
+    for (int j0 = threadIdx.x; j0 < n_vec; j0 += 1024) {
+        u32x4 raw[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) topk_insert(tv, ti, k, v[q], i + q);
-        } else {
-            for (int q = 0; i + q < hi; ++q) topk_insert(tv, ti, k, xr[i + q], i + q);
+        for (int u = 0; u < 4; ++u) raw[u] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (j0 + 256 * u) * 16, 0, 0);  // (past the end: zeros, unused)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float m4 = fmaxf(fmaxf(__uint_as_float(raw[u][0]), __uint_as_float(raw[u][1])),
+                                   fmaxf(__uint_as_float(raw[u][2]), __uint_as_float(raw[u][3])));
+            mx = j0 + 256 * u < n_vec ? fmaxf(mx, m4) : mx;
         }
     }
-    topk_merge(tv, ti, k, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    for (int i = lo + 4 * n_vec + threadIdx.x; i < hi; i += 256) mx = fmaxf(mx, xr[i]);  // (a last chunk whose end is not a multiple of 4)
+    tv[0] = mx;
+    ti[0] = mx > -INFINITY ? (int)threadIdx.x : 0x7FFFFFFF;
+    topk_merge<K>(tv, ti, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    const float floor_v = sm_tv[K - 1];  // (-inf when fewer than K threads saw a finite value: everything is looked at)
+    __syncthreads();  // (sm_tv is written again below)
+    tv[0] = -INFINITY;
+    ti[0] = 0x7FFFFFFF;
+    for (int j0 = threadIdx.x; j0 < n_vec; j0 += 1024) {
+        u32x4 raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) raw[u] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (j0 + 256 * u) * 16, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int jj = j0 + 256 * u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float v = __uint_as_float(raw[u][q]);
+                if (jj < n_vec && v >= floor_v) topk_insert<K>(tv, ti, v, lo + 4 * jj + q);
+            }
+        }
+    }
+    for (int i = lo + 4 * n_vec + threadIdx.x; i < hi; i += 256) {
+        const float v = xr[i];
+        if (v >= floor_v) topk_insert<K>(tv, ti, v, i);
+    }
+    topk_merge<K>(tv, ti, 256, sm_wv, sm_wi, sm_tv, sm_ti);
     if (threadIdx.x < k) {
         store_agent(&p.part_v[((size_t)row * p.chunks + c) * k + threadIdx.x], sm_tv[threadIdx.x]);
         store_agent(&p.part_i[((size_t)row * p.chunks + c) * k + threadIdx.x], sm_ti[threadIdx.x]);
@@ -681,6 +733,13 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
         const int seen = add_agent(&p.arrivals[row], 1);
         sm_last = seen == p.chunks - 1;
         if (sm_last) store_agent(&p.arrivals[row], 0);
+        if (p.rng) {
+            const int total = (int)(gridDim.x * gridDim.y);
+            if (add_agent(p.arrivals_all, 1) == total - 1) {  // every workgroup has read the count: the next launch's is count + 1
+                store_agent(p.arrivals_all, 0);
+                __hip_atomic_store(&p.rng[1], draw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
     __syncthreads();
     if (!sm_last) return;
@@ -693,9 +752,9 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
     for (int q = threadIdx.x; q < p.chunks * k; q += 256) {
         const float v = load_agent(&p.part_v[(size_t)row * p.chunks * k + q]);
         const int i = __hip_atomic_load(&p.part_i[(size_t)row * p.chunks * k + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (i != 0x7FFFFFFF) topk_insert(tv, ti, k, v, i);
+        if (i != 0x7FFFFFFF) topk_insert<K>(tv, ti, v, i);
     }
-    topk_merge(tv, ti, k, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    topk_merge<K>(tv, ti, 256, sm_wv, sm_wi, sm_tv, sm_ti);
     if (threadIdx.x == 0) {
         // softmax of logits / temperature over the candidates (best first), inverse CDF at the row's uniform number
         float e[kMaxSampleK], total = 0.f;
@@ -707,7 +766,15 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
             total += e[j];
             n = j + 1;
         }
-        const float target = p.uniforms[row] * total;
+        float u;
+        if (p.rng) {
+            const unsigned long long seed = __hip_atomic_load(&p.rng[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned long long z = splitmix64(seed ^ ((draw + 1) * 0x9E3779B97F4A7C15ull) ^ ((unsigned long long)(row + 1) * 0xD1B54A32D192ED03ull));
+            u = (float)(z >> 40) * 0x1p-24f;
+        } else {
+            u = p.uniforms[row];
+        }
+        const float target = u * total;
         float run = 0.f;
         int pick = n > 0 ? sm_ti[n - 1] : 0;
         for (int j = 0; j < n; ++j) {
@@ -887,10 +954,30 @@ extern "C" size_t lyra_sample_topk_workspace(int rows, int cols, int k) {
     return lyra::kArgmaxCounterBytes + ((size_t)rows * lyra::argmax_chunks(rows, cols) * k * 8 + 255) / 256 * 256;
 }
 
+namespace lyra {
+static int run_sample_topk(const float* x, const float* uniforms, unsigned long long* rng, int32_t* out, void* workspace,
+                           size_t workspace_bytes, int rows, int cols, int ld, int k, float temperature, int32_t* advance,
+                           lyra_stream_t stream);
+}
+
 extern "C" int lyra_sample_topk(const float* x, const float* uniforms, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
                                 int cols, int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream) {
-    using namespace lyra;
-    if (!x || !uniforms || !out || rows <= 0 || cols <= 0 || ld < cols || k <= 0 || !(temperature > 0.f)) return LYRA_E_BADARG;
+    if (!uniforms) return LYRA_E_BADARG;
+    return lyra::run_sample_topk(x, uniforms, nullptr, out, workspace, workspace_bytes, rows, cols, ld, k, temperature, advance, stream);
+}
+
+extern "C" int lyra_sample_topk_rng(const float* x, uint64_t* rng, int32_t* out, void* workspace, size_t workspace_bytes, int rows,
+                                    int cols, int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream) {
+    if (!rng || ((uintptr_t)rng % 8)) return LYRA_E_BADARG;
+    return lyra::run_sample_topk(x, nullptr, (unsigned long long*)rng, out, workspace, workspace_bytes, rows, cols, ld, k, temperature,
+                                 advance, stream);
+}
+
+namespace lyra {
+static int run_sample_topk(const float* x, const float* uniforms, unsigned long long* rng, int32_t* out, void* workspace,
+                           size_t workspace_bytes, int rows, int cols, int ld, int k, float temperature, int32_t* advance,
+                           lyra_stream_t stream) {
+    if (!x || !out || rows <= 0 || cols <= 0 || ld < cols || k <= 0 || !(temperature > 0.f)) return LYRA_E_BADARG;
     if (ld % 4 || ((uintptr_t)x % 16) || rows > 65535 || k > kMaxSampleK) return LYRA_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < lyra_sample_topk_workspace(rows, cols, k) || ((uintptr_t)workspace % 256))
         return LYRA_E_WORKSPACE;
@@ -908,8 +995,21 @@ extern "C" int lyra_sample_topk(const float* x, const float* uniforms, int32_t* 
     p.chunk_len = ((cols + p.chunks - 1) / p.chunks + 3) / 4 * 4;
     p.chunks = (cols + p.chunk_len - 1) / p.chunk_len;
     p.arrivals = (int*)workspace;
+    p.rng = rng;
+    p.arrivals_all = (int*)workspace + 65535;  // (rows <= 65535: the last counter of the region belongs to no row)
     p.part_v = (float*)((char*)workspace + kArgmaxCounterBytes);
     p.part_i = (int*)(p.part_v + (size_t)rows * argmax_chunks(rows, cols) * k);
-    hipLaunchKernelGGL(sample_topk_kernel, dim3(p.chunks, rows), dim3(256), 0, (hipStream_t)stream, p);
+    const dim3 grid(p.chunks, rows), block(256);
+    switch (p.k) {
+        case 1: hipLaunchKernelGGL(sample_topk_kernel<1>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 2: hipLaunchKernelGGL(sample_topk_kernel<2>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 3: hipLaunchKernelGGL(sample_topk_kernel<3>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 4: hipLaunchKernelGGL(sample_topk_kernel<4>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 5: hipLaunchKernelGGL(sample_topk_kernel<5>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 6: hipLaunchKernelGGL(sample_topk_kernel<6>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 7: hipLaunchKernelGGL(sample_topk_kernel<7>, grid, block, 0, (hipStream_t)stream, p); break;
+        default: hipLaunchKernelGGL(sample_topk_kernel<8>, grid, block, 0, (hipStream_t)stream, p); break;
+    }
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
+}  // namespace lyra

@@ -24,10 +24,15 @@ def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Genera
         return _into(out, torch.argmax(logits, dim=-1).to(torch.int32))
     if (logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla"
             and 0 < cfg.sample_topk <= 8):
-        # the draw is the inverse CDF over the k candidates at one uniform number per row
-        from lyra_amd.kernels.decode_fused import sample_topk
+        # the draw is the inverse CDF over the k candidates at one uniform number per row: from the caller's torch
+        # generator when one is given, else made inside the launch from the sampler's own state (no generator launches:
+        # inside a captured step torch.rand costs three small kernels per token)
+        from lyra_amd.kernels.decode_fused import rng_state, sample_topk
 
-        u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=generator)
+        if generator is None:
+            u = rng_state(logits.device)
+        else:
+            u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=generator)
         return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]), out, advance)
     if advance is not None:
         advance += 1
@@ -66,8 +71,8 @@ class GraphedDecoder:
 
     def __init__(self, model: ModelWeights, cache: ModelCache, cfg: ModelConfig, batch: int, warmup: int = 2,
                  greedy: bool = True, advance: bool = True):
-        # greedy=False: temperature / top-k sampling as configured, the uniform numbers drawn inside the graph from the
-        # device's default generator (its state advances with every replay)
+        # greedy=False: temperature / top-k sampling as configured, the uniform numbers made inside the sampler's launch
+        # from its own generator state on the device (the state moves on with every replay)
         self.cfg, self.model, self.cache, self.greedy, self.advance = cfg, model, cache, greedy, advance
         dev = model.emb.device
         self.tokens = torch.zeros(batch, dtype=torch.int32, device=dev)

@@ -414,17 +414,38 @@ def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperatur
                 out: torch.Tensor | None = None, advance: torch.Tensor | None = None) -> torch.Tensor:
     """Temperature / top-k token choice (lyra/generate.py:46-53 at temperature > 0) for every row of float32 ``logits``
     [rows, ld] over its first ``cols`` columns: softmax of the k largest ``logits / temperature`` (ties to the lower
-    index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows]."""
+    index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows].  ``uniforms`` may instead be the
+    generator state ``rng_state(seed)`` makes (int64 [2] on the device: seed, draws so far): the launch then makes its own
+    uniform numbers and moves the state on (lyra_sample_topk_rng)."""
     rows, ld = logits.shape
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
-    assert uniforms.dtype == torch.float32 and uniforms.shape == (rows,) and uniforms.is_contiguous()
+    own_rng = uniforms.dtype == torch.int64
+    if own_rng:
+        assert uniforms.shape == (2,) and uniforms.is_contiguous() and uniforms.device == logits.device
+    else:
+        assert uniforms.dtype == torch.float32 and uniforms.shape == (rows,) and uniforms.is_contiguous()
     if out is None:
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
     assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_sample_topk_workspace(rows, cols, k))
-    rc = _L.lyra_sample_topk(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,
-                             float(temperature), _ptr(advance), stream)
+    fn = _L.lyra_sample_topk_rng if own_rng else _L.lyra_sample_topk
+    rc = fn(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,
+            float(temperature), _ptr(advance), stream)
     _lib.check(rc, "lyra_sample_topk")
     return out
+
+
+_RNG_STATES: dict = {}
+
+
+def rng_state(device, seed: int | None = None) -> torch.Tensor:
+    """The state of the sampler's own generator on ``device`` (int64 [2]: seed, draws so far).  With ``seed`` a fresh state;
+    without, one state per device, seeded from torch's initial seed the first time it is asked for."""
+    if seed is not None:
+        return torch.tensor([seed & 0x7FFFFFFFFFFFFFFF, 0], dtype=torch.int64, device=device)
+    key = str(device)
+    if key not in _RNG_STATES:
+        _RNG_STATES[key] = torch.tensor([torch.initial_seed() & 0x7FFFFFFFFFFFFFFF, 0], dtype=torch.int64, device=device)
+    return _RNG_STATES[key]

@@ -466,6 +466,61 @@ def test_sample_token_draws_from_the_topk_softmax():
     np.testing.assert_allclose(got, want, atol=0.015)  # 32768 draws: ~4 standard errors
 
 
+def test_sampler_with_its_own_generator_follows_the_documented_stream():
+    """lyra_sample_topk_rng: the uniform number of row r at draw count c is the splitmix64 formula of the header; the launch
+    then equals lyra_sample_topk fed those numbers, and leaves count + 1 behind - also when replayed from a graph."""
+    from lyra_amd.kernels import decode_fused as F
+
+    M64 = (1 << 64) - 1
+
+    def splitmix(z):
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M64
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M64
+        return z ^ (z >> 31)
+
+    def uniforms(seed, count, rows):
+        return np.array([(splitmix(seed ^ (((count + 1) * 0x9E3779B97F4A7C15) & M64) ^ (((r + 1) * 0xD1B54A32D192ED03) & M64)) >> 40) * 2.0**-24
+                         for r in range(rows)], np.float32)
+
+    dev = U.dev()
+    rows, cols = 37, 5000
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    logits = torch.randn(rows, cols, generator=g, device=dev) * 3
+    seed = 0x1234567890ABCDEF
+    state = F.rng_state(dev, seed)
+    for count in range(3):
+        got = F.sample_topk(logits, state, 4, 0.8)
+        want = F.sample_topk(logits, torch.from_numpy(uniforms(seed, count, rows)).to(dev), 4, 0.8)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"draw {count}"
+        assert state.cpu().tolist() == [seed, count + 1]
+    # every draw differs from the one before somewhere, and the picks follow the top-4 softmax over many draws
+    row = torch.randn(cols, generator=g, device=dev) * 2
+    many = row[None].repeat(4096, 1).contiguous()
+    picks = torch.cat([F.sample_topk(many, state, 4, 0.8) for _ in range(4)]).cpu().numpy()
+    top = np.argsort(-U.to_np(row), kind="stable")[:4]
+    want_p = torch.softmax(torch.from_numpy(U.to_np(row)[top] / np.float32(0.8)), 0).numpy()
+    np.testing.assert_allclose(np.array([(picks == t).mean() for t in top]), want_p, atol=0.02)
+    # replayed from a graph: the count moves on by one per replay
+    out = torch.empty(rows, dtype=torch.int32, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        F.sample_topk(logits, state, 4, 0.8, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    start = state.cpu().tolist()[1]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        F.sample_topk(logits, state, 4, 0.8, out=out)
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        want = F.sample_topk(logits, torch.from_numpy(uniforms(seed, start + rep, rows)).to(dev), 4, 0.8)
+        assert torch.equal(out, want) and state.cpu().tolist()[1] == start + rep + 1
+
+
 @pytest.mark.parametrize("B,N,K,S,H,fp8,qknorm,sw,unsummed,positions", [
     (64, 16, 4, 4096, 128, True, True, 0, True, "full"),        # headline shape: one workgroup per (row, kv head)
     (64, 16, 4, 4096, 128, True, True, 128, True, "full"),      # sliding layer
