@@ -44,7 +44,7 @@ def _bias(b):
     return None if b is None else R(np.asarray(b, dtype=np.float32))
 
 
-def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins=None, hidden_out=None, inner="ref"):
+def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins=None, hidden_out=None, inner="ref", layer_offset=0):
     """tokens [B] int; weights/cache: dicts of NumPy arrays mirroring lyra_amd.model; pos: int.
     router_margins: optional list; receives one float32 [B] array per MoE layer, the gap between the last router logit
     that is selected and the first that is not (top-k is discontinuous: a row with a tiny gap is not a parity case).
@@ -56,6 +56,8 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
     rounds only its output - the form the acceptance tolerances of the kernels are stated against.
     hidden_out: optional list; receives the residual stream [B, C] as it enters every layer, then as it leaves the last
     one (before the final norm): n_layers + 1 arrays.
+    layer_offset: index, in the whole model, of the first layer of ``weights["layers"]`` (even layers have the sliding
+    window, model.py:337): lets a caller run a few layers of a deep model on their own, fed that layer's input as "emb".
     """
     B = tokens.shape[0]
     C, H, N, K = cfg.n_embd, cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
@@ -63,7 +65,7 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
     cos, sin = cos_t[pos], sin_t[pos]
     one = np.array([B], np.int32)
     h = R(weights["emb"][tokens])
-    for idx, lw in enumerate(weights["layers"]):
+    for idx, lw in enumerate(weights["layers"], layer_offset):
         if hidden_out is not None:
             hidden_out.append(h.copy())
         # ---- attention_apply ----
@@ -78,7 +80,7 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
             q = R(O.rms_norm(q, a["qnorm_scale"], cfg.norm_eps))
             k = R(O.rms_norm(k, a["knorm_scale"], cfg.norm_eps))
         q, k = R(O.rotate(q, cos, sin)), R(O.rotate(k, cos, sin))
-        ck, cv = cache["k"][idx], cache["v"][idx]
+        ck, cv = cache["k"][idx - layer_offset], cache["v"][idx - layer_offset]
         if isinstance(ck, tuple):  # qupdate: quantise the new token with block (1, H) and write it at pos
             for (cq, cs), new in ((ck, k), (cv, v)):
                 nq, ns = O.quantize(new[:, :, None, :], (1, H))

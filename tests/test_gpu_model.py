@@ -413,3 +413,119 @@ def test_width_2880_step_of_gpt_oss_20b_with_biases_32_experts_b64():
     assert cfg.n_embd == 2880 and cfg.expert_hidden == 2880 and cfg.use_qkv_bias and cfg.use_mlp_bias and cfg.n_shared_experts == 0
     cfg = apply_inference_overrides(cfg, fp8=True, fp8_attn=True, per_channel=True)
     _full_width_parity(cfg, B=64, S=1024, start=700, steps=2, min_clear=40, moe_layers=2, hidden_tol=0.03)
+
+
+def test_config5_lyra_max_full_depth_b128_ctx4096():
+    """Benchmark configuration 5 at its literal size: lyra-max, 32 layers (2 dense + 30 MoE with 63 + 1 experts), width 4096,
+    B=128, a cache of 4096 rows, FP8 weights and cache (about 135 GB resident).  Two eager steps and the same two steps
+    replayed from a captured graph: finite logits, the same tokens, bit-identical appended cache rows; and the first two
+    and last two layers, each run on the residual stream the GPU itself had at that layer's input, against the CPU
+    restatement of that layer (teacher forced, so the CPU side stays at four layers)."""
+    import time
+
+    from lyra_amd import model as M
+    from lyra_amd.generate import GraphedDecoder, generate
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.model import MODEL_VARIANTS, ModelWeights, apply_inference_overrides, init_cache, init_weights
+    from lyra_amd.nn.quant import QArray
+
+    dev = U.dev()
+    free, _ = torch.cuda.mem_get_info()
+    if free < 170e9:
+        pytest.skip(f"needs ~150 GB of free device memory, {free / 1e9:.0f} GB are free")
+    B, S, start, n = 128, 4096, 4094, 2
+    cfg = apply_inference_overrides(replace(MODEL_VARIANTS["lyra-max"], implementation="pallas", sample_temperature=0.0), fp8=True,
+                                    fp8_attn=True, per_channel=True)
+    assert cfg.n_layers == 32 and cfg.n_routed_experts == 63 and cfg.use_learned_xsa
+    t0 = time.perf_counter()
+    w = init_weights(cfg, dev, seed=3)
+    bias_gen = torch.Generator(device=dev)
+    bias_gen.manual_seed(77)
+    for lw in w.layers:  # (spread the router logits: random-init ones lie within bf16 noise of each other)
+        if getattr(lw.mlp, "router_bias", None) is not None:
+            lw.mlp.router_bias.copy_(torch.randn(lw.mlp.router_bias.shape, device=dev, generator=bias_gen))
+    cache = init_cache(cfg, B, S, dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1005)
+    for layer in cache.layers:  # history: random finite FP8 codes with scales of N(0,1) rows
+        for arr in (layer.k, layer.v):
+            codes = torch.randint(0, 0x78, arr.qval.shape, generator=gen, device=dev, dtype=torch.uint8)
+            signs = torch.randint(0, 2, arr.qval.shape, generator=gen, device=dev, dtype=torch.uint8) << 7
+            arr.qval.view(torch.uint8).copy_(codes | signs)
+            arr.scale.copy_(torch.rand(arr.scale.shape, generator=gen, device=dev) * 0.004 + 0.006)
+    torch.cuda.synchronize()
+    print(f"config 5: model and caches built in {time.perf_counter() - t0:.0f} s", file=sys.stderr, flush=True)
+    first = torch.randint(0, cfg.vocab_size, (B,), generator=gen, device=dev, dtype=torch.int32)
+
+    def appended():
+        rows = []
+        for layer in cache.layers:
+            for arr in (layer.k, layer.v):
+                rows.append(arr.qval.view(torch.uint8)[:, :, start : start + n].clone())
+                rows.append(arr.scale[:, :, start : start + n].clone())
+        return rows
+
+    # ---- eager ----
+    cache.pos.fill_(start)
+    tok, eager_tokens = first, []
+    for s_ in range(n):
+        print(f"config 5: eager step {s_}", file=sys.stderr, flush=True)
+        logits, _ = M.model_apply(tok, w, cache, cfg)
+        assert torch.isfinite(logits[:, : cfg.vocab_size]).all() and torch.isneginf(logits[:, cfg.vocab_size :]).all()
+        tok = F.argmax(logits, cfg.vocab_size)
+        eager_tokens.append(tok.clone())
+    torch.cuda.synchronize()
+    assert int(cache.pos.item()) == start + n
+    eager_rows = appended()
+    # ---- the same two steps from a captured graph ----
+    cache.pos.fill_(start)
+    dec = GraphedDecoder(w, cache, cfg, batch=B)
+    dec.tokens.copy_(first)
+    t1 = time.perf_counter()
+    drawn = dec.decode(n)
+    torch.cuda.synchronize()
+    print(f"config 5: {n} graph replays in {(time.perf_counter() - t1) * 1e3:.1f} ms", file=sys.stderr, flush=True)
+    assert int(cache.pos.item()) == start + n
+    for s_ in range(n):
+        assert torch.equal(drawn[s_], eager_tokens[s_]), f"tokens of step {s_} differ between the graph and eager calls"
+    for a, b in zip(appended(), eager_rows):
+        assert torch.equal(a, b), "appended cache rows differ between the graph and eager calls"
+    del dec
+    # ---- layers 0, 1, 30, 31 on the GPU's own inputs against the CPU restatement of the layer ----
+    pos = torch.tensor(start, dtype=torch.int32, device=dev)
+    cos_t, sin_t = M._rope_tables(cfg, dev)
+    ones = torch.ones(cfg.n_embd, dtype=torch.float32, device=dev)
+    h = w.emb[first.long()]
+    inputs, outputs = {}, {}
+    check = (0, 1, cfg.n_layers - 2, cfg.n_layers - 1)
+    for idx, layer in enumerate(w.layers):
+        if idx in check:
+            inputs[idx] = U.to_np(h)
+        h, _ = M.attention_apply_fused(h, layer.attn, idx, pos, cos_t, sin_t, cache.layers[idx], cfg)
+        h = M.moe_apply_fused(h, layer.mlp, cfg) if isinstance(layer.mlp, M.MoEWeights) else M.dense_mlp_apply_fused(h, layer.mlp, cfg)
+        if isinstance(h, (F.Unsummed, F.Uncombined)):
+            h = F.rmsnorm_proj(h, ones, cfg.norm_eps)[2]
+        if idx in check:
+            outputs[idx] = U.to_np(h)
+    torch.cuda.synchronize()
+    for idx in check:
+        t2 = time.perf_counter()
+        one_layer = ModelWeights(emb=torch.zeros(1, 8, device=dev), unemb_t=torch.zeros(1, cfg.n_embd, 8, dtype=torch.bfloat16, device=dev),
+                                 norm_scale=ones, layers=[w.layers[idx]])
+        wn = D.weights_to_numpy(one_layer, cfg)
+        wn["emb"] = inputs[idx]
+        lc = cache.layers[idx]
+        cn = {"k": [(lc.k.qval.view(torch.uint8).cpu().numpy(), lc.k.scale.float().cpu().numpy())],
+              "v": [(lc.v.qval.view(torch.uint8).cpu().numpy(), lc.v.scale.float().cpu().numpy())]}
+        cfg1 = replace(cfg, vocab_size=8, padded_vocab_size=8)  # (the residual scales depend on the depth: all 32 layers stay configured)
+        margins, hidden = [], []
+        D.decode_step(np.arange(B), wn, cn, start, cfg1, use_c=True, router_margins=margins, hidden_out=hidden, inner="fp32",
+                      layer_offset=idx)
+        want, got = hidden[-1], outputs[idx]
+        ok = np.ones(B, bool) if not margins else margins[0] > 0.03
+        assert ok.sum() >= 96, f"layer {idx}: too few rows with unambiguous routing"
+        rel = np.linalg.norm(got - want, axis=-1) / np.linalg.norm(want, axis=-1)
+        print(f"config 5: layer {idx} ({cfg.mlp_map[idx]}): worst relative error {rel[ok].max():.5f} over {ok.sum()} rows, "
+              f"CPU side {time.perf_counter() - t2:.0f} s", file=sys.stderr, flush=True)
+        assert rel[ok].max() <= 0.01, f"layer {idx}: {rel[ok].max()}"
+        del wn, cn
