@@ -162,7 +162,11 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
         u32x2 d;
         d[0] = pack_bf16(v[0], v[1]);
         d[1] = pack_bf16(v[2], v[3]);
-        if (share == 0) *(u32x2*)(p.h + (size_t)b * p.C + c) = d;
+        if (share == 0) {
+            // (mode bit 2: h in tiles of 16 rows x 32 columns, the layout the expert matmul reads fastest)
+            const size_t at = (p.mode & 4) ? ((((size_t)(b >> 4) * (p.C >> 5) + (c >> 5)) * 16 + (b & 15)) << 5) + (c & 31) : (size_t)b * p.C + c;
+            *(u32x2*)(p.h + at) = d;
+        }
         sm_h[c] = __uint_as_float(d[0] << 16);
         sm_h[c + 1] = __uint_as_float(d[0] & 0xFFFF0000u);
         sm_h[c + 2] = __uint_as_float(d[1] << 16);
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
         if (lane == 0) {
             if (p.bias) v += p.bias[j];
             const size_t o = (size_t)b * p.n + j;
-            if (p.mode == 1) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(2.f / (1.f + __expf(-v)));
+            if ((p.mode & 3) == 1) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(2.f / (1.f + __expf(-v)));
             else ((float*)p.y)[o] = v;
         }
     }
@@ -814,7 +818,8 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     if (partials ? (!residual || !x_out || splits <= 0) : !x) return LYRA_E_BADARG;
     if (partials && (double)splits * B * C * 4 >= 2147483648.0) return LYRA_E_UNSUPPORTED;
     if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
-    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (proj_t && (!y || n <= 0 || ((mode & 3) != 1 && (mode & 3) != 2))) return LYRA_E_BADARG;
+    if ((mode & ~7) || ((mode & 4) && C % 32)) return LYRA_E_UNSUPPORTED;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr, 0};
@@ -827,7 +832,8 @@ extern "C" int lyra_rmsnorm_proj_embed(const void* table, const int32_t* tokens,
     using namespace lyra;
     if (!table || !tokens || !x_out || table_rows <= 0) return LYRA_E_BADARG;
     if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
-    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (proj_t && (!y || n <= 0 || ((mode & 3) != 1 && (mode & 3) != 2))) return LYRA_E_BADARG;
+    if ((mode & ~7) || ((mode & 4) && C % 32)) return LYRA_E_UNSUPPORTED;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)table, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      nullptr, 0, B, nullptr, 1.0f, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, tokens, table_rows};
@@ -840,7 +846,8 @@ extern "C" int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, 
     using namespace lyra;
     if (!rows || !scores || !dest || !residual || !x_out || topk <= 0) return LYRA_E_BADARG;
     if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
-    if (proj_t && (!y || n <= 0 || (mode != 1 && mode != 2))) return LYRA_E_BADARG;
+    if (proj_t && (!y || n <= 0 || ((mode & 3) != 1 && (mode & 3) != 2))) return LYRA_E_BADARG;
+    if ((mode & ~7) || ((mode & 4) && C % 32)) return LYRA_E_UNSUPPORTED;
     if (C % 4 || C > 32768 || topk > 16) return LYRA_E_UNSUPPORTED;
     NormProjParams p{nullptr, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
                      nullptr, 0, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out,

@@ -53,7 +53,18 @@ struct GemmParams {
     // 2 = the same with span s = gate columns 64 s ... followed by their linear columns N/2 + 64 s ...
     int packed;
     int pspans;
+    // Activations in tiles of 16 rows x 32 columns (1 KB each, tiles of a row block side by side): element (r, k) of an
+    // array of C columns lies at (((r >> 4) * (C >> 5) + (k >> 5)) * 16 + (r & 15)) * 32 + (k & 31).  The 16 lanes that feed
+    // one matrix instruction with 16 consecutive rows then read one contiguous KB instead of 16 pieces a row apart.
+    // lhs_tiled: lhs comes in that layout (grouped kernel); out_tiled: the bf16 output is written in it (for the next matmul).
+    int lhs_tiled, out_tiled;
 };
+
+// Element index of output (row, col .. col + 3) in an array of NO columns, row-major or tiled (GemmParams::out_tiled).
+__device__ __forceinline__ size_t out_index(const GemmParams& p, int row, int col, int NO) {
+    if (p.out_tiled) return ((((size_t)(row >> 4) * (NO >> 5) + (col >> 5)) * 16 + (row & 15)) << 5) + (col & 31);
+    return (size_t)row * NO + col;
+}
 
 // Results go out with plain stores; only the float32 K slices that the next kernel sums are written through at agent
 // scope (store_through): a K-split launch leaves 3-8 MB of them, and written back at the end of the kernel instead they
@@ -865,7 +876,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
 // Finishes 4 consecutive output columns of one row: vg holds the accumulated columns (the gate columns with SwiGLU, vl
 // then holds the matching linear columns): bias, SwiGLU, residual epilogue, cast, store.  oc = first output column.
 __device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[4], float (&vl)[4], int g, int row, int oc, int NO) {
-    const size_t oidx = (size_t)row * NO + oc;
+    const size_t oidx = (size_t)row * NO + oc;      // (residual: always row-major)
+    const size_t sidx = out_index(p, row, oc, NO);  // where the result goes
     float o[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -880,12 +892,12 @@ __device__ __forceinline__ void group_epilogue(const GemmParams& p, float (&vg)[
         o[c] = a;
     }
     if (p.out_f32) {
-        out_store(p.out, oidx * 4, f32x4{o[0], o[1], o[2], o[3]});
+        out_store(p.out, sidx * 4, f32x4{o[0], o[1], o[2], o[3]});
     } else {
         u32x2 d;
         d[0] = pack_bf16(o[0], o[1]);
         d[1] = pack_bf16(o[2], o[3]);
-        out_store(p.out, oidx * 2, d);
+        out_store(p.out, sidx * 2, d);
     }
 }
 
@@ -1003,6 +1015,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
     const int row_bytes = PACKED ? 128 * ES : p.N * ES;
     const int steps = p.K >> 5;
     const int half_stride = p.swiglu ? (p.N >> 1) : 128;
+    const int a_step = p.lhs_tiled ? 32 : 2;  // bytes from the activations of K row k to those of k + 1 ... (a step is 32 rows of K)
     bool wide;
     int spans, kw, wslot, half, span_cols, tile_cols, n_my, trips;
     auto set_layout = [&](bool w) {
@@ -1172,14 +1185,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
             const int r = mt * 16 + x;
             int src = row0 + min(r, max(rows - 1, 0));
             if (p.row_map) src = p.row_map[src];
-            avoff[mt] = r < rows ? (src * p.K + 8 * kb) * 2 : kNoLoad;
+            avoff[mt] = r >= rows ? kNoLoad
+                                  : (p.lhs_tiled ? (src >> 4) * (p.K >> 5) * 1024 + (src & 15) * 64 + kb * 16 : (src * p.K + 8 * kb) * 2);
         }
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int idx = seg_r0 * TRIP + d;
             const bool live = valid && idx < n_my;
             const int kk = (wslot + kw * idx) << 5;
-            const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
+            const int soff = __builtin_amdgcn_readfirstlane(live ? kk * a_step : 0);
             if (d < ADEPTH) {
 #pragma unroll
                 for (int mt = 0; mt < MTM; ++mt)
@@ -1284,7 +1298,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         __builtin_amdgcn_sched_barrier(0);
                         // the registers just consumed are requested again: the activations for step idx + ADEPTH, the converted
                         // weight rows for step idx + 1 + DEPTH
-                        const int soff_act = __builtin_amdgcn_readfirstlane(more_act ? kk_act * 2 : 0);
+                        const int soff_act = __builtin_amdgcn_readfirstlane(more_act ? kk_act * a_step : 0);
 #pragma unroll
                         for (int mt = 0; mt < NMT; ++mt)  // (only the row tiles the unit has)
                             a[ad][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more_act ? cur_avoff[mt] : kNoLoad, soff_act, 0);
@@ -1445,8 +1459,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                     res_a = load_bf16x4(res_rsrc, a_live ? (int)(oa * 2) : kNoLoad);
                     res_b = load_bf16x4(res_rsrc, b_live ? (int)((oa + 64) * 2) : kNoLoad);
                 }
-                if (a_live) finish4(p, ga, la, bias_ga, bias_la, res_a, oa);
-                if (b_live) finish4(p, gb, lb, bias_gb, bias_lb, res_b, oa + 64);
+                if (a_live) finish4(p, ga, la, bias_ga, bias_la, res_a, out_index(p, cur_row0 + r, oc_a, NO));
+                if (b_live) finish4(p, gb, lb, bias_gb, bias_lb, res_b, out_index(p, cur_row0 + r, oc_b, NO));
             }
         } else if (finish) {
             // biases of this thread's columns once per unit; residual values per row; every load unconditional (a null
@@ -1479,15 +1493,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         }
                     }
                     if (wide && !p.swiglu) {  // two plain spans: finish them one after the other
-                        if (oc_live) finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, oa);
-                        if (oc2_live) finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, oa + 128);
+                        if (oc_live) finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, zero4, bias_v, zero4, ra, out_index(p, cur_row0 + r, oc, NO));
+                        if (oc2_live) finish4(p, f32x4{al[0], al[1], al[2], al[3]}, zero4, bias_l, zero4, ra2, out_index(p, cur_row0 + r, oc + 128, NO));
                         if (two) {
-                            if (oc_live) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, ob);
-                            if (oc2_live) finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, ob + 128);
+                            if (oc_live) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, zero4, bias_v, zero4, rb4, out_index(p, cur_row0 + rb, oc, NO));
+                            if (oc2_live) finish4(p, f32x4{bl[0], bl[1], bl[2], bl[3]}, zero4, bias_l, zero4, rb2, out_index(p, cur_row0 + rb, oc + 128, NO));
                         }
                     } else if (oc_live) {
-                        finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, oa);
-                        if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, ob);
+                        finish4(p, f32x4{ag[0], ag[1], ag[2], ag[3]}, f32x4{al[0], al[1], al[2], al[3]}, bias_v, bias_l, ra, out_index(p, cur_row0 + r, oc, NO));
+                        if (two) finish4(p, f32x4{bg[0], bg[1], bg[2], bg[3]}, f32x4{bl[0], bl[1], bl[2], bl[3]}, bias_v, bias_l, rb4, out_index(p, cur_row0 + rb, oc, NO));
                     }
                 }
             };
@@ -1769,6 +1783,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
                                    lyra_stream_t stream) {
     using namespace lyra;
     const bool bias_post = (post_scale & 2) != 0;  // post_scale: bit 0 the scale / residual epilogue, bit 1 the bias after the cast
+    const bool lhs_tiled = (post_scale & 4) != 0, out_tiled = (post_scale & 8) != 0;  // bits 2, 3: activations in 16 x 32 tiles
     post_scale &= 1;
     // span-major weights (lyra_gemm_pack): the layout travels in the upper bits of rhs_dtype
     const int layout = (rhs_dtype & LYRA_RHS_SPAN_MAJOR) ? 1 : ((rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU) ? 2 : 0);
@@ -1809,6 +1824,11 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
     p.packed = layout;
     p.pspans = layout ? packed_spans(N, layout) : 0;
+    // tiled activations: the grouped kernel only; a tiled output is bf16, a whole number of 32-column tiles, no residual
+    if ((lhs_tiled || out_tiled) && !pl.grouped) return LYRA_E_UNSUPPORTED;
+    if (out_tiled && (out_dtype != LYRA_DTYPE_BF16 || residual || (fused_swiglu ? N / 2 : N) % 32)) return LYRA_E_UNSUPPORTED;
+    p.lhs_tiled = lhs_tiled;
+    p.out_tiled = out_tiled;
     p.lhs = (const uint16_t*)lhs;
     p.rhs = (const uint8_t*)rhs;
     p.scale = rhs_scale;

@@ -62,6 +62,27 @@ class Uncombined:
         self.rows, self.scores, self.dest, self.residual, self.scale = rows, scores, dest, residual, scale
 
 
+class Tiled16:
+    """bf16 activations [rows, cols] in tiles of 16 rows x 32 columns (element (r, c) at
+    (((r >> 4) * (cols >> 5) + (c >> 5)) * 16 + (r & 15)) * 32 + (c & 31)): what ``rmsnorm_proj(..., tiled=True)`` and
+    ``gemm(..., out_tiled=True)`` write and ``gemm`` reads as lhs when the rows feed an expert matmul."""
+
+    __slots__ = ("data", "rows", "cols")
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @staticmethod
+    def empty(rows: int, cols: int, device) -> "Tiled16":
+        assert cols % 32 == 0
+        return Tiled16(torch.empty(((rows + 15) // 16 * 16) * cols, dtype=torch.bfloat16, device=device), rows, cols)
+
+    def untiled(self) -> torch.Tensor:
+        """The row-major [rows, cols] array (tests)."""
+        rb = self.data.numel() // (16 * self.cols)
+        return self.data.reshape(rb, self.cols // 32, 16, 32).permute(0, 2, 1, 3).reshape(rb * 16, self.cols)[: self.rows]
+
+
 class SpanMajor:
     """Weights [G, K, N] (bf16, or FP8 with their QArray scales) in the span-major copy ``lyra_gemm_pack`` makes once when a
     model is loaded: every 128-column span of every matrix is one contiguous run of K rows.  ``layout`` 1: spans of 128
@@ -154,9 +175,10 @@ def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed
 
 
 def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None = None,
-                 bias: torch.Tensor | None = None, gate: bool = False):
+                 bias: torch.Tensor | None = None, gate: bool = False, tiled: bool = False):
     """rms_norm (lyra/model.py:189-191) of x [B,C] bf16; with ``proj`` [C,n] f32 also f32(h) @ proj (+ bias) as
     float32 logits, or bf16 ``2*sigmoid`` gates when ``gate`` is set (model.py:343-347).  Returns (h, y | None).
+    ``tiled``: h comes back as a ``Tiled16`` (the layout an expert matmul reads its rows fastest in; C % 32 == 0).
 
     ``x`` may be an ``Unsummed`` projection with its residual: the row is then first formed as
     ``bf16(residual + bf16(bf16(sum of slices) * scale))`` and returned as a third value.  Likewise for an ``Uncombined``
@@ -168,7 +190,7 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
         assert u.residual.dtype == torch.bfloat16 and u.residual.is_contiguous()
         assert u.rows.dtype == torch.bfloat16 and u.rows.is_contiguous() and tuple(u.rows.shape) == (B * topk, C)
         x_out = torch.empty_like(u.residual)
-        h = torch.empty_like(u.residual)
+        h_obj, h, mode = _norm_out(u.residual, tiled, gate)
         y, n = None, 0
         if proj is not None:
             n = proj.shape[1]
@@ -176,15 +198,15 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
             proj = _f32(_transposed(proj))
         rc = _L.lyra_rmsnorm_proj_combine(u.rows.data_ptr(), _f32(u.scores).data_ptr(), u.dest.data_ptr(), topk, u.residual.data_ptr(),
                                           float(u.scale), x_out.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj),
-                                          _ptr(bias), _ptr(y), B, C, n, 1 if gate else 2, float(eps), _stream(h.device))
+                                          _ptr(bias), _ptr(y), B, C, n, mode, float(eps), _stream(h.device))
         _lib.check(rc, "lyra_rmsnorm_proj_combine")
-        return h, y, x_out
+        return h_obj, y, x_out
     if isinstance(x, Unsummed):
         u = x
         splits, B, C = u.partials.shape
         assert u.residual is not None and u.residual.dtype == torch.bfloat16 and u.residual.is_contiguous()
         x_out = torch.empty_like(u.residual)
-        h = torch.empty_like(u.residual)
+        h_obj, h, mode = _norm_out(u.residual, tiled, gate)
         y, n = None, 0
         if proj is not None:
             n = proj.shape[1]
@@ -192,21 +214,31 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
             proj = _f32(_transposed(proj))
         rc = _L.lyra_rmsnorm_proj_sum(None, u.partials.data_ptr(), splits, u.residual.data_ptr(), float(u.scale), x_out.data_ptr(),
                                       _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
-                                      1 if gate else 2, float(eps), _stream(h.device))
+                                      mode, float(eps), _stream(h.device))
         _lib.check(rc, "lyra_rmsnorm_proj_sum")
-        return h, y, x_out
+        return h_obj, y, x_out
     B, C = x.shape
     assert x.dtype == torch.bfloat16 and x.is_contiguous()
-    h = torch.empty_like(x)
+    h_obj, h, mode = _norm_out(x, tiled, gate)
     y, n = None, 0
     if proj is not None:
         n = proj.shape[1]
         y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=x.device)
         proj = _f32(_transposed(proj))
     rc = _L.lyra_rmsnorm_proj(x.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
-                              1 if gate else 2, float(eps), _stream(x.device))
+                              mode, float(eps), _stream(x.device))
     _lib.check(rc, "lyra_rmsnorm_proj")
-    return h, y
+    return h_obj, y
+
+
+def _norm_out(like: torch.Tensor, tiled: bool, gate: bool):
+    """(what the caller gets, the tensor the kernel writes, the kernel's mode word) for the normalised rows of a norm launch."""
+    mode = 1 if gate else 2
+    if not tiled:
+        h = torch.empty_like(like)
+        return h, h, mode
+    obj = Tiled16.empty(like.shape[0], like.shape[1], like.device)
+    return obj, obj.data, mode | 4
 
 
 def embed_rmsnorm_proj(table: torch.Tensor, tokens: torch.Tensor, scale: torch.Tensor, eps: float,
@@ -323,20 +355,32 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
 def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None = None, row_map: torch.Tensor | None = None,
          residual: torch.Tensor | None = None, out_scale: float | None = None, fused_swiglu: bool = False,
          swiglu_beta: float = 1.702, swiglu_limit: float = 7.0, out_f32: bool = False,
-         bias: torch.Tensor | None = None, bias_after_cast: bool = False) -> torch.Tensor:
+         bias: torch.Tensor | None = None, bias_after_cast: bool = False, out_tiled: bool = False):
     """lyra_decode_gemm_ex: the decode grouped matmul with an optional row gather on the input and an optional
     ``bf16(residual + bf16(bf16(t) * out_scale))`` epilogue.  rhs: bf16 [G,K,N] tensor or FP8 QArray.
     A ``SpanMajor`` rhs (``pack_weights``) is read in that layout.
     ``bias`` [G, N] float32 is added to the float32 product (lyra/kernels/gemm.py:1600-1605), or with ``bias_after_cast``
     (one group, no SwiGLU) to the product rounded to bf16, in bf16, as a caller does that adds a bias to the operator's
     result (lyra/model.py:310-313, 367-368)."""
-    dev = lhs.device
     rv, rs, bk, bn, rd, (G, K, N) = _rhs_args(rhs)
-    M = rows if rows is not None else lhs.shape[0]
-    assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
+    lhs_tiled = isinstance(lhs, Tiled16)
+    if lhs_tiled:  # (several groups only: rows in tiles of 16 x 32, what the norm or the matmul before wrote)
+        assert lhs.cols == K and G > 1
+        M = rows if rows is not None else lhs.rows
+        lhs_t = lhs.data
+    else:
+        M = rows if rows is not None else lhs.shape[0]
+        assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
+        lhs_t = lhs
+    dev = lhs_t.device
     assert group_sizes.dtype == torch.int32 and group_sizes.numel() == G
     NO = N // 2 if fused_swiglu else N
-    out = torch.empty((M, NO), dtype=torch.float32 if out_f32 else torch.bfloat16, device=dev)
+    if out_tiled:
+        assert not out_f32 and residual is None and G > 1 and NO % 32 == 0
+        out_obj = Tiled16.empty(M, NO, dev)
+        out = out_obj.data
+    else:
+        out = torch.empty((M, NO), dtype=torch.float32 if out_f32 else torch.bfloat16, device=dev)
     if residual is not None:
         assert residual.dtype == torch.bfloat16 and residual.is_contiguous() and tuple(residual.shape) == (M, NO)
     if row_map is not None:
@@ -346,9 +390,9 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     stream = _stream(dev)
     need = _L.lyra_decode_gemm_workspace(M, G, K, N, int(fused_swiglu))
     ws = _lib.workspace("gemm", dev, stream, need)
-    rc = _L.lyra_decode_gemm_ex(lhs.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
+    rc = _L.lyra_decode_gemm_ex(lhs_t.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
                                 _ptr(residual), 1.0 if out_scale is None else float(out_scale),
-                                int(out_scale is not None) | (2 if bias_after_cast else 0),
+                                int(out_scale is not None) | (2 if bias_after_cast else 0) | (4 if lhs_tiled else 0) | (8 if out_tiled else 0),
                                 out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
                                 _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
                                 float(swiglu_limit), stream)
@@ -356,9 +400,9 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
         # (a shape whose plan has no span-major kernel, e.g. one group with too many rows for the K-split kernel)
         return gemm(lhs, rhs.fallback, group_sizes, rows=rows, row_map=row_map, residual=residual, out_scale=out_scale,
                     fused_swiglu=fused_swiglu, swiglu_beta=swiglu_beta, swiglu_limit=swiglu_limit, out_f32=out_f32, bias=bias,
-                    bias_after_cast=bias_after_cast)
+                    bias_after_cast=bias_after_cast, out_tiled=out_tiled)
     _lib.check(rc, "lyra_decode_gemm_ex")
-    return out
+    return out_obj if out_tiled else out
 
 
 def moe_route(logits: torch.Tensor, n_routed: int, n_shared: int, k_routed: int):

@@ -456,6 +456,7 @@ def _one_group(rows: int, device) -> torch.Tensor:
 _ONE_GROUP: dict = {}
 _SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tuning override: combine in a launch of its own
 _SEPARATE_QKV_POST = os.environ.get("LYRA_QKV_POST_KERNEL") is not None  # tuning override: QK norm + RoPE + cache append in a launch of its own
+_TILED_ACTIVATIONS = os.environ.get("LYRA_ROW_MAJOR_ACTIVATIONS") is None  # tuning override: expert matmuls read row-major activations
 
 
 @dataclass
@@ -528,17 +529,20 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None 
     from lyra_amd.kernels import decode_fused as F
 
     topk = cfg.n_active_experts
+    # (the normalised rows and the up projection's output feed expert matmuls only: both travel in 16 x 32 tiles, which is
+    # how units of many rows - the shared expert's - read them fastest)
+    tiled = _TILED_ACTIVATIONS and cfg.n_embd % 32 == 0 and cfg.expert_hidden % 32 == 0 and cfg.n_experts > 1
     if isinstance(x, (F.Unsummed, F.Uncombined)):
-        xn, logits, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+        xn, logits, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias, tiled=tiled)
     else:
-        xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias)
+        xn, logits = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.router, w.router_bias, tiled=tiled)
     B = x.shape[0]
     scores, groups, row_map, dest = F.moe_route(logits, cfg.n_routed_experts, cfg.n_shared_experts, cfg.n_active_routed_experts)
     if groups_out is not None:
         groups_out.append(groups)
     G = cfg.n_experts
     t = F.gemm(xn, F.span_major(w.mlp_up, glu=True), groups, rows=B * topk, row_map=row_map, fused_swiglu=True,
-               swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, bias=_bf16_bias(w.mlp_up_bias, G))
+               swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit, bias=_bf16_bias(w.mlp_up_bias, G), out_tiled=tiled)
     t = F.gemm(t, F.span_major(w.mlp_down), groups, bias=_bf16_bias(w.mlp_down_bias, G))
     if topk <= 16 and not _SEPARATE_COMBINE:  # the combine step is left to the norm that follows (the next layer's, or the final one)
         return F.Uncombined(t, scores, dest, x, cfg.residual_scale)

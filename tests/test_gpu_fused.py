@@ -647,3 +647,76 @@ def test_gemm_bias_after_the_cast(fp8, M, K, N):
     pre = F.gemm(x, w, one, bias=b32)
     assert not torch.equal(pre, plain + bias)
     U.assert_close(U.to_np(pre), U.to_np(plain).astype(np.float32) + U.to_np(bias), atol=2e-2, rtol=1e-2, what="bias in float32")
+
+
+def _tile16(x: torch.Tensor):
+    """Row-major [rows, cols] bf16 -> Tiled16 (the documented layout, built with torch ops)."""
+    from lyra_amd.kernels import decode_fused as F
+
+    rows, cols = x.shape
+    rb = (rows + 15) // 16
+    pad = torch.zeros(rb * 16, cols, dtype=x.dtype, device=x.device)
+    pad[:rows] = x
+    data = pad.reshape(rb, 16, cols // 32, 32).permute(0, 2, 1, 3).contiguous().reshape(-1)
+    return F.Tiled16(data, rows, cols)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("M,G,K,N,swiglu,gather", [(300, 16, 512, 4096, True, True), (300, 16, 2048, 2048, False, False),
+                                                     (11, 4, 512, 512, True, True), (130, 3, 320, 2880, False, False),
+                                                     (256, 16, 2048, 4096, True, True)])
+def test_expert_matmul_reads_and_writes_activations_in_tiles(fp8, M, G, K, N, swiglu, gather):
+    """post_scale bits 2 and 3 of lyra_decode_gemm_ex: activations in tiles of 16 rows x 32 columns in, and out.  Only
+    addresses change, so the result is the row-major call's bit for bit - with the token gather, with span-major weights,
+    and with rows past the last group."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import quantize
+
+    _say(f"tiled activations fp8={fp8} M{M} G{G} K{K} N{N} swiglu={swiglu} gather={gather}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(M + N)
+    rng = np.random.default_rng(M + K)
+    cuts = np.sort(rng.integers(0, M - 2, G - 1))
+    sizes = np.diff(np.concatenate([[0], cuts, [M - 3]])).astype(np.int32)  # three rows past the last group
+    sizes[int(np.argmax(sizes))] += 0
+    gs = torch.from_numpy(sizes).to(dev)
+    tokens = 64 if gather else M
+    x = torch.randn(tokens, K, generator=g, device=dev).to(torch.bfloat16)
+    row_map = torch.randint(0, tokens, (M,), generator=g, device=dev, dtype=torch.int32) if gather else None
+    w = (torch.randn(G, K, N, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    if fp8:
+        w = quantize(w, torch.float8_e4m3fn, (K, 1))
+    bias = torch.randn(G, N, generator=g, device=dev)
+    kw = dict(rows=M, row_map=row_map, fused_swiglu=swiglu, bias=bias)
+    want = F.gemm(x, w, gs, **kw)
+    got_in = F.gemm(_tile16(x), w, gs, **kw)
+    assert torch.equal(got_in, want), "tiled input"
+    NO = N // 2 if swiglu else N
+    if NO % 32 == 0:
+        got_out = F.gemm(_tile16(x), w, gs, out_tiled=True, **kw)
+        assert isinstance(got_out, F.Tiled16) and torch.equal(got_out.untiled(), want), "tiled output"
+        packed = F.pack_weights(w, glu=swiglu)
+        got_pk = F.gemm(_tile16(x), packed, gs, out_tiled=True, **kw)
+        assert torch.equal(got_pk.untiled(), F.gemm(x, packed, gs, **kw)), "tiled, span-major weights"
+
+
+@pytest.mark.parametrize("B,C,n", [(64, 2048, 15), (5, 256, 7), (128, 4096, 63), (33, 2880, 32)])
+def test_norm_writes_its_rows_in_tiles(B, C, n):
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"tiled norm B{B} C{C} n{n}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(B + C)
+    x = (torch.randn(B, C, generator=g, device=dev) * 3).to(torch.bfloat16)
+    scale = 1 + 0.1 * torch.randn(C, generator=g, device=dev)
+    proj = torch.randn(C, n, generator=g, device=dev) / C**0.5
+    h, y = F.rmsnorm_proj(x, scale, 1e-5, proj, None)
+    ht, yt = F.rmsnorm_proj(x, scale, 1e-5, proj, None, tiled=True)
+    assert isinstance(ht, F.Tiled16) and torch.equal(ht.untiled(), h) and torch.equal(yt, y)
+    # ... and when the row is first formed from unsummed slices
+    part = torch.randn(3, B, C, generator=g, device=dev)
+    h2, _, x2 = F.rmsnorm_proj(F.Unsummed(part, x, 0.25), scale, 1e-5, proj, None)
+    h2t, _, x2t = F.rmsnorm_proj(F.Unsummed(part, x, 0.25), scale, 1e-5, proj, None, tiled=True)
+    assert torch.equal(h2t.untiled(), h2) and torch.equal(x2t, x2)
