@@ -28,6 +28,15 @@ extern "C" {
  * the span-major copy of it that lyra_gemm_pack writes (layout 1 or 2 below). */
 #define LYRA_RHS_SPAN_MAJOR 0x100     /* layout 1: spans of 128 consecutive columns */
 #define LYRA_RHS_SPAN_MAJOR_GLU 0x200 /* layout 2: spans of 64 gate columns + their 64 linear columns (fused_swiglu) */
+/* ... and, likewise OR-ed into rhs_dtype: bf16 activations in tiles of 16 rows x 32 columns (1 KB each; the tiles of 16 rows
+ * side by side, then the next 16 rows): element (r, c) of an array of C columns (C % 32 == 0) lies at
+ *   (((r >> 4) * (C >> 5) + (c >> 5)) * 16 + (r & 15)) * 32 + (c & 31),
+ * with room for the rows rounded up to 16.  The 16 lanes that feed one matrix instruction with 16 consecutive rows then
+ * read one contiguous KB instead of 16 pieces a row apart, which is what workgroups with many rows (a shared expert's
+ * units, the 32- and 64-row blocks of the K-split projections) spend their extra time on.  An internal layout of a fused
+ * decode step: lyra_rmsnorm_proj (mode | 4) and the calls below with LYRA_OUT_TILED16 write it, no reference array has it. */
+#define LYRA_LHS_TILED16 0x400 /* lhs is tiled: lyra_decode_gemm_ex with several groups or a K-split plan, lyra_decode_gemm_partials */
+#define LYRA_OUT_TILED16 0x800 /* out is written tiled (bf16, no residual, output width % 32 == 0): lyra_decode_gemm_ex, same plans */
 
 #define LYRA_OK 0
 #define LYRA_E_BADARG (-1)      /* null pointer, non-positive size, N % K != 0 ... */
@@ -207,11 +216,7 @@ size_t lyra_decode_gemm_workspace_for(int M, int G, int K, int N, int bk, int fu
  *               t = bf16(bf16(product) + bias), as the model does for the q/k/v, output and dense down
  *               projections (model.py:310-313, 367-368, 629-630: a bf16 bias added to the operator's bf16
  *               result); without it the bias is added to the float32 product (gemm.py:1600-1605).
- *               bit 2 (several groups): lhs comes in tiles of 16 rows x 32 columns (see lyra_rmsnorm_proj, mode | 4): the 16
- *               lanes that feed a matrix instruction with 16 consecutive rows read one contiguous KB instead of 16
- *               pieces a row apart, which is what units of many rows (a shared expert's) spend their extra time on.
- *               bit 3 (several groups, bf16 output, no residual, output width % 32 == 0): out is written in that
- *               layout, for the matmul that reads it next (the expert down projection after the up projection).
+ *   rhs_dtype   may carry LYRA_RHS_SPAN_MAJOR(_GLU), LYRA_LHS_TILED16 and LYRA_OUT_TILED16 (above).
  */
 int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
                         int bn, const int32_t* group_sizes, const float* bias, const void* residual, float out_scale,
@@ -266,9 +271,7 @@ int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const float* rhs
  *   reference's [C,n] parameter transposed once at load time so that each output reads a contiguous row.  C % 4 == 0.
  *   mode 1: y -> bf16(2 * sigmoid(y)), the per-head output gate (model.py:343-347), y is bf16 [B,n];
  *   mode 2: y float32 [B,n], the router logits (model.py:455-457).  proj_t NULL: norm only.
- *   mode | 4: h is written in tiles of 16 rows x 32 columns - element (b, c) at
- *             (((b >> 4) * (C >> 5) + (c >> 5)) * 16 + (b & 15)) * 32 + (c & 31), room for B rounded up to 16 rows -
- *             which is how lyra_decode_gemm_ex (post_scale bit 2) reads the rows of many-row experts fastest; C % 32 == 0.
+ *   mode | 4: h is written in tiles of 16 rows x 32 columns (LYRA_LHS_TILED16 above; C % 32 == 0), for the matmul behind it.
  */
 int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C,
                       int n, int mode, float eps, lyra_stream_t stream);

@@ -9,6 +9,7 @@ LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
 RHS_SPAN_MAJOR, RHS_SPAN_MAJOR_GLU = 0x100, 0x200  # LYRA_RHS_SPAN_MAJOR(_GLU): OR-ed into a matmul's rhs_dtype
+LHS_TILED16, OUT_TILED16 = 0x400, 0x800  # LYRA_LHS_TILED16 / LYRA_OUT_TILED16, likewise
 ABI_VERSION = 12
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 

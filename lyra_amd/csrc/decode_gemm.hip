@@ -480,7 +480,7 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
         u32x2 d;
         d[0] = pack_bf16(a[0], a[1]);
         d[1] = pack_bf16(a[2], a[3]);
-        out_store(p.out, ((size_t)row * NO + col) * 2, d);
+        out_store(p.out, out_index(p, row, col, NO) * 2, d);
     }
 }
 
@@ -734,8 +734,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
         const int arow = row0 + mt * 16 + x;
         const bool mine = arow < p.M && mt * 16 < p.row_block;
         const int asrc = mine ? (p.row_map ? p.row_map[arow] : arow) : 0;
-        avoff[mt] = mine ? (asrc * p.K + 8 * kb) * 2 : kNoLoad;
+        avoff[mt] = !mine ? kNoLoad : (p.lhs_tiled ? (asrc >> 4) * (p.K >> 5) * 1024 + (asrc & 15) * 64 + kb * 16 : (asrc * p.K + 8 * kb) * 2);
     }
+    const int a_step = p.lhs_tiled ? 32 : 2;  // (activations in tiles of 16 rows x 32 columns: GemmParams::lhs_tiled)
     const int n_mt = min(min(p.row_block >> 4, MT), (p.M - row0 + 15) >> 4);  // 16-row tiles of this block that exist
 
     // all operands are requested before anything is waited for, in the order they are consumed
@@ -745,7 +746,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
     for (int d = 0; d < DEPTH; ++d) {
         const bool live = d < n_my;
         const int kk = step_row(d);
-        const int soff = __builtin_amdgcn_readfirstlane(live ? kk * 2 : 0);
+        const int soff = __builtin_amdgcn_readfirstlane(live ? kk * a_step : 0);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {  // (row tiles the block does not have are not requested: a load that fetches nothing
             if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, live ? avoff[mt] : kNoLoad, soff, 0);  // still takes its turn)
@@ -805,7 +806,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(Ge
                 const bool more = idx + DEPTH < n_my;
                 const int kk_next = step_row(idx + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
-                const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * 2 : 0);
+                const int soff = __builtin_amdgcn_readfirstlane(more ? kk_next * a_step : 0);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     if (mt < n_mt) a[d][mt] = __builtin_amdgcn_raw_buffer_load_b128(arsrc, more ? avoff[mt] : kNoLoad, soff, 0);
@@ -1783,12 +1784,12 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
                                    lyra_stream_t stream) {
     using namespace lyra;
     const bool bias_post = (post_scale & 2) != 0;  // post_scale: bit 0 the scale / residual epilogue, bit 1 the bias after the cast
-    const bool lhs_tiled = (post_scale & 4) != 0, out_tiled = (post_scale & 8) != 0;  // bits 2, 3: activations in 16 x 32 tiles
     post_scale &= 1;
+    const bool lhs_tiled = (rhs_dtype & LYRA_LHS_TILED16) != 0, out_tiled = (rhs_dtype & LYRA_OUT_TILED16) != 0;
     // span-major weights (lyra_gemm_pack): the layout travels in the upper bits of rhs_dtype
     const int layout = (rhs_dtype & LYRA_RHS_SPAN_MAJOR) ? 1 : ((rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU) ? 2 : 0);
     if ((rhs_dtype & LYRA_RHS_SPAN_MAJOR) && (rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU)) return LYRA_E_BADARG;
-    rhs_dtype &= ~(LYRA_RHS_SPAN_MAJOR | LYRA_RHS_SPAN_MAJOR_GLU);
+    rhs_dtype &= ~(LYRA_RHS_SPAN_MAJOR | LYRA_RHS_SPAN_MAJOR_GLU | LYRA_LHS_TILED16 | LYRA_OUT_TILED16);
     if (residual && (!post_scale || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
     if (bias_post && (!bias || out_dtype != LYRA_DTYPE_BF16)) return LYRA_E_BADARG;
     if (bias_post && (G != 1 || fused_swiglu)) return LYRA_E_UNSUPPORTED;
@@ -1824,8 +1825,9 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
     p.packed = layout;
     p.pspans = layout ? packed_spans(N, layout) : 0;
-    // tiled activations: the grouped kernel only; a tiled output is bf16, a whole number of 32-column tiles, no residual
-    if ((lhs_tiled || out_tiled) && !pl.grouped) return LYRA_E_UNSUPPORTED;
+    // tiled activations: the grouped kernel and the K-split kernel (whose finish step writes the output); a tiled output is
+    // bf16, a whole number of 32-column tiles, no residual
+    if ((lhs_tiled || out_tiled) && !pl.grouped && !pl.split_k) return LYRA_E_UNSUPPORTED;
     if (out_tiled && (out_dtype != LYRA_DTYPE_BF16 || residual || (fused_swiglu ? N / 2 : N) % 32)) return LYRA_E_UNSUPPORTED;
     p.lhs_tiled = lhs_tiled;
     p.out_tiled = out_tiled;
@@ -2015,7 +2017,9 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     if (!lhs || !rhs || !group_sizes || !partials || M <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
     if (rhs_dtype & LYRA_RHS_SPAN_MAJOR_GLU) return LYRA_E_UNSUPPORTED;
     const int layout = (rhs_dtype & LYRA_RHS_SPAN_MAJOR) ? 1 : 0;
-    rhs_dtype &= ~LYRA_RHS_SPAN_MAJOR;
+    const bool lhs_tiled = (rhs_dtype & LYRA_LHS_TILED16) != 0;
+    if (rhs_dtype & LYRA_OUT_TILED16) return LYRA_E_UNSUPPORTED;  // (the slices are float32, row-major)
+    rhs_dtype &= ~(LYRA_RHS_SPAN_MAJOR | LYRA_LHS_TILED16);
     if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
     if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
@@ -2049,5 +2053,6 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     p.row_block = pl.row_block;
     p.packed = layout;
     p.pspans = layout ? packed_spans(N, layout) : 0;
+    p.lhs_tiled = lhs_tiled;
     return launch_split_k(p, pl, fp8, (hipStream_t)stream);
 }

@@ -83,6 +83,15 @@ class Tiled16:
         return self.data.reshape(rb, self.cols // 32, 16, 32).permute(0, 2, 1, 3).reshape(rb * 16, self.cols)[: self.rows]
 
 
+def tile16(x: torch.Tensor) -> Tiled16:
+    """Row-major [rows, cols] bf16 -> Tiled16, with torch ops (tests, fallbacks)."""
+    rows, cols = x.shape
+    rb = (rows + 15) // 16
+    pad = torch.zeros(rb * 16, cols, dtype=x.dtype, device=x.device)
+    pad[:rows] = x
+    return Tiled16(pad.reshape(rb, 16, cols // 32, 32).permute(0, 2, 1, 3).contiguous().reshape(-1), rows, cols)
+
+
 class SpanMajor:
     """Weights [G, K, N] (bf16, or FP8 with their QArray scales) in the span-major copy ``lyra_gemm_pack`` makes once when a
     model is loaded: every 128-column span of every matrix is one contiguous run of K rows.  ``layout`` 1: spans of 128
@@ -159,17 +168,20 @@ def _rhs_args(rhs):
 
 def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed | None:
     """lyra_decode_gemm_partials for a one-group projection; None when the shape does not run split over K."""
-    M, K = lhs.shape
+    tiled = isinstance(lhs, Tiled16)
+    M, K = (lhs.rows, lhs.cols) if tiled else lhs.shape
+    lhs_t = lhs.data if tiled else lhs
     rv, rs, bk, bn, rd, (G, _, N) = _rhs_args(rhs)
     if G != 1 or K % 32 or N % 128 or (isinstance(rhs, SpanMajor) and rhs.layout != 1):
         return None
     splits = _L.lyra_decode_gemm_splits(M, K, N, bk)
     if splits <= 0:
         return None
-    assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous()
-    part = torch.empty((splits, M, N), dtype=torch.float32, device=lhs.device)
-    rc = _L.lyra_decode_gemm_partials(lhs.data_ptr(), rv.data_ptr(), _ptr(rs), bk, bn,
-                                      group_sizes.data_ptr(), part.data_ptr(), part.numel() * 4, M, K, N, rd, _stream(lhs.device))
+    assert lhs_t.dtype == torch.bfloat16 and lhs_t.is_contiguous()
+    part = torch.empty((splits, M, N), dtype=torch.float32, device=lhs_t.device)
+    rc = _L.lyra_decode_gemm_partials(lhs_t.data_ptr(), rv.data_ptr(), _ptr(rs), bk, bn,
+                                      group_sizes.data_ptr(), part.data_ptr(), part.numel() * 4, M, K, N,
+                                      rd | (_lib.LHS_TILED16 if tiled else 0), _stream(lhs_t.device))
     _lib.check(rc, "lyra_decode_gemm_partials")
     return Unsummed(part)
 
@@ -242,7 +254,7 @@ def _norm_out(like: torch.Tensor, tiled: bool, gate: bool):
 
 
 def embed_rmsnorm_proj(table: torch.Tensor, tokens: torch.Tensor, scale: torch.Tensor, eps: float,
-                       proj: torch.Tensor | None = None, bias: torch.Tensor | None = None, gate: bool = False):
+                       proj: torch.Tensor | None = None, bias: torch.Tensor | None = None, gate: bool = False, tiled: bool = False):
     """The first norm of a decode step with the token gather folded in (lyra/model.py:752 + :303): rows
     ``table[tokens]`` (table [V,C] bf16, tokens [B] int32) are normalised as in ``rmsnorm_proj``; returns (h, y | None, x)
     with x [B,C] the gathered rows, i.e. the residual stream."""
@@ -250,16 +262,16 @@ def embed_rmsnorm_proj(table: torch.Tensor, tokens: torch.Tensor, scale: torch.T
     B = tokens.shape[0]
     assert table.dtype == torch.bfloat16 and table.is_contiguous() and tokens.dtype == torch.int32 and tokens.is_contiguous()
     x = torch.empty((B, C), dtype=torch.bfloat16, device=table.device)
-    h = torch.empty_like(x)
+    h_obj, h, mode = _norm_out(x, tiled, gate)
     y, n = None, 0
     if proj is not None:
         n = proj.shape[1]
         y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=x.device)
         proj = _f32(_transposed(proj))
     rc = _L.lyra_rmsnorm_proj_embed(table.data_ptr(), tokens.data_ptr(), V, x.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(),
-                                    _ptr(proj), _ptr(bias), _ptr(y), B, C, n, 1 if gate else 2, float(eps), _stream(x.device))
+                                    _ptr(proj), _ptr(bias), _ptr(y), B, C, n, mode, float(eps), _stream(x.device))
     _lib.check(rc, "lyra_rmsnorm_proj_embed")
-    return h, y, x
+    return h_obj, y, x
 
 
 def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: torch.Tensor, cache_k, cache_v,
@@ -364,8 +376,8 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     result (lyra/model.py:310-313, 367-368)."""
     rv, rs, bk, bn, rd, (G, K, N) = _rhs_args(rhs)
     lhs_tiled = isinstance(lhs, Tiled16)
-    if lhs_tiled:  # (several groups only: rows in tiles of 16 x 32, what the norm or the matmul before wrote)
-        assert lhs.cols == K and G > 1
+    if lhs_tiled:  # (rows in tiles of 16 x 32, what the norm or the matmul before wrote)
+        assert lhs.cols == K
         M = rows if rows is not None else lhs.rows
         lhs_t = lhs.data
     else:
@@ -376,7 +388,7 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     assert group_sizes.dtype == torch.int32 and group_sizes.numel() == G
     NO = N // 2 if fused_swiglu else N
     if out_tiled:
-        assert not out_f32 and residual is None and G > 1 and NO % 32 == 0
+        assert not out_f32 and residual is None and NO % 32 == 0
         out_obj = Tiled16.empty(M, NO, dev)
         out = out_obj.data
     else:
@@ -392,10 +404,17 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     ws = _lib.workspace("gemm", dev, stream, need)
     rc = _L.lyra_decode_gemm_ex(lhs_t.data_ptr(), _ptr(row_map), rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
                                 _ptr(residual), 1.0 if out_scale is None else float(out_scale),
-                                int(out_scale is not None) | (2 if bias_after_cast else 0) | (4 if lhs_tiled else 0) | (8 if out_tiled else 0),
-                                out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N, rd,
+                                int(out_scale is not None) | (2 if bias_after_cast else 0),
+                                out.data_ptr(), ws.data_ptr(), ws.numel(), M, G, K, N,
+                                rd | (_lib.LHS_TILED16 if lhs_tiled else 0) | (_lib.OUT_TILED16 if out_tiled else 0),
                                 _lib.DTYPE_F32 if out_f32 else _lib.DTYPE_BF16, int(fused_swiglu), float(swiglu_beta),
                                 float(swiglu_limit), stream)
+    if rc == _lib.E_UNSUPPORTED and (lhs_tiled or out_tiled):
+        # (a plan without tiled activations, e.g. one group with more rows than the K-split kernel takes: through row-major copies)
+        res = gemm(lhs.untiled().contiguous() if lhs_tiled else lhs, rhs, group_sizes, rows=rows, row_map=row_map, residual=residual,
+                   out_scale=out_scale, fused_swiglu=fused_swiglu, swiglu_beta=swiglu_beta, swiglu_limit=swiglu_limit, out_f32=out_f32,
+                   bias=bias, bias_after_cast=bias_after_cast)
+        return tile16(res) if out_tiled else res
     if rc == _lib.E_UNSUPPORTED and isinstance(rhs, SpanMajor) and rhs.fallback is not None:
         # (a shape whose plan has no span-major kernel, e.g. one group with too many rows for the K-split kernel)
         return gemm(lhs, rhs.fallback, group_sizes, rows=rows, row_map=row_map, residual=residual, out_scale=out_scale,

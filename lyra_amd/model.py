@@ -487,12 +487,13 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     from lyra_amd.kernels import decode_fused as F
 
     H, N, K = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
+    tiled = _TILED_ACTIVATIONS and cfg.n_embd % 32 == 0  # (the normalised rows only feed the q/k/v projection: 16 x 32 tiles)
     if isinstance(x, TokenRows):  # first layer of a step: the embedding rows are gathered by the norm kernel
-        h, gate, x = F.embed_rmsnorm_proj(x.table, x.tokens, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+        h, gate, x = F.embed_rmsnorm_proj(x.table, x.tokens, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True, tiled=tiled)
     elif isinstance(x, (F.Unsummed, F.Uncombined)):
-        h, gate, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+        h, gate, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True, tiled=tiled)
     else:
-        h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True)
+        h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True, tiled=tiled)
     B = x.shape[0]
     one = _one_group(B, x.device)
     w_qkv, w_out = F.span_major(w.qkv), F.span_major(w.out)  # (the arrays themselves unless their rows straddle cache lines)
@@ -552,14 +553,15 @@ def moe_apply_fused(x, w: MoEWeights, cfg: ModelConfig, groups_out: list | None 
 def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     from lyra_amd.kernels import decode_fused as F
 
+    tiled = _TILED_ACTIVATIONS and cfg.n_embd % 32 == 0 and cfg.dense_hidden % 32 == 0
     if isinstance(x, (F.Unsummed, F.Uncombined)):
-        t, _, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
+        t, _, x = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, tiled=tiled)
     else:
-        t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps)
+        t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, tiled=tiled)
     one = _one_group(x.shape[0], x.device)
     w_up, w_down = F.span_major(w.mlp_up), F.span_major(w.mlp_down)
     t = F.gemm(t, w_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
-               bias=_bf16_bias(w.mlp_up_bias))
+               bias=_bf16_bias(w.mlp_up_bias), out_tiled=tiled)
     if w.mlp_down_bias is not None:  # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result
         return F.gemm(t, w_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=True, residual=x,
                       out_scale=cfg.dense_residual_scale)

@@ -664,9 +664,12 @@ def _tile16(x: torch.Tensor):
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("M,G,K,N,swiglu,gather", [(300, 16, 512, 4096, True, True), (300, 16, 2048, 2048, False, False),
                                                      (11, 4, 512, 512, True, True), (130, 3, 320, 2880, False, False),
-                                                     (256, 16, 2048, 4096, True, True)])
+                                                     (256, 16, 2048, 4096, True, True),
+                                                     # one group: the K-split projections (their finish step writes the tiles)
+                                                     (67, 1, 2048, 6144, True, False), (67, 1, 3072, 2048, False, False),
+                                                     (36, 1, 2880, 5120, False, False), (131, 1, 4096, 4096, False, False)])
 def test_expert_matmul_reads_and_writes_activations_in_tiles(fp8, M, G, K, N, swiglu, gather):
-    """post_scale bits 2 and 3 of lyra_decode_gemm_ex: activations in tiles of 16 rows x 32 columns in, and out.  Only
+    """LYRA_LHS_TILED16 / LYRA_OUT_TILED16 of lyra_decode_gemm_ex: activations in tiles of 16 rows x 32 columns in, and out.  Only
     addresses change, so the result is the row-major call's bit for bit - with the token gather, with span-major weights,
     and with rows past the last group."""
     from lyra_amd.kernels import decode_fused as F
@@ -696,9 +699,12 @@ def test_expert_matmul_reads_and_writes_activations_in_tiles(fp8, M, G, K, N, sw
     if NO % 32 == 0:
         got_out = F.gemm(_tile16(x), w, gs, out_tiled=True, **kw)
         assert isinstance(got_out, F.Tiled16) and torch.equal(got_out.untiled(), want), "tiled output"
-        packed = F.pack_weights(w, glu=swiglu)
+        packed = F.pack_weights(w, glu=swiglu and G > 1)
         got_pk = F.gemm(_tile16(x), packed, gs, out_tiled=True, **kw)
         assert torch.equal(got_pk.untiled(), F.gemm(x, packed, gs, **kw)), "tiled, span-major weights"
+    if G == 1 and not swiglu and N % 128 == 0:  # the unsummed slices of a projection, from tiled rows
+        a, b = F.gemm_unsummed(x[:M], w, gs), F.gemm_unsummed(_tile16(x[:M]), w, gs)
+        assert (a is None) == (b is None) and (a is None or torch.equal(a.partials, b.partials))
 
 
 @pytest.mark.parametrize("B,C,n", [(64, 2048, 15), (5, 256, 7), (128, 4096, 63), (33, 2880, 32)])
