@@ -275,7 +275,9 @@ def time_expert_matmuls(dev, one_step, stream, rounds=10):
     lyra-medium MoE layer (benchmark configuration 3: width 4096, 31 routed + 1 shared experts of hidden 4096, 64 tokens,
     3 routed experts per token drawn from Zipf(1.1) + the shared one, seeded) and at the shape of the lyra-small layer the
     step itself runs (15 + 1 experts, width 2048, hidden 2048).  FP8 weights, one scale per output channel.  The group
-    sizes are the instances `--kernels` times as "lyra-medium expert ... T=64" and "lyra-small expert ... B=64"."""
+    sizes are the instances `--kernels` times as "lyra-medium expert ... T=64" and "lyra-small expert ... B=64".  The launches
+    are the decode step's: lyra_decode_gemm_ex with the activations in tiles of 16 rows x 32 columns, as the norm in front
+    of the up projection and the up projection itself leave them (LYRA_LHS_TILED16 / LYRA_OUT_TILED16)."""
     import numpy as np
     import torch
 
@@ -294,16 +296,18 @@ def time_expert_matmuls(dev, one_step, stream, rounds=10):
         for name, K, N, swiglu in (("up+SwiGLU", C, 2 * Hd, True), ("down", Hd, C, False)):
             w = torch.randint(0, 0x78, (E, K, N), generator=gen, device=dev, dtype=torch.uint8)
             sc = torch.rand(E, 1, N, generator=gen, device=dev) * 0.001 + 0.0005
-            lhs = x if K == C else torch.randn(M, K, generator=gen, device=dev, dtype=torch.bfloat16)
-            out = torch.empty(M, N // 2 if swiglu else N, device=dev, dtype=torch.bfloat16)
+            # (random values: the tiled layout is a permutation of the same bytes, rows rounded up to 16)
+            lhs = torch.randn((M + 15) // 16 * 16, K, generator=gen, device=dev, dtype=torch.bfloat16)
+            out = torch.empty((M + 15) // 16 * 16, N // 2 if swiglu else N, device=dev, dtype=torch.bfloat16)
             ws = torch.zeros(max(L.lyra_decode_gemm_workspace(M, E, K, N, int(swiglu)), 256), dtype=torch.uint8, device=dev)
-            nbytes = touched * (K * N + N * 4) + M * K * 2 + out.numel() * 2
+            nbytes = touched * (K * N + N * 4) + M * K * 2 + M * (N // 2 if swiglu else N) * 2
+            flags = _lib.LHS_TILED16 | (_lib.OUT_TILED16 if swiglu else 0)
 
-            def launch(lhs=lhs, w=w, sc=sc, out=out, ws=ws, K=K, N=N, swiglu=swiglu):
-                rc = L.lyra_decode_gemm(lhs.data_ptr(), w.data_ptr(), sc.data_ptr(), K, 1, gs.data_ptr(), None, out.data_ptr(),
-                                        ws.data_ptr(), ws.numel(), M, E, K, N, _lib.DTYPE_E4M3FN, _lib.DTYPE_BF16, int(swiglu),
-                                        1.702, 7.0, stream.cuda_stream)
-                _lib.check(rc, "lyra_decode_gemm")
+            def launch(lhs=lhs, w=w, sc=sc, out=out, ws=ws, K=K, N=N, swiglu=swiglu, flags=flags):
+                rc = L.lyra_decode_gemm_ex(lhs.data_ptr(), None, w.data_ptr(), sc.data_ptr(), K, 1, gs.data_ptr(), None, None, 1.0, 0,
+                                           out.data_ptr(), ws.data_ptr(), ws.numel(), M, E, K, N, _lib.DTYPE_E4M3FN | flags,
+                                           _lib.DTYPE_BF16, int(swiglu), 1.702, 7.0, stream.cuda_stream)
+                _lib.check(rc, "lyra_decode_gemm_ex")
 
             cases.append((f"{label} expert {name} ({E}x{K}x{N} fp8), 64 tokens, {touched} experts with rows", nbytes, launch, []))
         for r in range(rounds + 2):  # the first two rounds warm up
@@ -318,7 +322,7 @@ def time_expert_matmuls(dev, one_step, stream, rounds=10):
         stream.synchronize()
         for case, nbytes, _, pairs in cases:
             t = sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / len(pairs)
-            out_rows.append({"kernel": "decode_gemm_group_kernel<fp8>", "case": case, "bound": "hbm", "achieved": nbytes / t / 1e9,
+            out_rows.append({"kernel": "decode_gemm_group_kernel<fp8> (tiled activations, as in the decode step)", "case": case, "bound": "hbm", "achieved": nbytes / t / 1e9,
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
                              "algorithmic_bytes": nbytes, "us_per_launch": t * 1e6})
         del cases
@@ -369,7 +373,7 @@ def zipf_group_sizes(rng, tokens, n_routed, k_routed, n_shared):
     return np.bincount(ids.reshape(-1), minlength=n_routed + n_shared).astype(np.int32)
 
 
-def kernel_table(dev, only="", span_major=False):
+def kernel_table(dev, only="", span_major=False, tiled=False):
     """Stand-alone timings of the two operators through the C ABI at the shapes of the named model variants: HIP events
     over back-to-back launches, once rotating over enough distinct caches / weight sets that every launch streams from
     HBM ("cold") and once re-using one set ("hot", which the 256 MB last-level cache may serve in part)."""
@@ -455,9 +459,13 @@ def kernel_table(dev, only="", span_major=False):
 
         dt = _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16
         flag = 0
+        if tiled and N < 100000 and K % 32 == 0:  # activations in tiles of 16 rows x 32 columns, as the fused decode step hands them over
+            flag |= _lib.LHS_TILED16
+            lhs = torch.randn((M + 15) // 16 * 16, K, generator=gen, device=dev, dtype=torch.bfloat16)
+            label += " [tiled activations]"
         if span_major and N < 100000:  # the weights in the span-major copy lyra_gemm_pack makes (not for the LM head's kernel)
             layout = 2 if (swiglu and G > 1) else 1
-            flag = _lib.RHS_SPAN_MAJOR if layout == 1 else _lib.RHS_SPAN_MAJOR_GLU
+            flag |= _lib.RHS_SPAN_MAJOR if layout == 1 else _lib.RHS_SPAN_MAJOR_GLU
             packed = []
             for w in weights:
                 buf = torch.empty(L.lyra_gemm_packed_bytes(G, K, N, dt, layout), dtype=torch.uint8, device=dev)
@@ -612,6 +620,8 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the decode step, time both operators stand-alone at the shapes of every model variant")
     ap.add_argument("--only", default="", help="with --kernels: only the cases whose name contains this text")
+    ap.add_argument("--tiled", action="store_true",
+                    help="with --kernels: the matmuls read their activations in tiles of 16 rows x 32 columns (LYRA_LHS_TILED16)")
     ap.add_argument("--span-major", action="store_true",
                     help="with --kernels: the matmuls read the span-major copy of their weights (lyra_gemm_pack)")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -625,7 +635,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.kernels:
-        rows = kernel_table(dev, args.only, args.span_major)
+        rows = kernel_table(dev, args.only, args.span_major, args.tiled)
         if args.traffic_probe:
             traffic_probe(dev)
         for r in rows:

@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 12
+#define LYRA_ABI_VERSION 13
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -364,6 +364,28 @@ size_t lyra_sample_topk_workspace(int rows, int cols, int k);
  */
 int lyra_sample_topk_rng(const float* x, uint64_t* rng, int32_t* out, void* workspace, size_t workspace_bytes, int rows, int cols,
                          int ld, int k, float temperature, int32_t* advance, lyra_stream_t stream);
+/*
+ * Samplers for logits whose matmul also left the maximum of every 128-column tile of every row.
+ * lyra_decode_gemm_tile_max is lyra_decode_gemm_ex without the residual / scale epilogue and without SwiGLU, for the
+ * shapes its plain kernel takes (one group whose weights are too many for the K-split kernel - the LM head,
+ * lyra/model.py:784-790 - float32 output): besides `out` it writes tile_max [M, (N + 127) / 128] float32, the maximum
+ * of out[row, 128 t .. 128 t + 127] with the bias added, NaNs skipped; LYRA_E_UNSUPPORTED for any other shape (call
+ * lyra_decode_gemm_ex and the samplers above).  lyra_argmax_tiles / lyra_sample_topk_tiles return what lyra_argmax /
+ * lyra_sample_topk (uniforms given, rng null) / lyra_sample_topk_rng (rng given, uniforms null) return on the same
+ * logits, from one launch of one workgroup per row that reads the row's tile maxima and only the tiles that can hold
+ * its k best values: 64 x 201088 logits in 6 us instead of 27.  tile_ld: row pitch of tile_max (>= (cols + 127) / 128).
+ * The workspace is only used with rng (lyra_sample_topk_workspace bytes, may be the one lyra_sample_topk_rng uses).
+ * The logits must be as the matmul left them.
+ */
+int lyra_decode_gemm_tile_max(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk, int bn,
+                              const int32_t* group_sizes, const float* bias, void* out, float* tile_max, void* workspace,
+                              size_t workspace_bytes, int M, int G, int K, int N, int rhs_dtype, int out_dtype,
+                              lyra_stream_t stream);
+int lyra_argmax_tiles(const float* x, const float* tile_max, int32_t* out, int rows, int cols, int ld, int tile_ld,
+                      int32_t* advance, lyra_stream_t stream);
+int lyra_sample_topk_tiles(const float* x, const float* tile_max, const float* uniforms, uint64_t* rng, int32_t* out,
+                           void* workspace, size_t workspace_bytes, int rows, int cols, int ld, int tile_ld, int k,
+                           float temperature, int32_t* advance, lyra_stream_t stream);
 
 
 /*

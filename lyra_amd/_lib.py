@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
 RHS_SPAN_MAJOR, RHS_SPAN_MAJOR_GLU = 0x100, 0x200  # LYRA_RHS_SPAN_MAJOR(_GLU): OR-ed into a matmul's rhs_dtype
 LHS_TILED16, OUT_TILED16 = 0x400, 0x800  # LYRA_LHS_TILED16 / LYRA_OUT_TILED16, likewise
-ABI_VERSION = 12
+ABI_VERSION = 13
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 
 _c = ctypes
@@ -87,6 +87,15 @@ SIGNATURES = {
     "lyra_sample_topk": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p, _c.c_void_p]),
     "lyra_sample_topk_rng": (_c.c_int, [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p, _c.c_void_p]),
     "lyra_sample_topk_workspace": (_c.c_size_t, [_c.c_int] * 3),
+    "lyra_decode_gemm_tile_max": (
+        _c.c_int,
+        [_c.c_void_p] * 4 + [_c.c_int] * 2 + [_c.c_void_p] * 5 + [_c.c_size_t] + [_c.c_int] * 6 + [_c.c_void_p],
+    ),
+    "lyra_argmax_tiles": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_int] * 4 + [_c.c_void_p] * 2),
+    "lyra_sample_topk_tiles": (
+        _c.c_int,
+        [_c.c_void_p] * 6 + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float, _c.c_void_p, _c.c_void_p],
+    ),
     "lyra_selftest": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
 }
 

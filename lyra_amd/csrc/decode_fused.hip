@@ -661,6 +661,44 @@ __device__ __forceinline__ void topk_merge(float (&tv)[kMaxSampleK], int (&ti)[k
     }
 }
 
+// Softmax of logits / temperature over a row's K candidates (best first, a candidate without an index ends the list),
+// inverse CDF at the row's uniform number.  (K at compile time: the exponentials stay in registers.)
+template <int K>
+__device__ __forceinline__ int draw_token(const float* cand_v, const int* cand_i, float temperature, float u) {
+    float e[K], total = 0.f;
+    const float top = cand_v[0] / temperature;
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        const bool have = n == j && cand_i[j] != 0x7FFFFFFF;
+        e[j] = have ? expf(cand_v[j] / temperature - top) : 0.f;
+        if (have) {
+            total += e[j];
+            n = j + 1;
+        }
+    }
+    const float target = u * total;
+    float run = 0.f;
+    int pick = 0;
+    bool found = false;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        if (j < n) {
+            if (!found) pick = cand_i[j];  // (the last candidate when the number lies beyond every partial sum)
+            run += e[j];
+            found = found || target < run;
+        }
+    }
+    return pick;
+}
+
+// The uniform number of (seed, draw, row): 24 bits of a splitmix64 of the three.
+__device__ __forceinline__ float rng_uniform(const unsigned long long* rng, unsigned long long draw, int row) {
+    const unsigned long long seed = __hip_atomic_load(&rng[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long z = splitmix64(seed ^ ((draw + 1) * 0x9E3779B97F4A7C15ull) ^ ((unsigned long long)(row + 1) * 0xD1B54A32D192ED03ull));
+    return (float)(z >> 40) * 0x1p-24f;
+}
+
 template <int K>
 __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
     __shared__ float sm_wv[4], sm_tv[kMaxSampleK];
@@ -760,36 +798,216 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(SampleParams p) {
     }
     topk_merge<K>(tv, ti, 256, sm_wv, sm_wi, sm_tv, sm_ti);
     if (threadIdx.x == 0) {
-        // softmax of logits / temperature over the candidates (best first), inverse CDF at the row's uniform number
-        float e[kMaxSampleK], total = 0.f;
-        const float top = sm_tv[0] / p.temperature;
-        int n = 0;
-        for (int j = 0; j < k; ++j) {
-            if (sm_ti[j] == 0x7FFFFFFF) break;
-            e[j] = expf(sm_tv[j] / p.temperature - top);
-            total += e[j];
-            n = j + 1;
+        p.out[row] = draw_token<K>(sm_tv, sm_ti, p.temperature, p.rng ? rng_uniform(p.rng, draw, row) : p.uniforms[row]);
+        if (p.advance && row == 0) *p.advance += 1;
+    }
+}
+
+// ---- the two samplers over logits whose producer also left the maximum of every 128-column tile ------------------
+// (GemmParams::tile_max of the matmul that wrote them.)  One workgroup per row reads the row's tile maxima - 1571 numbers
+// for 201088 logits - and then only the tiles that can hold what it looks for: the first tile with the row maximum
+// (greedy), or the tiles whose maximum reaches the k-th largest tile maximum (k tiles, unless values repeat).  Results are
+// those of argmax_kernel / sample_topk_kernel on the same logits.
+struct TileSampleParams {
+    const float* x;
+    const float* tile_max;  // [rows, tile_ld]
+    const float* uniforms;
+    int32_t* out;
+    int rows, cols, ld, tile_ld;
+    float temperature;
+    int32_t* advance;
+    unsigned long long* rng;
+    int* arrivals_all;
+};
+
+// Maximum of tile t over the row's first `cols` columns: the producer's number, or - the one tile that `cols` cuts - a
+// walk over its valid columns.
+__device__ __forceinline__ float tile_value(const float* tm, const float* xr, int t, int cols) {
+    if (128 * t + 128 <= cols) return tm[t];
+    float m = -INFINITY;
+    for (int c = 128 * t; c < cols; ++c) m = fmaxf(m, xr[c]);
+    return m;
+}
+
+__global__ __launch_bounds__(256) void argmax_tiles_kernel(TileSampleParams p) {
+    __shared__ float sm_v[4];
+    __shared__ int sm_i[4];
+    const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const float* xr = p.x + (size_t)row * p.ld;
+    const float* tm = p.tile_max + (size_t)row * p.tile_ld;
+    const int n_tiles = (p.cols + 127) >> 7;
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int t = threadIdx.x; t < n_tiles; t += 256) take_better(bv, bi, tile_value(tm, xr, t, p.cols), t);
+    wave_best(bv, bi, [](float& v, int& i, float ov, int oi) { take_better(v, i, ov, oi); });
+    if (lane == 0) {
+        sm_v[wave] = bv;
+        sm_i[wave] = bi;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    for (int w = 1; w < 4; ++w) take_better(bv, bi, sm_v[w], sm_i[w]);
+    // the first tile that holds the row maximum: its first column with that value
+    const int tile = bi;
+    bv = -INFINITY;
+    bi = 0x7FFFFFFF;
+    if (tile != 0x7FFFFFFF && lane < 32) {
+        const int c0 = 128 * tile + 4 * lane;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (c0 + q < p.cols) take_better(bv, bi, xr[c0 + q], c0 + q);
+    }
+    wave_best(bv, bi, [](float& v, int& i, float ov, int oi) { take_better(v, i, ov, oi); });
+    if (lane == 0) {
+        p.out[row] = bi == 0x7FFFFFFF ? 0 : bi;
+        if (p.advance && row == 0) *p.advance += 1;
+    }
+}
+
+constexpr int kTileList = 1024;  // tiles a workgroup lists for a closer look; more (many equal logits): a slower walk
+
+// The tile maxima that thread `tid` looks at in one batch: tiles base + tid + 256 j, j < 8 (-inf past the last tile).
+// All eight are requested before any is used; the one tile that `cols` cuts is walked by its owner.
+__device__ __forceinline__ void load_tile_values(float (&m)[8], const float* tm, const float* xr, int base, int n_tiles, int cols) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int t = base + (int)threadIdx.x + 256 * j;
+        const float v = tm[min(t, n_tiles - 1)];
+        m[j] = t < n_tiles ? v : -INFINITY;
+    }
+    if (cols & 127) {
+        const int cut = cols >> 7, rel = cut - base - (int)threadIdx.x;
+        if (rel >= 0 && rel < 2048 && (rel & 255) == 0) {
+            const float v = tile_value(tm, xr, cut, cols);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (rel == 256 * j) m[j] = v;
         }
-        float u;
-        if (p.rng) {
-            const unsigned long long seed = __hip_atomic_load(&p.rng[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const unsigned long long z = splitmix64(seed ^ ((draw + 1) * 0x9E3779B97F4A7C15ull) ^ ((unsigned long long)(row + 1) * 0xD1B54A32D192ED03ull));
-            u = (float)(z >> 40) * 0x1p-24f;
-        } else {
-            u = p.uniforms[row];
-        }
-        const float target = u * total;
-        float run = 0.f;
-        int pick = n > 0 ? sm_ti[n - 1] : 0;
-        for (int j = 0; j < n; ++j) {
-            run += e[j];
-            if (target < run) {
-                pick = sm_ti[j];
-                break;
+    }
+}
+
+constexpr int kCandMax = 256;  // values a workgroup collects for the final ranking; more (many equal logits): the slower walk
+
+template <int K>
+__global__ __launch_bounds__(256) void sample_tiles_kernel(TileSampleParams p) {
+    __shared__ float sm_wv[4], sm_tv[kMaxSampleK], sm_g[16], sm_cv[kCandMax];
+    __shared__ int sm_wi[4], sm_ti[kMaxSampleK], sm_ci[kCandMax];
+    __shared__ int sm_list[kTileList];
+    __shared__ int sm_count, sm_ncand;
+    __shared__ float sm_floor;
+    const int tid = threadIdx.x, row = blockIdx.x, wave = tid >> 6, lane = tid & 63;
+    // (the draw count is read before this workgroup is counted as arrived, and replaced only after all have been)
+    const unsigned long long draw = (p.rng && tid == 0) ? __hip_atomic_load(&p.rng[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+    const float* xr = p.x + (size_t)row * p.ld;
+    const float* tm = p.tile_max + (size_t)row * p.tile_ld;
+    const int n_tiles = (p.cols + 127) >> 7;
+    const bool one_batch = n_tiles <= 2048;  // (then the second look still holds the first one's values)
+    if (tid == 0) sm_count = sm_ncand = 0;
+    if (tid < kMaxSampleK) {
+        sm_tv[tid] = -INFINITY;
+        sm_ti[tid] = 0x7FFFFFFF;
+    }
+    // A lower bound of the row's K-th best value: the K-th largest of the 16 maxima that groups of 16 threads find
+    // among their tiles - K different tiles hold a value at least that large.  (Not the K-th largest tile maximum itself:
+    // that costs K rounds over the workgroup, this costs one, and lists a few tiles more.)
+    float m[8], mine = -INFINITY;
+    for (int base = 0; base < n_tiles; base += 2048) {
+        load_tile_values(m, tm, xr, base, n_tiles, p.cols);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mine = fmaxf(mine, m[j]);
+    }
+    mine = row16_max(mine);
+    if ((tid & 15) == 0) sm_g[tid >> 4] = mine;
+    __syncthreads();
+    int seen = 0;
+    if (p.rng && tid == 0) {  // (its own read of the count has returned: every load above has)
+        wait_all_memory();
+        seen = add_agent(p.arrivals_all, 1);
+    }
+    if (tid < 16) {
+        const float v = sm_g[tid];
+        int rank = 0;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) rank += (sm_g[j] > v || (sm_g[j] == v && j < tid)) ? 1 : 0;
+        if (rank == K - 1) sm_floor = v;  // (-inf when fewer than K groups hold a finite value: every tile is looked at)
+    }
+    __syncthreads();
+    const float floor_v = sm_floor;
+    for (int base = 0; base < n_tiles; base += 2048) {
+        if (!one_batch) load_tile_values(m, tm, xr, base, n_tiles, p.cols);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int t = base + tid + 256 * j;
+            if (t < n_tiles && m[j] >= floor_v) {
+                const int slot = atomicAdd(&sm_count, 1);
+                if (slot < kTileList) sm_list[slot] = t;
             }
         }
-        p.out[row] = pick;
+    }
+    __syncthreads();
+    const int count = sm_count;
+    bool ranked = false;
+    if (count <= kTileList) {  // a wavefront per listed tile, 32 lanes x 4 columns: values >= the bound go on a list
+        const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(xr), 0, (uint32_t)p.cols * 4u, 0x00020000);
+        for (int e = wave; e < count; e += 4) {
+            const int c0 = 128 * sm_list[e] + 4 * (lane & 31);
+            const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, c0 * 4, 0, 0);  // (past `cols`: zeros, unused)
+            if (lane < 32) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float v = __uint_as_float(raw[q]);
+                    if (c0 + q < p.cols && v >= floor_v) {
+                        const int slot = atomicAdd(&sm_ncand, 1);
+                        if (slot < kCandMax) {
+                            sm_cv[slot] = v;
+                            sm_ci[slot] = c0 + q;
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int ncand = sm_ncand;
+        if (ncand <= kCandMax) {  // rank by counting: how many candidates come before mine
+            if (tid < ncand) {
+                const float v = sm_cv[tid];
+                const int i = sm_ci[tid];
+                int rank = 0;
+                for (int j = 0; j < ncand; ++j) rank += better(sm_cv[j], sm_ci[j], v, i) ? 1 : 0;
+                if (rank < K) {
+                    sm_tv[rank] = v;
+                    sm_ti[rank] = i;
+                }
+            }
+            ranked = true;
+            __syncthreads();
+        }
+    }
+    if (!ranked) {  // many equal values: every thread walks the tiles it looked at and keeps its K best, then K rounds
+        float tv[kMaxSampleK];
+        int ti[kMaxSampleK];
+#pragma unroll
+        for (int j = 0; j < kMaxSampleK; ++j) {
+            tv[j] = -INFINITY;
+            ti[j] = 0x7FFFFFFF;
+        }
+        for (int t = tid; t < n_tiles; t += 256) {
+            if (!(tile_value(tm, xr, t, p.cols) >= floor_v)) continue;
+            for (int c = 128 * t; c < min(128 * t + 128, p.cols); ++c) {
+                const float v = xr[c];
+                if (v >= floor_v) topk_insert<K>(tv, ti, v, c);
+            }
+        }
+        __syncthreads();
+        topk_merge<K>(tv, ti, 256, sm_wv, sm_wi, sm_tv, sm_ti);
+    }
+    if (tid == 0) {
+        p.out[row] = draw_token<K>(sm_tv, sm_ti, p.temperature, p.rng ? rng_uniform(p.rng, draw, row) : p.uniforms[row]);
         if (p.advance && row == 0) *p.advance += 1;
+        if (p.rng && seen == (int)gridDim.x - 1) {  // every workgroup has read the count
+            store_agent(p.arrivals_all, 0);
+            __hip_atomic_store(&p.rng[1], draw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -978,6 +1196,41 @@ extern "C" int lyra_sample_topk_rng(const float* x, uint64_t* rng, int32_t* out,
     if (!rng || ((uintptr_t)rng % 8)) return LYRA_E_BADARG;
     return lyra::run_sample_topk(x, nullptr, (unsigned long long*)rng, out, workspace, workspace_bytes, rows, cols, ld, k, temperature,
                                  advance, stream);
+}
+
+extern "C" int lyra_argmax_tiles(const float* x, const float* tile_max, int32_t* out, int rows, int cols, int ld, int tile_ld,
+                                 int32_t* advance, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!x || !tile_max || !out || rows <= 0 || cols <= 0 || ld < cols || tile_ld < (cols + 127) / 128) return LYRA_E_BADARG;
+    TileSampleParams p{x, tile_max, nullptr, out, rows, cols, ld, tile_ld, 0.f, advance, nullptr, nullptr};
+    hipLaunchKernelGGL(argmax_tiles_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
+extern "C" int lyra_sample_topk_tiles(const float* x, const float* tile_max, const float* uniforms, uint64_t* rng, int32_t* out,
+                                      void* workspace, size_t workspace_bytes, int rows, int cols, int ld, int tile_ld, int k,
+                                      float temperature, int32_t* advance, lyra_stream_t stream) {
+    using namespace lyra;
+    if (!x || !tile_max || !out || rows <= 0 || cols <= 0 || ld < cols || tile_ld < (cols + 127) / 128 || k <= 0 || !(temperature > 0.f))
+        return LYRA_E_BADARG;
+    if ((uniforms != nullptr) == (rng != nullptr) || ((uintptr_t)rng % 8)) return LYRA_E_BADARG;  // one source of uniform numbers
+    if (k > kMaxSampleK || ld % 4 || ((uintptr_t)x % 16)) return LYRA_E_UNSUPPORTED;
+    // (the generator's launch counter lives where lyra_sample_topk_rng keeps its own: the two may share a workspace)
+    if (rng && (!workspace || workspace_bytes < kArgmaxCounterBytes || ((uintptr_t)workspace % 256))) return LYRA_E_WORKSPACE;
+    TileSampleParams p{x, tile_max, uniforms, out, rows, cols, ld, tile_ld, temperature, advance, (unsigned long long*)rng,
+                       rng ? (int*)workspace + 65535 : nullptr};
+    const dim3 grid(rows), block(256);
+    switch (std::min(k, cols)) {
+        case 1: hipLaunchKernelGGL(sample_tiles_kernel<1>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 2: hipLaunchKernelGGL(sample_tiles_kernel<2>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 3: hipLaunchKernelGGL(sample_tiles_kernel<3>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 4: hipLaunchKernelGGL(sample_tiles_kernel<4>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 5: hipLaunchKernelGGL(sample_tiles_kernel<5>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 6: hipLaunchKernelGGL(sample_tiles_kernel<6>, grid, block, 0, (hipStream_t)stream, p); break;
+        case 7: hipLaunchKernelGGL(sample_tiles_kernel<7>, grid, block, 0, (hipStream_t)stream, p); break;
+        default: hipLaunchKernelGGL(sample_tiles_kernel<8>, grid, block, 0, (hipStream_t)stream, p); break;
+    }
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
 
 namespace lyra {

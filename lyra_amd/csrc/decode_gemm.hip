@@ -58,6 +58,11 @@ struct GemmParams {
     // one matrix instruction with 16 consecutive rows then read one contiguous KB instead of 16 pieces a row apart.
     // lhs_tiled: lhs comes in that layout (grouped kernel); out_tiled: the bf16 output is written in it (for the next matmul).
     int lhs_tiled, out_tiled;
+    // Plain kernel, one group, float32 output, K not split: the maximum of every 128-column tile of every output row,
+    // [M, tile_ld] float32 (tile t = columns 128 t ...; NaNs are skipped as fmaxf skips them), for a sampler that then
+    // only looks into the few tiles that can hold a row's best values.  Null: not wanted.
+    float* tile_max;
+    int tile_ld;
 };
 
 // Element index of output (row, col .. col + 3) in an array of NO columns, row-major or tiled (GemmParams::out_tiled).
@@ -241,7 +246,17 @@ __device__ __forceinline__ void finish_row(const GemmParams& p, float (&t)[8], c
     }
 }
 
-template <bool FP8, int MT>
+// GemmParams::tile_max: the 16 lanes that hold the 128 columns of one row of a span reduce their finished values (t as
+// finish_row left it: bias added) and lane 0 of them (`writer`) stores the maximum.  Called by all lanes.
+__device__ __forceinline__ void store_tile_max(const GemmParams& p, const float (&t)[8], int row, int span, bool lane_ok, bool writer) {
+    float m = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])), fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
+    m = row16_max(lane_ok ? m : -INFINITY);
+    if (writer) p.tile_max[(size_t)row * p.tile_ld + span] = m;
+}
+
+constexpr int kTileMaxPitch = 20;  // floats per row of a wavefront's tile-maximum staging area (conflict-free for 4 rows x 16 lanes)
+
+template <bool FP8, int MT, bool TMAX = false>
 __global__ __launch_bounds__(MT == 1 ? 768 : 512) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 3 : 2)))
 void decode_gemm_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
@@ -259,6 +274,8 @@ void decode_gemm_kernel(GemmParams p) {
     const int first_span = p.even_spans ? (int)((long)blockIdx.x * total_spans / gridDim.x) : (int)blockIdx.x * kGemmWaves;
     const int end_span = p.even_spans ? (int)((long)(blockIdx.x + 1) * total_spans / gridDim.x) : total_spans;
     const int span = first_span + wave;
+    // (TMAX: behind the activations, 16 * MT rows of kTileMaxPitch floats per wavefront)
+    float* const sm_t = (float*)(sm_x + 16 * MT * XPITCH) + wave * (16 * MT * kTileMaxPitch);
 
     // rows of this group: [off, off + cnt)
     int part_sum = 0;
@@ -398,8 +415,28 @@ void decode_gemm_kernel(GemmParams p) {
 #pragma unroll
                     for (int c = 0; c < 8; ++c) t[c] = acc[mt][c][r] * colscale[c];
                     finish_row(p, t, bias8, rowbase + lr, ncol, out_col, ks, span_ok && lr < rows_here, is_lin_lane);
+                    if (TMAX) {  // this lane's 8 columns of the row; the row's 16 lanes meet in LDS below
+                        const float m = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])), fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
+                        sm_t[lr * kTileMaxPitch + x] = span_ok ? m : -INFINITY;
+                    }
                 }
             }
+        }
+        if (TMAX) {
+            // Lane l takes row l of the block: 16 partial maxima, one store.  Only this wavefront touches its staging area
+            // and LDS serves a wavefront's requests in order, so no barrier - the fences keep the compiler from moving
+            // the reads above the writes (or the next block's writes above these reads).
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (lane < 16 * MT) {
+                const f32x4 a = *(const f32x4*)(sm_t + lane * kTileMaxPitch), b = *(const f32x4*)(sm_t + lane * kTileMaxPitch + 4);
+                const f32x4 c = *(const f32x4*)(sm_t + lane * kTileMaxPitch + 8), d = *(const f32x4*)(sm_t + lane * kTileMaxPitch + 12);
+                const float m = fmaxf(fmaxf(fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), fmaxf(fmaxf(b[0], b[1]), fmaxf(b[2], b[3]))),
+                                      fmaxf(fmaxf(fmaxf(c[0], c[1]), fmaxf(c[2], c[3])), fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3]))));
+                if (lane < rows_here && span < end_span) p.tile_max[(size_t)(rowbase + lane) * p.tile_ld + span] = m;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     }
 
@@ -412,6 +449,7 @@ void decode_gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) t[c] = 0.f;
         finish_row(p, t, pad_bias8, row0 + kb, ncol, out_col, ks, span_ok && row0 + kb < p.M, is_lin_lane);
+        if (TMAX) store_tile_max(p, t, row0 + kb, span, span_ok, span < end_span && row0 + kb < p.M && x == 0);
     }
 }
 
@@ -1777,12 +1815,39 @@ extern "C" int lyra_decode_gemm(const void* lhs, const void* rhs, const float* r
                                workspace_bytes, M, G, K, N, rhs_dtype, out_dtype, fused_swiglu, swiglu_beta, swiglu_limit, stream);
 }
 
+namespace lyra {
+static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk, int bn,
+                           const int32_t* group_sizes, const float* bias, const void* residual, float out_scale, int post_scale,
+                           void* out, float* tile_max, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
+                           int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
+                           lyra_stream_t stream);
+}
+
 extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
                                    int bn, const int32_t* group_sizes, const float* bias, const void* residual, float out_scale,
                                    int post_scale, void* out, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
                                    int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
                                    lyra_stream_t stream) {
-    using namespace lyra;
+    return lyra::run_decode_gemm(lhs, lhs_row_map, rhs, rhs_scale, bk, bn, group_sizes, bias, residual, out_scale, post_scale, out,
+                                 nullptr, workspace, workspace_bytes, M, G, K, N, rhs_dtype, out_dtype, fused_swiglu, swiglu_beta,
+                                 swiglu_limit, stream);
+}
+
+extern "C" int lyra_decode_gemm_tile_max(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk,
+                                         int bn, const int32_t* group_sizes, const float* bias, void* out, float* tile_max,
+                                         void* workspace, size_t workspace_bytes, int M, int G, int K, int N, int rhs_dtype,
+                                         int out_dtype, lyra_stream_t stream) {
+    if (!tile_max) return LYRA_E_BADARG;
+    return lyra::run_decode_gemm(lhs, lhs_row_map, rhs, rhs_scale, bk, bn, group_sizes, bias, nullptr, 1.0f, 0, out, tile_max,
+                                 workspace, workspace_bytes, M, G, K, N, rhs_dtype, out_dtype, 0, 0.f, 0.f, stream);
+}
+
+namespace lyra {
+static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const void* rhs, const float* rhs_scale, int bk, int bn,
+                           const int32_t* group_sizes, const float* bias, const void* residual, float out_scale, int post_scale,
+                           void* out, float* tile_max, void* workspace, size_t workspace_bytes, int M, int G, int K, int N,
+                           int rhs_dtype, int out_dtype, int fused_swiglu, float swiglu_beta, float swiglu_limit,
+                           lyra_stream_t stream) {
     const bool bias_post = (post_scale & 2) != 0;  // post_scale: bit 0 the scale / residual epilogue, bit 1 the bias after the cast
     post_scale &= 1;
     const bool lhs_tiled = (rhs_dtype & LYRA_LHS_TILED16) != 0, out_tiled = (rhs_dtype & LYRA_OUT_TILED16) != 0;
@@ -1831,6 +1896,12 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     if (out_tiled && (out_dtype != LYRA_DTYPE_BF16 || residual || (fused_swiglu ? N / 2 : N) % 32)) return LYRA_E_UNSUPPORTED;
     p.lhs_tiled = lhs_tiled;
     p.out_tiled = out_tiled;
+    // tile maxima: what the plain kernel's epilogue can give - every (row, span) finished by one wavefront, in float32
+    if (tile_max && (G != 1 || pl.grouped || pl.split_k || pl.one_pass || pl.ksplit > 1 || fused_swiglu ||
+                     out_dtype != LYRA_DTYPE_F32 || post_scale || bias_post))
+        return LYRA_E_UNSUPPORTED;
+    p.tile_max = tile_max;
+    p.tile_ld = (N + 127) / 128;
     p.lhs = (const uint16_t*)lhs;
     p.rhs = (const uint8_t*)rhs;
     p.scale = rhs_scale;
@@ -1981,8 +2052,19 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
         grid = dim3(kGroupMaxWgs, 1, 1);
         block = dim3(per_cu * 64);
     }
-    const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t);
-#define LYRA_LAUNCH_GEMM(F, T) hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p)
+    const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t) +
+                       (tile_max ? (size_t)(block.x / 64) * 16 * pl.mt * kTileMaxPitch * sizeof(float) : 0);
+#define LYRA_LAUNCH_GEMM(F, T)                                                                                         \
+    do {                                                                                                               \
+        if (tile_max) {                                                                                                \
+            static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_kernel<F, T, true>,            \
+                                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                              \
+            hipLaunchKernelGGL((decode_gemm_kernel<F, T, true>), grid, block, lds, st, p);                             \
+        } else {                                                                                                       \
+            hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p);                                   \
+        }                                                                                                              \
+    } while (0)
     if (fp8) {
         if (pl.mt == 1) LYRA_LAUNCH_GEMM(true, 1);
         else if (pl.mt == 2) LYRA_LAUNCH_GEMM(true, 2);
@@ -2003,6 +2085,7 @@ extern "C" int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, 
     }
     return LYRA_OK;
 }
+}  // namespace lyra
 
 extern "C" int lyra_decode_gemm_splits(int M, int K, int N, int bk) {
     if (M <= 0 || K <= 0 || N <= 0 || K % 32 || N % 128) return 0;

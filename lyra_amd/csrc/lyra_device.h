@@ -198,13 +198,13 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // same butterfly through __shfl_xor goes through LDS six times (~0.3 us each time a small kernel reduces a row).
 template <int CTRL> __device__ __forceinline__ int dpp_row(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, true); }
 template <int CTRL> __device__ __forceinline__ float dpp_row(float x) { return __uint_as_float((uint32_t)dpp_row<CTRL>((int)__float_as_uint(x))); }
-__device__ __forceinline__ float wave_max(float x) {
+__device__ __forceinline__ float row16_max(float x) {  // over the 16 lanes of a row, result in each of them
     x = fmaxf(x, dpp_row<0xB1>(x));   // quad_perm [1, 0, 3, 2]
     x = fmaxf(x, dpp_row<0x4E>(x));   // quad_perm [2, 3, 0, 1]
     x = fmaxf(x, dpp_row<0x141>(x));  // row_half_mirror
-    x = fmaxf(x, dpp_row<0x140>(x));  // row_mirror
-    return group4_max(x);
+    return fmaxf(x, dpp_row<0x140>(x));  // row_mirror
 }
+__device__ __forceinline__ float wave_max(float x) { return group4_max(row16_max(x)); }
 __device__ __forceinline__ float wave_sum(float x) {
     x += dpp_row<0xB1>(x);
     x += dpp_row<0x4E>(x);

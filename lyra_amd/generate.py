@@ -14,11 +14,14 @@ def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Genera
     temperature scaling, top-k masking (lowest index wins ties, like lax.top_k) and a categorical draw.
     ``advance``: an int32 device scalar (the cache position) to increment by one once the tokens are chosen; the HIP
     samplers do it in the same launch."""
+    # tile maxima the LM head left with these logits (model.py: `logits.tile_max`), while the tensor is as it left them
+    tile_max = getattr(logits, "tile_max", None)
+    tile_max = tile_max[0] if tile_max is not None and tile_max[1] == logits._version else None
     if cfg.sample_temperature <= 0:
         if logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and cfg.implementation != "xla":
             from lyra_amd.kernels.decode_fused import argmax
 
-            return argmax(logits, min(cfg.vocab_size, logits.shape[-1]), out, advance)
+            return argmax(logits, min(cfg.vocab_size, logits.shape[-1]), out, advance, tile_max)
         if advance is not None:
             advance += 1
         return _into(out, torch.argmax(logits, dim=-1).to(torch.int32))
@@ -33,7 +36,8 @@ def sample_token(logits: torch.Tensor, cfg: ModelConfig, generator: torch.Genera
             u = rng_state(logits.device)
         else:
             u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=generator)
-        return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]), out, advance)
+        return sample_topk(logits, u, cfg.sample_topk, cfg.sample_temperature, min(cfg.vocab_size, logits.shape[-1]), out, advance,
+                           tile_max)
     if advance is not None:
         advance += 1
     logits = logits.to(torch.float32) / cfg.sample_temperature

@@ -424,6 +424,32 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, *, rows: int | None 
     return out_obj if out_tiled else out
 
 
+def gemm_tile_max(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, bias: torch.Tensor | None = None):
+    """lyra_decode_gemm_tile_max: float32 ``lhs @ rhs (+ bias)`` for one group (the LM head, lyra/model.py:784-790) together
+    with the maximum of every 128-column tile of every result row, which ``argmax`` / ``sample_topk`` take as
+    ``tile_max``.  Returns (out [M, N], tile_max [M, ceil(N / 128)]) or None for a shape the launch does not take."""
+    rv, rs, bk, bn, rd, (G, K, N) = _rhs_args(rhs)
+    if G != 1 or isinstance(rhs, SpanMajor) or not isinstance(lhs, torch.Tensor):
+        return None
+    M = lhs.shape[0]
+    assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
+    assert group_sizes.dtype == torch.int32 and group_sizes.numel() == 1
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N
+    dev = lhs.device
+    out = torch.empty((M, N), dtype=torch.float32, device=dev)
+    tmax = torch.empty((M, (N + 127) // 128), dtype=torch.float32, device=dev)
+    stream = _stream(dev)
+    ws = _lib.workspace("gemm", dev, stream, _L.lyra_decode_gemm_workspace(M, 1, K, N, 0))
+    rc = _L.lyra_decode_gemm_tile_max(lhs.data_ptr(), None, rv.data_ptr(), _ptr(rs), bk, bn, group_sizes.data_ptr(), _ptr(bias),
+                                      out.data_ptr(), tmax.data_ptr(), ws.data_ptr(), ws.numel(), M, 1, K, N, rd, _lib.DTYPE_F32,
+                                      stream)
+    if rc == _lib.E_UNSUPPORTED:
+        return None
+    _lib.check(rc, "lyra_decode_gemm_tile_max")
+    return out, tmax
+
+
 def moe_route(logits: torch.Tensor, n_routed: int, n_shared: int, k_routed: int):
     """Router top-k + softmax + shared experts + stable sort by expert (lyra/model.py:459-491).
     Returns (scores [T,topk] f32, groups [E] i32, row_map [T*topk] i32, dest [T*topk] i32)."""
@@ -454,11 +480,17 @@ def moe_combine(rows: torch.Tensor, scores: torch.Tensor, dest: torch.Tensor, x:
     return out
 
 
+def _check_tile_max(tile_max: torch.Tensor, rows: int, cols: int, device) -> None:
+    assert tile_max.dtype == torch.float32 and tile_max.is_contiguous() and tile_max.device == device
+    assert tile_max.dim() == 2 and tile_max.shape[0] == rows and tile_max.shape[1] >= (cols + 127) // 128
+
+
 def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | None = None,
-           advance: torch.Tensor | None = None) -> torch.Tensor:
+           advance: torch.Tensor | None = None, tile_max: torch.Tensor | None = None) -> torch.Tensor:
     """Greedy token choice (lyra/generate.py:46-53 at temperature 0): first index of each row's maximum over the first
     ``cols`` columns of float32 ``logits`` [rows, ld]; returns int32 [rows].  ``advance``: an int32 device scalar (the
-    cache position) the launch increments by one."""
+    cache position) the launch increments by one.  ``tile_max``: what ``gemm_tile_max`` returned with these logits -
+    the launch then reads those and one tile per row (lyra_argmax_tiles)."""
     rows, ld = logits.shape
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
@@ -466,6 +498,13 @@ def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | No
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
     assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
+    if tile_max is not None:
+        _check_tile_max(tile_max, rows, cols, logits.device)
+        assert advance is None or (advance.dtype == torch.int32 and advance.numel() == 1)
+        rc = _L.lyra_argmax_tiles(logits.data_ptr(), tile_max.data_ptr(), out.data_ptr(), rows, cols, ld, tile_max.shape[1],
+                                  _ptr(advance), stream)
+        _lib.check(rc, "lyra_argmax_tiles")
+        return out
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_argmax_workspace(rows, cols))
     assert advance is None or (advance.dtype == torch.int32 and advance.numel() == 1)
     rc = _L.lyra_argmax(logits.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, _ptr(advance), stream)
@@ -474,12 +513,14 @@ def argmax(logits: torch.Tensor, cols: int | None = None, out: torch.Tensor | No
 
 
 def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperature: float, cols: int | None = None,
-                out: torch.Tensor | None = None, advance: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, advance: torch.Tensor | None = None,
+                tile_max: torch.Tensor | None = None) -> torch.Tensor:
     """Temperature / top-k token choice (lyra/generate.py:46-53 at temperature > 0) for every row of float32 ``logits``
     [rows, ld] over its first ``cols`` columns: softmax of the k largest ``logits / temperature`` (ties to the lower
     index), inverse CDF at ``uniforms`` [rows] in [0, 1); returns int32 [rows].  ``uniforms`` may instead be the
     generator state ``rng_state(seed)`` makes (int64 [2] on the device: seed, draws so far): the launch then makes its own
-    uniform numbers and moves the state on (lyra_sample_topk_rng)."""
+    uniform numbers and moves the state on (lyra_sample_topk_rng).  ``tile_max``: what ``gemm_tile_max`` returned with
+    these logits - same result from the tile maxima and a few tiles per row (lyra_sample_topk_tiles)."""
     rows, ld = logits.shape
     cols = ld if cols is None else cols
     assert logits.dtype == torch.float32 and logits.is_contiguous()
@@ -493,6 +534,14 @@ def sample_topk(logits: torch.Tensor, uniforms: torch.Tensor, k: int, temperatur
     assert out.dtype == torch.int32 and out.is_contiguous() and out.numel() == rows
     stream = _stream(logits.device)
     ws = _lib.workspace("argmax", logits.device, stream, _L.lyra_sample_topk_workspace(rows, cols, k))
+    if tile_max is not None and k <= 8:
+        _check_tile_max(tile_max, rows, cols, logits.device)
+        rc = _L.lyra_sample_topk_tiles(logits.data_ptr(), tile_max.data_ptr(), None if own_rng else uniforms.data_ptr(),
+                                       uniforms.data_ptr() if own_rng else None, out.data_ptr(), ws.data_ptr(), ws.numel(), rows,
+                                       cols, ld, tile_max.shape[1], k, float(temperature), _ptr(advance), stream)
+        if rc != _lib.E_UNSUPPORTED:  # (rows that are not 16-byte aligned: the whole-row sampler below)
+            _lib.check(rc, "lyra_sample_topk_tiles")
+            return out
     fn = _L.lyra_sample_topk_rng if own_rng else _L.lyra_sample_topk
     rc = fn(logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, ld, k,
             float(temperature), _ptr(advance), stream)

@@ -457,6 +457,7 @@ _ONE_GROUP: dict = {}
 _SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tuning override: combine in a launch of its own
 _SEPARATE_QKV_POST = os.environ.get("LYRA_QKV_POST_KERNEL") is not None  # tuning override: QK norm + RoPE + cache append in a launch of its own
 _TILED_ACTIVATIONS = os.environ.get("LYRA_ROW_MAJOR_ACTIVATIONS") is None  # tuning override: expert matmuls read row-major activations
+_LOGIT_TILE_MAX = os.environ.get("LYRA_NO_LOGIT_TILE_MAX") is None  # tuning override: samplers read the whole vocabulary
 
 
 @dataclass
@@ -600,9 +601,18 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     if hidden_out is not None:  # the residual stream after the last layer (the norm kernel completes it on its way)
         hidden_out.append(normed[2] if len(normed) > 2 else h)
     h = normed[0]
-    logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
+    # The LM head also leaves the maximum of every 128-column tile of the logits; they travel with the tensor (with the
+    # version it had when they were taken) and `sample_token` hands them to a sampler that reads a few tiles per row instead
+    # of the whole vocabulary - unless the logits have been written to since.
+    with_max = F.gemm_tile_max(h, model.unemb_t, _one_group(h.shape[0], h.device), bias=model.vocab_mask) if _LOGIT_TILE_MAX else None
+    if with_max is not None:
+        logits = with_max[0]
+    else:
+        logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
     if model.vocab_mask is None:
         logits[:, cfg.vocab_size :] = float("-inf")
+    elif with_max is not None:
+        logits.tile_max = (with_max[1], logits._version)
     if advance:
         cache.pos += 1
     return logits, cache

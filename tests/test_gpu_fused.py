@@ -521,6 +521,105 @@ def test_sampler_with_its_own_generator_follows_the_documented_stream():
         assert torch.equal(out, want) and state.cpu().tolist()[1] == start + rep + 1
 
 
+def _tile_maxima(x: torch.Tensor) -> torch.Tensor:
+    """Maximum of every 128-column tile of every row (the last tile may be short), as lyra_decode_gemm_tile_max leaves them."""
+    rows, n = x.shape
+    pad = torch.full((rows, (n + 127) // 128 * 128), float("-inf"), device=x.device)
+    pad[:, :n] = x
+    return pad.view(rows, -1, 128).amax(dim=2).contiguous()
+
+
+@pytest.mark.parametrize("rows,cols,ld,case", [(64, 201088, 201088, "random"), (64, 201000, 201088, "random"), (3, 1000, 1024, "random"),
+                                               (1, 7, 8, "random"), (5, 4097, 4104, "random"), (130, 50000, 50048, "random"),
+                                               (4, 201088, 201088, "flat"), (6, 3000, 3072, "sparse")])
+def test_tile_samplers_equal_the_full_samplers(rows, cols, ld, case):
+    """lyra_argmax_tiles / lyra_sample_topk_tiles, which read a row's tile maxima and a few tiles, must return what
+    lyra_argmax / lyra_sample_topk / lyra_sample_topk_rng return from the whole row: random logits with planted ties and a
+    fully masked row, `cols` that cuts a tile, "flat" rows (every logit equal or one of two values: more tiles qualify than
+    a workgroup lists) and "sparse" rows (fewer finite values than k)."""
+    from lyra_amd.kernels import decode_fused as F
+
+    _say(f"tile samplers rows{rows} cols{cols} ld{ld} {case}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(rows + cols)
+    x = torch.randn(rows, ld, generator=g, device=dev)
+    if case == "flat":
+        x[0] = 1.5
+        x[1] = torch.where(torch.rand(ld, generator=g, device=dev) < 0.5, 2.0, 1.0)
+        x[2, ::128] = 7.0  # one equal maximum in every tile
+    elif case == "sparse":
+        x[:] = float("-inf")
+        x[0, 5] = 1.0
+        x[1, 129], x[1, 2999] = 2.0, 2.5
+        x[2, 100], x[2, 101], x[2, 102] = 0.5, 0.5, 0.25
+        x[4, :] = torch.randn(ld, generator=g, device=dev)
+    else:
+        x[0, : min(cols, 5)] = 50.0  # ties: the first index wins
+        if rows > 1:
+            x[1, :cols] = float("-inf")
+        if rows > 2:
+            x[2, cols - 1] = 60.0  # the last valid column
+    x[:, cols:] = 100.0  # padding columns must not win (their tiles' maxima say 100)
+    tm = _tile_maxima(x)
+    u = torch.rand(rows, generator=g, device=dev)
+    for _ in range(2):
+        assert torch.equal(F.argmax(x, cols, tile_max=tm), F.argmax(x, cols))
+        for k, temp in ((4, 0.8), (1, 0.3), (8, 1.5)):
+            assert torch.equal(F.sample_topk(x, u, k, temp, cols, tile_max=tm), F.sample_topk(x, u, k, temp, cols)), (k, temp)
+    a, b = F.rng_state(dev, 77), F.rng_state(dev, 77)
+    for draw in range(3):
+        assert torch.equal(F.sample_topk(x, a, 4, 0.8, cols, tile_max=tm), F.sample_topk(x, b, 4, 0.8, cols)), draw
+    torch.cuda.synchronize()
+    assert a.cpu().tolist() == b.cpu().tolist() == [77, 3]
+
+
+@pytest.mark.parametrize("M,K,N,fp8,mask", [(64, 2048, 201088, False, True), (5, 1024, 200008, False, False), (17, 512, 400000, True, True)])
+def test_lm_head_leaves_tile_maxima(M, K, N, fp8, mask):
+    """lyra_decode_gemm_tile_max: the logits are bit for bit lyra_decode_gemm_ex's, the tile maxima are theirs, and
+    sample_token with them (model.py hangs them on the logits tensor) picks what it picks without."""
+    from dataclasses import replace
+
+    from lyra_amd.generate import sample_token
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.model import MODEL_VARIANTS
+    from lyra_amd.nn.quant import quantize
+
+    _say(f"lm head tile max M{M} K{K} N{N} fp8={fp8}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(M + N)
+    h = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(1, K, N, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    if fp8:
+        w = quantize(w, torch.float8_e4m3fn, (K, 1))
+    vocab = N - 40
+    bias = None
+    if mask:
+        bias = torch.zeros(N, device=dev)
+        bias[vocab:] = float("-inf")
+    one = torch.full((1,), M, dtype=torch.int32, device=dev)
+    got = F.gemm_tile_max(h, w, one, bias=bias)
+    assert got is not None
+    logits, tm = got
+    want = F.gemm(h, w, one, out_f32=True, bias=bias)
+    assert torch.equal(logits, want)
+    assert torch.equal(tm, _tile_maxima(want))
+    cfg = replace(MODEL_VARIANTS["dev"], vocab_size=vocab, sample_topk=4, sample_temperature=0.8, implementation="pallas")
+    plain = logits.clone()
+    logits.tile_max = (tm, logits._version)
+    for c in (cfg, replace(cfg, sample_temperature=0.0)):
+        a, b = F.rng_state(dev, 5), F.rng_state(dev, 5)
+        gen_a, gen_b = torch.Generator(device=dev), torch.Generator(device=dev)
+        gen_a.manual_seed(3), gen_b.manual_seed(3)
+        assert torch.equal(sample_token(logits, c, gen_a), sample_token(plain, c, gen_b))
+    logits[0, 3] = 1e9  # written to since: the maxima are stale and must not be used
+    assert int(sample_token(logits, replace(cfg, sample_temperature=0.0))[0]) == 3
+    # a small projection goes to other kernels: no tile maxima
+    ws = (torch.randn(1, 256, 1024, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    assert F.gemm_tile_max(h[:, :256].contiguous(), ws, one) is None
+
+
 @pytest.mark.parametrize("B,N,K,S,H,fp8,qknorm,sw,unsummed,positions", [
     (64, 16, 4, 4096, 128, True, True, 0, True, "full"),        # headline shape: one workgroup per (row, kv head)
     (64, 16, 4, 4096, 128, True, True, 128, True, "full"),      # sliding layer
