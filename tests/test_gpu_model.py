@@ -248,6 +248,8 @@ def _full_width_parity(cfg, B, S, start, steps, *, min_clear, moe_layers, hidden
         clear &= np.min(np.stack(margins), axis=0) > margin
         print("router margins (min over layers):", np.min(np.stack(margins), axis=0), file=sys.stderr, flush=True)
         assert clear.sum() >= min_clear, f"too few rows with unambiguous routing: {clear}"
+        print(f"step {s}: {int(clear.sum())} of {B} rows compared ({B - int(clear.sum())} left out for a routing margin <= {margin}; "
+              f"at least {min_clear} required)", file=sys.stderr, flush=True)
         if s == 0:
             worst = _layer_by_layer(cfg, w, cache, start, want_hidden, margins, margin)
             print(f"layer by layer: worst relative error of a layer output {worst:.5f} (bound {layer_tol})", file=sys.stderr, flush=True)
