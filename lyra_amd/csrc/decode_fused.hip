@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
 }
 
 // ---- MoE routing: top-k, softmax, shared experts, stable counting sort ------------------------------------
-// lyra/model.py:459-491.  One workgroup; thread t < tokens routes token t, then every assignment finds its
+// lyra/model.py:459-491.  One workgroup; a token is routed by a few neighbouring lanes, then every assignment finds its
 // destination row: start of its expert's rows + number of earlier assignments to the same expert.
 struct RouteParams {
     const float* logits;  // [tokens, n_routed] (bias already added)
@@ -338,14 +338,29 @@ struct RouteParams {
     int lanes;  // lanes that share the routing of one token: a power of two <= 16
 };
 
+// LDS ints the routing needs (host and device agree on this layout): assignments [M], counts [E], starts [E], one pad
+// int, one bit per (expert, token) in 64-bit words [E][ceil(tokens / 64)], staged logits [tokens * n_routed] when
+// stage_logits.
+static inline size_t route_lds_ints(int tokens, int n_routed, int n_shared, int k_routed, int stage_logits) {
+    const size_t topk = (size_t)k_routed + n_shared, E = (size_t)n_routed + n_shared, W = ((size_t)tokens + 63) / 64;
+    return (size_t)tokens * topk + 2 * E + 2 + 2 * E * W + (stage_logits ? (size_t)tokens * n_routed : 0);
+}
+
+// The whole routing by one workgroup of any size (a multiple of 64 threads).  `sm_i`: LDS of route_lds_ints() ints, 8-byte
+// aligned.
+//
+// The stable counting sort needs, for every assignment (token t, expert e), the number of earlier assignments to e.  A
+// token picks an expert at most once and assignments are in token order, so that is the number of tokens before t that
+// picked e: every pick sets bit t of its expert's mask, and a rank is a population count of the bits below t.
 __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
-    extern __shared__ int sm_i[];
-    const int topk = p.k_routed + p.n_shared, E = p.n_routed + p.n_shared, M = p.tokens * topk;
+    extern __shared__ __align__(16) int sm_i[];
+    const int topk = p.k_routed + p.n_shared, E = p.n_routed + p.n_shared, M = p.tokens * topk, W = (p.tokens + 63) >> 6;
     int* sm_expert = sm_i;        // [M]
     int* sm_count = sm_i + M;     // [E]
     int* sm_start = sm_count + E; // [E]
-    float* sm_logits = (float*)(sm_start + E);  // [tokens * n_routed] when p.stage_logits (coalesced copy, then row reads)
-    for (int e = threadIdx.x; e < E; e += blockDim.x) sm_count[e] = 0;
+    unsigned long long* sm_mask = (unsigned long long*)(sm_i + ((M + 2 * E + 1) & ~1));  // [E][W]
+    float* sm_logits = (float*)(sm_mask + (size_t)E * W);  // [tokens * n_routed] when p.stage_logits (coalesced copy, then row reads)
+    for (int e = threadIdx.x; e < E * W; e += blockDim.x) sm_mask[e] = 0ull;
     if (p.stage_logits)
         for (int i = threadIdx.x; i < p.tokens * p.n_routed; i += blockDim.x) sm_logits[i] = p.logits[i];
     __syncthreads();
@@ -394,65 +409,48 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteParams p) {
                 den += top[j];
             }
         }
+        const unsigned long long bit = 1ull << (t & 63);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             if (j < p.k_routed) {
                 p.scores[(size_t)t * topk + j] = top[j] / den;
                 sm_expert[t * topk + j] = idx[j];
-                atomicAdd(&sm_count[idx[j]], 1);
+                atomicOr(&sm_mask[(size_t)idx[j] * W + (t >> 6)], bit);
             }
         }
         for (int s = 0; s < p.n_shared; ++s) {
             p.scores[(size_t)t * topk + p.k_routed + s] = 1.f;  // model.py:476
             sm_expert[t * topk + p.k_routed + s] = p.n_routed + s;
-            atomicAdd(&sm_count[p.n_routed + s], 1);
+            atomicOr(&sm_mask[(size_t)(p.n_routed + s) * W + (t >> 6)], bit);
         }
     }
     __syncthreads();
-    // first row of every expert: thread e adds the counts of the experts before it (independent loads)
-    for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        int run = 0;
-        for (int j = 0; j < e; ++j) run += sm_count[j];
-        sm_start[e] = run;
-        p.groups[e] = sm_count[e];
-    }
-    if (M <= (int)blockDim.x) {
-        // One assignment per thread.  Its rank among the assignments to the same expert = lanes below it in its wavefront
-        // with that expert (one ballot per distinct expert of the wavefront) + that expert's count in the wavefronts before.
-        const int i = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
-        int* sm_wave_count = (int*)(sm_logits + (p.stage_logits ? p.tokens * p.n_routed : 0));  // [n_waves][E]
-        for (int j = threadIdx.x; j < n_waves * E; j += blockDim.x) sm_wave_count[j] = 0;
-        __syncthreads();
-        const int e = i < M ? sm_expert[i] : -1;
-        int rank = 0;
-        unsigned long long todo = __ballot(i < M);
-        while (todo) {  // same trip count for the whole wavefront
-            const int ev = __shfl(e, __ffsll((long long)todo) - 1, 64);
-            const unsigned long long same = __ballot(e == ev);
-            if (e == ev) {
-                const unsigned long long below = same & ((1ull << lane) - 1ull);
-                rank = __popcll(below);
-                if (below == 0ull) sm_wave_count[wave * E + ev] = __popcll(same);
+    // group sizes and the first row of every expert: the first wavefront counts the bits of 64 experts at a time and
+    // scans the counts
+    if (threadIdx.x < 64) {
+        int carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + (int)threadIdx.x;
+            int cnt = 0;
+            if (e < E)
+                for (int w = 0; w < W; ++w) cnt += __popcll(sm_mask[(size_t)e * W + w]);
+            const int incl = wave_scan_inclusive(cnt);
+            if (e < E) {
+                sm_count[e] = cnt;
+                sm_start[e] = carry + incl - cnt;
+                p.groups[e] = cnt;
             }
-            todo &= ~same;
+            carry += __builtin_amdgcn_readlane(incl, 63);
         }
-        __syncthreads();
-        if (i < M) {
-            for (int w = 0; w < wave; ++w) rank += sm_wave_count[w * E + e];
-            const int d = sm_start[e] + rank;
-            p.dest[i] = d;
-            p.row_map[d] = i / topk;
-        }
-        return;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < M; i += blockDim.x) {
-        const int e = sm_expert[i];
-        int rank = 0;
-        for (int j = 0; j < i; ++j) rank += sm_expert[j] == e;
+        const int e = sm_expert[i], t = i / topk;
+        int rank = __popcll(sm_mask[(size_t)e * W + (t >> 6)] & ((1ull << (t & 63)) - 1ull));
+        for (int w = 0; w < (t >> 6); ++w) rank += __popcll(sm_mask[(size_t)e * W + w]);
         const int d = sm_start[e] + rank;
         p.dest[i] = d;
-        p.row_map[d] = i / topk;
+        p.row_map[d] = t;
     }
 }
 
@@ -1112,12 +1110,11 @@ extern "C" int lyra_moe_route(const float* logits, float* scores, int32_t* group
     int lanes = 1;
     while (lanes < 16 && 2 * lanes <= n_routed && (long)tokens * 2 * lanes <= 1024) lanes *= 2;
     const int threads = std::min(1024, std::max(64, (std::max(tokens * topk, tokens * lanes) + 63) / 64 * 64));
-    // assignments, counts and starts, per-wavefront expert counts of the ranking step
-    size_t lds = ((size_t)tokens * topk + 2 * E + (size_t)(threads / 64) * E) * sizeof(int);
+    // assignments, counts and starts, the (expert, token) bit masks of the ranking step (+ the logits when they fit)
+    size_t lds = route_lds_ints(tokens, n_routed, n_shared, k_routed, 0) * sizeof(int);
     if (lds > 60000) return LYRA_E_UNSUPPORTED;
-    const size_t staged = (size_t)tokens * n_routed * sizeof(float);
-    const int stage = lds + staged <= 64000;
-    if (stage) lds += staged;
+    const int stage = route_lds_ints(tokens, n_routed, n_shared, k_routed, 1) * sizeof(int) <= 64000;
+    if (stage) lds = route_lds_ints(tokens, n_routed, n_shared, k_routed, 1) * sizeof(int);
     RouteParams p{logits, scores, groups, row_map, dest, tokens, n_routed, n_shared, k_routed, stage, lanes};
     hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
