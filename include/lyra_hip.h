@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 13
+#define LYRA_ABI_VERSION 14
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
@@ -121,6 +121,19 @@ int lyra_decode_attention_qkv(const void* qkv, const float* partials, int splits
                               int position_stride, const void* gate, void* out, void* workspace, size_t workspace_bytes,
                               int B, int N, int K, int S, int H, float sm_scale, int sliding_window, int kv_dtype,
                               int out_dtype, lyra_stream_t stream);
+/*
+ * The same for a q/k/v projection that has a bias (lyra/model.py:310-313: added to the projection's bf16 result, in
+ * bf16) and is handed over as unsummed slices: qkv_bias [(N + 2K) * H] float32 holding bf16 values; every head row is
+ * bf16(bf16(sum of slices) + bias) before the QK norm, as lyra_decode_gemm_ex with bit 1 of post_scale leaves it.  Saves
+ * the launch that would sum the slices only to add the bias.  qkv_bias needs partials (a summed projection carries its
+ * bias already); null = lyra_decode_attention_qkv.
+ */
+int lyra_decode_attention_qkv_bias(const void* qkv, const float* partials, int splits, const float* qkv_bias, const float* qnorm,
+                                   const float* knorm, const float* cos_t, const float* sin_t, int rope_rows, float eps, void* k,
+                                   void* v, float* k_scale, float* v_scale, const float* sinks, const int32_t* position,
+                                   int position_stride, const void* gate, void* out, void* workspace, size_t workspace_bytes,
+                                   int B, int N, int K, int S, int H, float sm_scale, int sliding_window, int kv_dtype,
+                                   int out_dtype, lyra_stream_t stream);
 
 /*
  * Ragged batches, rows dealt out by length (an extension of the boundary, like position_stride 1: the reference passes one
@@ -255,6 +268,8 @@ int lyra_gemm_pack(const void* rhs, void* packed, int G, int K, int N, int rhs_d
  *   lyra_decode_gemm_partials  partials[s] = lhs[:, slice s] @ rhs[slice s, :] (weight scales applied), no epilogue;
  *                              partials holds splits * M * N floats, 16-byte aligned.
  * The sum over slices is taken in slice order in float32, then rounded as the projection's bf16 output would be.
+ * K % 32 == 0, N % 8 == 0 (a last 128-column span that N does not fill is fine).  A projection with a bias of its own
+ * hands the bias to the consumer too: lyra_decode_attention_qkv_bias, lyra_rmsnorm_proj_sum_bias.
  */
 int lyra_decode_gemm_splits(int M, int K, int N, int bk);
 int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const float* rhs_scale, int bk, int bn,
@@ -281,6 +296,13 @@ int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, const float* p
 int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale, void* x_out,
                           const float* scale, void* h, const float* proj_t, const float* bias, void* y, int B, int C, int n,
                           int mode, float eps, lyra_stream_t stream);
+/* Same for a projection with a bias of its own (output and dense-down projections of the gpt-oss variants,
+ * lyra/model.py:367-368, 629-630): sum_bias [C] float32 holding bf16 values, and
+ * x_out = bf16(residual + bf16(bf16(bf16(sum of slices) + sum_bias) * out_scale)), what lyra_decode_gemm_ex with bit 1 of
+ * post_scale and the residual epilogue gives; null = lyra_rmsnorm_proj_sum. */
+int lyra_rmsnorm_proj_sum_bias(const void* x, const float* partials, int splits, const float* sum_bias, const void* residual,
+                               float out_scale, void* x_out, const float* scale, void* h, const float* proj_t, const float* bias,
+                               void* y, int B, int C, int n, int mode, float eps, lyra_stream_t stream);
 /* Same, but the row to normalise is the residual update that ends a MoE layer (lyra/model.py:557-567; what lyra_moe_combine
  * computes): x_out = bf16(residual + bf16(bf16(sum_k scores[b,k] * rows[dest[b*topk+k]]) * out_scale)), rows [B*topk, C]
  * bf16 in sorted order, scores [B, topk] float32, dest [B*topk] int32, topk <= 16.  Same aliasing rule. */

@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
 RHS_SPAN_MAJOR, RHS_SPAN_MAJOR_GLU = 0x100, 0x200  # LYRA_RHS_SPAN_MAJOR(_GLU): OR-ed into a matmul's rhs_dtype
 LHS_TILED16, OUT_TILED16 = 0x400, 0x800  # LYRA_LHS_TILED16 / LYRA_OUT_TILED16, likewise
-ABI_VERSION = 13
+ABI_VERSION = 14
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
 
 _c = ctypes
@@ -34,6 +34,11 @@ SIGNATURES = {
     "lyra_decode_attention_qkv": (
         _c.c_int,
         [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 4 + [_c.c_int, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] + [_c.c_void_p] * 3
+        + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
+    ),
+    "lyra_decode_attention_qkv_bias": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int] + [_c.c_void_p] * 5 + [_c.c_int, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] + [_c.c_void_p] * 3
         + [_c.c_size_t] + [_c.c_int] * 5 + [_c.c_float] + [_c.c_int] * 3 + [_c.c_void_p],
     ),
     "lyra_decode_attention_static": (
@@ -69,6 +74,10 @@ SIGNATURES = {
     "lyra_rmsnorm_proj_sum": (
         _c.c_int,
         [_c.c_void_p] * 2 + [_c.c_int, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
+    ),
+    "lyra_rmsnorm_proj_sum_bias": (
+        _c.c_int,
+        [_c.c_void_p] * 2 + [_c.c_int, _c.c_void_p, _c.c_void_p, _c.c_float] + [_c.c_void_p] * 6 + [_c.c_int] * 4 + [_c.c_float, _c.c_void_p],
     ),
     "lyra_rmsnorm_proj_embed": (
         _c.c_int,

@@ -56,6 +56,7 @@ struct AttnParams {
     const float* qkv_partials;  // [splits, B, (N + 2K) * H] float32 slices of the q/k/v projection, or null (then qkv)
     const uint16_t* qkv;        // [B, (N + 2K) * H] bf16
     int qkv_splits;
+    const float* qkv_bias;      // with the slices: the projection's bias [(N + 2K) * H] (bf16 values as float32), or null
     const float* qnorm;  // [H] or null (both)
     const float* knorm;
     const float* cos_t;  // [rope_rows, H/2]
@@ -447,6 +448,16 @@ __device__ __forceinline__ void sum_head(const AttnParams& p, __amdgpu_buffer_rs
     }
     a = bf16r(a);
     c = bf16r(c);
+    if (p.qkv_bias) {
+        // lyra/model.py:310-313: the bias is added to the projection's bf16 result, in bf16.  Fetched here, in the one
+        // branch of the front step that holds loads: launches without a bias (every lyra variant) skip it, and two more
+        // requests per head at kernel start cost those 0.3 us per sliding-window launch.
+        const int heads = p.N + 2 * p.K;
+        const __amdgpu_buffer_rsrc_t bias_rsrc = make_rsrc(p.qkv_bias, (uint32_t)heads * (uint32_t)H * 4u);
+        const int offb = lane < half ? (hd * H + lane) * 4 : kNoLoad;
+        a = bf16r(a + __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(bias_rsrc, offb, 0, 0)));
+        c = bf16r(c + __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(bias_rsrc, offb, half * 4, 0)));
+    }
 }
 
 // The cache bytes of one finished row (this lane's elements a, c) of the key (slot 0) or value (slot 1) head, left in
@@ -1149,6 +1160,7 @@ struct QkvFront {
     const void* qkv;
     const float* partials;
     int splits;
+    const float* bias;  // of the projection whose slices `partials` are, or null
     const float *qnorm, *knorm, *cos_t, *sin_t;
     int rope_rows;
     float eps;
@@ -1217,6 +1229,7 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     p.qkv_partials = nullptr;
     p.qkv = nullptr;
     p.qkv_splits = 0;
+    p.qkv_bias = nullptr;
     p.qnorm = p.knorm = p.cos_t = p.sin_t = nullptr;
     p.rope_rows = 0;
     p.norm_eps = 0.f;
@@ -1224,6 +1237,7 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
         p.qkv_partials = front->partials;
         p.qkv = (const uint16_t*)front->qkv;
         p.qkv_splits = front->splits;
+        p.qkv_bias = front->partials ? front->bias : nullptr;
         p.qnorm = front->qnorm;
         p.knorm = front->knorm;
         p.cos_t = front->cos_t;
@@ -1362,7 +1376,20 @@ extern "C" int lyra_decode_attention_qkv(const void* qkv, const float* partials,
                                          void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
                                          float sm_scale, int sliding_window, int kv_dtype, int out_dtype,
                                          lyra_stream_t stream) {
-    const lyra::QkvFront front{qkv, partials, splits, qnorm, knorm, cos_t, sin_t, rope_rows, eps};
+    return lyra_decode_attention_qkv_bias(qkv, partials, splits, nullptr, qnorm, knorm, cos_t, sin_t, rope_rows, eps, k, v, k_scale,
+                                          v_scale, sinks, position, position_stride, gate, out, workspace, workspace_bytes, B, N, K, S,
+                                          H, sm_scale, sliding_window, kv_dtype, out_dtype, stream);
+}
+
+extern "C" int lyra_decode_attention_qkv_bias(const void* qkv, const float* partials, int splits, const float* qkv_bias,
+                                              const float* qnorm, const float* knorm, const float* cos_t, const float* sin_t,
+                                              int rope_rows, float eps, void* k, void* v, float* k_scale, float* v_scale,
+                                              const float* sinks, const int32_t* position, int position_stride, const void* gate,
+                                              void* out, void* workspace, size_t workspace_bytes, int B, int N, int K, int S, int H,
+                                              float sm_scale, int sliding_window, int kv_dtype, int out_dtype,
+                                              lyra_stream_t stream) {
+    if (qkv_bias && !partials) return LYRA_E_BADARG;  // (a summed projection already carries its bias)
+    const lyra::QkvFront front{qkv, partials, splits, qkv_bias, qnorm, knorm, cos_t, sin_t, rope_rows, eps};
     return lyra::run_attention(nullptr, k, v, k_scale, v_scale, sinks, position, position_stride, gate, out, workspace,
                                workspace_bytes, LYRA_E_WORKSPACE, false, nullptr, nullptr, B, N, K, S, H, sm_scale,
                                sliding_window, kv_dtype, out_dtype, stream, &front);

@@ -52,6 +52,9 @@ struct NormProjParams {
     const int32_t* row_index;   // [B] or null
     int row_limit;              // rows of x when row_index is set: an index outside [0, row_limit) is clamped into it, so a
                                 // bad token id (padding such as -1, a stale buffer) reads a valid row instead of faulting
+    // with `partials`: the projection's bias [C] (bf16 values as float32), added to the bf16-rounded sum in bf16 before the
+    // scale / residual step (lyra/model.py:367-368, 629-630), or null
+    const float* sum_bias;
 };
 
 constexpr int kNormThreads = 1024;
@@ -138,6 +141,11 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
                 }
             }
             const u32x2 r = *(const u32x2*)(p.residual + (size_t)b * p.C + c);
+            if (p.sum_bias) {  // (the projection's own bias: bf16(bf16(sum) + bias), as the matmul's epilogue forms it)
+                const f32x4 bb = *(const f32x4*)(p.sum_bias + c);
+                t[0] = bf16r(bf16r(t[0]) + bb[0]); t[1] = bf16r(bf16r(t[1]) + bb[1]);
+                t[2] = bf16r(bf16r(t[2]) + bb[2]); t[3] = bf16r(bf16r(t[3]) + bb[3]);
+            }
             const float r0 = __uint_as_float(r[0] << 16), r1 = __uint_as_float(r[0] & 0xFFFF0000u);
             const float r2 = __uint_as_float(r[1] << 16), r3 = __uint_as_float(r[1] & 0xFFFF0000u);
             d[0] = pack_bf16(r0 + bf16r(bf16r(t[0]) * p.out_scale), r1 + bf16r(bf16r(t[1]) * p.out_scale));
@@ -1030,7 +1038,15 @@ extern "C" int lyra_rmsnorm_proj(const void* x, const float* scale, void* h, con
 extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int splits, const void* residual, float out_scale,
                                      void* x_out, const float* scale, void* h, const float* proj_t, const float* bias, void* y,
                                      int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
+    return lyra_rmsnorm_proj_sum_bias(x, partials, splits, nullptr, residual, out_scale, x_out, scale, h, proj_t, bias, y, B, C, n, mode,
+                                      eps, stream);
+}
+
+extern "C" int lyra_rmsnorm_proj_sum_bias(const void* x, const float* partials, int splits, const float* sum_bias, const void* residual,
+                                          float out_scale, void* x_out, const float* scale, void* h, const float* proj_t,
+                                          const float* bias, void* y, int B, int C, int n, int mode, float eps, lyra_stream_t stream) {
     using namespace lyra;
+    if (sum_bias && (!partials || ((uintptr_t)sum_bias % 16))) return LYRA_E_BADARG;
     if (partials ? (!residual || !x_out || splits <= 0) : !x) return LYRA_E_BADARG;
     if (partials && (double)splits * B * C * 4 >= 2147483648.0) return LYRA_E_UNSUPPORTED;
     if (!scale || !h || B <= 0 || C <= 0) return LYRA_E_BADARG;
@@ -1038,7 +1054,8 @@ extern "C" int lyra_rmsnorm_proj_sum(const void* x, const float* partials, int s
     if ((mode & ~7) || ((mode & 4) && C % 32)) return LYRA_E_UNSUPPORTED;
     if (C % 4 || C > 32768) return LYRA_E_UNSUPPORTED;
     NormProjParams p{(const uint16_t*)x, scale, (uint16_t*)h, proj_t, bias, y, C, proj_t ? n : 0, mode, eps,
-                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr, 0};
+                     partials, splits, B, (const uint16_t*)residual, out_scale, (uint16_t*)x_out, nullptr, nullptr, nullptr, 0, nullptr, 0,
+                     sum_bias};
     return launch_rmsnorm_proj(p, B, stream);
 }
 

@@ -2088,7 +2088,7 @@ static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const vo
 }  // namespace lyra
 
 extern "C" int lyra_decode_gemm_splits(int M, int K, int N, int bk) {
-    if (M <= 0 || K <= 0 || N <= 0 || K % 32 || N % 128) return 0;
+    if (M <= 0 || K <= 0 || N <= 0 || K % 32 || N % 8) return 0;  // (a last span that N does not fill is fine)
     const lyra::GemmPlan pl = lyra::plan_gemm(M, 1, K, N, bk, 0);
     return pl.split_k ? pl.ksplit : 0;
 }
@@ -2107,7 +2107,7 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
     const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
-    if (K % 32 || N % 128) return LYRA_E_UNSUPPORTED;
+    if (K % 32 || N % 8) return LYRA_E_UNSUPPORTED;
     GemmParams p = {};
     p.bk = p.bn = p.KB = p.NB = 1;
     if (fp8) {

@@ -43,12 +43,16 @@ def _transposed(w: torch.Tensor) -> torch.Tensor:
 
 class Unsummed:
     """A projection whose K slices are still separate: ``partials`` [splits, M, N] float32, plus the residual update that
-    follows it (``residual`` [M, N] bf16 and ``scale``), to be applied by the kernel that consumes it."""
+    follows it (``residual`` [M, N] bf16 and ``scale``), to be applied by the kernel that consumes it.  ``bias``: the
+    projection's own bias [N] (float32 holding bf16 values), which the consumer adds to the bf16-rounded sum in bf16
+    (lyra/model.py:310-313, 367-368, 629-630); the attention launch with the front step and the norm kernel take it,
+    ``qkv_post`` does not."""
 
-    __slots__ = ("partials", "residual", "scale")
+    __slots__ = ("partials", "residual", "scale", "bias")
 
-    def __init__(self, partials: torch.Tensor, residual: torch.Tensor | None = None, scale: float = 1.0):
-        self.partials, self.residual, self.scale = partials, residual, scale
+    def __init__(self, partials: torch.Tensor, residual: torch.Tensor | None = None, scale: float = 1.0,
+                 bias: torch.Tensor | None = None):
+        self.partials, self.residual, self.scale, self.bias = partials, residual, scale, bias
 
 
 class Uncombined:
@@ -172,7 +176,7 @@ def gemm_unsummed(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor) -> Unsummed
     M, K = (lhs.rows, lhs.cols) if tiled else lhs.shape
     lhs_t = lhs.data if tiled else lhs
     rv, rs, bk, bn, rd, (G, _, N) = _rhs_args(rhs)
-    if G != 1 or K % 32 or N % 128 or (isinstance(rhs, SpanMajor) and rhs.layout != 1):
+    if G != 1 or K % 32 or N % 8 or (isinstance(rhs, SpanMajor) and rhs.layout != 1):
         return None
     splits = _L.lyra_decode_gemm_splits(M, K, N, bk)
     if splits <= 0:
@@ -224,10 +228,12 @@ def rmsnorm_proj(x, scale: torch.Tensor, eps: float, proj: torch.Tensor | None =
             n = proj.shape[1]
             y = torch.empty((B, n), dtype=torch.bfloat16 if gate else torch.float32, device=h.device)
             proj = _f32(_transposed(proj))
-        rc = _L.lyra_rmsnorm_proj_sum(None, u.partials.data_ptr(), splits, u.residual.data_ptr(), float(u.scale), x_out.data_ptr(),
-                                      _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y), B, C, n,
-                                      mode, float(eps), _stream(h.device))
-        _lib.check(rc, "lyra_rmsnorm_proj_sum")
+        if u.bias is not None:
+            assert u.bias.dtype == torch.float32 and u.bias.is_contiguous() and u.bias.numel() == C
+        rc = _L.lyra_rmsnorm_proj_sum_bias(None, u.partials.data_ptr(), splits, _ptr(u.bias), u.residual.data_ptr(), float(u.scale),
+                                           x_out.data_ptr(), _f32(scale).data_ptr(), h.data_ptr(), _ptr(proj), _ptr(bias), _ptr(y),
+                                           B, C, n, mode, float(eps), _stream(h.device))
+        _lib.check(rc, "lyra_rmsnorm_proj_sum_bias")
         return h_obj, y, x_out
     B, C = x.shape
     assert x.dtype == torch.bfloat16 and x.is_contiguous()
@@ -283,6 +289,7 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
     N, K, H = n_heads, n_kv_heads, head_dim
     unsummed = isinstance(qkv, Unsummed)
     if unsummed:  # the projection arrives as K slices; they are summed while reading
+        assert qkv.bias is None, "a projection with a bias comes summed (gemm with bias_after_cast) to qkv_post"
         part = qkv.partials
         splits, B, width = part.shape
         assert width == (N + 2 * K) * H and qkv.residual is None
@@ -351,8 +358,11 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
     stream = _stream(dev)
     need = _L.lyra_decode_attention_workspace(B, N, K, S, H, int(sliding_window))
     ws = _lib.workspace("attention", dev, stream, need)
-    rc = _L.lyra_decode_attention_qkv(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None,
-                                      splits if unsummed else 0, _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(),
+    qkv_bias = qkv.bias if unsummed else None
+    if qkv_bias is not None:
+        assert qkv_bias.dtype == torch.float32 and qkv_bias.is_contiguous() and qkv_bias.numel() == (N + 2 * K) * H
+    rc = _L.lyra_decode_attention_qkv_bias(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None,
+                                      splits if unsummed else 0, _ptr(qkv_bias), _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(),
                                       _f32(sin_t).data_ptr(), cos_t.shape[0], float(eps), kq.data_ptr(), vq.data_ptr(), _ptr(ks),
                                       _ptr(vs), sinks.data_ptr(), pos.data_ptr(), 0 if pos.numel() == 1 else 1, _ptr(gate),
                                       out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, float(sm_scale),

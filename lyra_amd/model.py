@@ -498,16 +498,23 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
     B = x.shape[0]
     one = _one_group(B, x.device)
     w_qkv, w_out = F.span_major(w.qkv), F.span_major(w.out)  # (the arrays themselves unless their rows straddle cache lines)
-    qkv = F.gemm_unsummed(h, w_qkv, one) if w.qkv_bias is None else None
+    # (:310-313: a bias is added to the projection's bf16 result, in bf16: by the attention launch that sums the slices when
+    # that launch is certain to take them - one position for the batch, no learned exclusive self attention - else inside
+    # the matmul's epilogue, which costs the launch that sums the slices)
+    front_step = w.xsa_alpha is None and not _SEPARATE_QKV_POST
+    qkv = F.gemm_unsummed(h, w_qkv, one) if (w.qkv_bias is None or (front_step and pos.numel() == 1)) else None
+    if qkv is not None and w.qkv_bias is not None:
+        qkv.bias = _bf16_bias(w.qkv_bias).reshape(-1)
     if qkv is None:
-        # (:310-313: a bias is added to the projection's bf16 result, in bf16 - inside the matmul's epilogue)
         qkv = F.gemm(h, w_qkv, one, bias=_bf16_bias(w.qkv_bias), bias_after_cast=w.qkv_bias is not None)
     sliding_window = cfg.sliding_window if idx % 2 == 0 else 0
     t = None
-    if w.xsa_alpha is None and not _SEPARATE_QKV_POST:  # QK norm + RoPE + cache append inside the attention launch
+    if front_step:  # QK norm + RoPE + cache append inside the attention launch
         t = F.attention_qkv(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, w.sinks, H**-0.5,
                             sliding_window, N, K, H, cfg.norm_eps, gate=gate)
     if t is None:  # (learned exclusive self attention, or a ragged batch the whole-row attention kernel takes)
+        if isinstance(qkv, F.Unsummed) and qkv.bias is not None:  # (refused after all: the summed form carries the bias)
+            qkv = F.gemm(h, w_qkv, one, bias=_bf16_bias(w.qkv_bias), bias_after_cast=True)
         q = F.qkv_post(qkv, w.qnorm_scale, w.knorm_scale, cos_t, sin_t, pos, cache.k, cache.v, N, K, H, cfg.norm_eps,
                        unit_v=w.xsa_alpha is not None)
         xsa_v = None
@@ -516,12 +523,13 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         attn = attn_op(cfg.mode, cfg.implementation)
         t = attn(q[:, :, None, :], cache.k, cache.v, w.sinks, H**-0.5, sliding_window, pos, gate=gate, xsa_v=xsa_v,
                  xsa_alpha=w.xsa_alpha).reshape(B, N * H)
-    if w.out_bias is not None:  # :366-373: projection, + bias, * residual scale, + residual, each a bf16 result
-        return F.gemm(t, w_out, one, bias=_bf16_bias(w.out_bias), bias_after_cast=True, residual=x, out_scale=cfg.residual_scale), cache
+    # :366-373: projection, + bias, * residual scale, + residual, each a bf16 result - left to the norm that sums the slices
     out = F.gemm_unsummed(t, w_out, one)
     if out is None:
-        return F.gemm(t, w_out, one, residual=x, out_scale=cfg.residual_scale), cache
+        return F.gemm(t, w_out, one, bias=_bf16_bias(w.out_bias), bias_after_cast=w.out_bias is not None, residual=x,
+                      out_scale=cfg.residual_scale), cache
     out.residual, out.scale = x, cfg.residual_scale
+    out.bias = None if w.out_bias is None else _bf16_bias(w.out_bias).reshape(-1)
     return out, cache
 
 
@@ -563,13 +571,13 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     w_up, w_down = F.span_major(w.mlp_up), F.span_major(w.mlp_down)
     t = F.gemm(t, w_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
                bias=_bf16_bias(w.mlp_up_bias), out_tiled=tiled)
-    if w.mlp_down_bias is not None:  # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result
-        return F.gemm(t, w_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=True, residual=x,
-                      out_scale=cfg.dense_residual_scale)
+    # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result - left to the norm that sums the slices
     down = F.gemm_unsummed(t, w_down, one)
     if down is None:
-        return F.gemm(t, w_down, one, residual=x, out_scale=cfg.dense_residual_scale)
+        return F.gemm(t, w_down, one, bias=_bf16_bias(w.mlp_down_bias), bias_after_cast=w.mlp_down_bias is not None, residual=x,
+                      out_scale=cfg.dense_residual_scale)
     down.residual, down.scale = x, cfg.dense_residual_scale
+    down.bias = None if w.mlp_down_bias is None else _bf16_bias(w.mlp_down_bias).reshape(-1)
     return down
 
 

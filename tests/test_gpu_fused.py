@@ -381,6 +381,68 @@ def test_unsummed_projection_consumers_equal_summed_path(fp8, B, C, N, K, H):
     assert torch.equal(x1, x2) and torch.equal(h1, h2) and torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("B,C,N,K,H,sw", [(64, 2880, 64, 8, 64, 0), (64, 2880, 64, 8, 64, 128), (5, 256, 2, 1, 64, 0), (8, 2048, 16, 4, 128, 0)])
+def test_biased_projections_left_unsummed_equal_the_summed_path(fp8, B, C, N, K, H, sw):
+    """Projections with a bias of their own (gpt-oss variants, lyra/model.py:310-313, 367-368): handing the K slices and
+    the bias to the consumer - the attention launch with the front step, the norm kernel - must give bit for bit what the
+    matmul's epilogue (bias added to the bf16 result, in bf16) followed by the consumer on the summed form gives."""
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray, quantize
+
+    _say(f"biased unsummed fp8={fp8} B{B} C{C} N{N} K{K} H{H} sw{sw}")
+    dev = U.dev()
+    g = torch.Generator(device=dev)
+    g.manual_seed(B + C + sw)
+    rnd = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).to(torch.bfloat16)
+    width = (N + 2 * K) * H
+    w_qkv, w_out = rnd(1, C, width, std=0.03), rnd(1, N * H, C, std=0.03)
+    if fp8:
+        w_qkv, w_out = quantize(w_qkv, torch.float8_e4m3fn, (C, 1)), quantize(w_out, torch.float8_e4m3fn, (N * H, 1))
+    b_qkv = rnd(width, std=0.5).to(torch.float32)  # (bf16 values as float32, what the epilogue takes)
+    b_out = rnd(C, std=0.5).to(torch.float32)
+    one = torch.full((1,), B, dtype=torch.int32, device=dev)
+    h, x = rnd(B, C), rnd(B, C)
+    S = 256
+    cos_t, sin_t = (U.t_f32(t) for t in O.rope_tables(S, H))
+    pos = torch.tensor(77, dtype=torch.int32, device=dev)
+    sinks = torch.randn(N, generator=g, device=dev)
+
+    def caches():
+        kv = []
+        for _ in range(2):
+            c = rnd(B, K, S, H)
+            kv.append(quantize(c, torch.float8_e4m3fn, (1, H)) if fp8 else c)
+        return kv
+
+    g.manual_seed(99)
+    ck1, cv1 = caches()
+    g.manual_seed(99)
+    ck2, cv2 = caches()
+    # q/k/v projection -> front step of the attention launch
+    un = F.gemm_unsummed(h, w_qkv, one)
+    assert un is not None
+    un.bias = b_qkv
+    a1 = F.attention_qkv(un, None, None, cos_t, sin_t, pos, ck1, cv1, sinks, H**-0.5, sw, N, K, H, 1e-5)
+    summed = F.gemm(h, w_qkv, one, bias=b_qkv.reshape(1, -1), bias_after_cast=True)
+    a2 = F.attention_qkv(summed, None, None, cos_t, sin_t, pos, ck2, cv2, sinks, H**-0.5, sw, N, K, H, 1e-5)
+    assert a1 is not None and a2 is not None and torch.equal(a1, a2)
+    raw = lambda c: c.qval.view(torch.uint8) if isinstance(c, QArray) else c.view(torch.int16)
+    assert torch.equal(raw(ck1), raw(ck2)) and torch.equal(raw(cv1), raw(cv2))
+    if fp8:
+        assert torch.equal(ck1.scale, ck2.scale) and torch.equal(cv1.scale, cv2.scale)
+    # output projection -> residual update -> next norm
+    t = rnd(B, N * H)
+    un = F.gemm_unsummed(t, w_out, one)
+    assert un is not None
+    un.residual, un.scale, un.bias = x, 0.1767766952966369, b_out
+    scale = torch.rand(C, generator=g, device=dev) + 0.5
+    h1, _, x1 = F.rmsnorm_proj(un, scale, 1e-5)
+    x2 = F.gemm(t, w_out, one, bias=b_out.reshape(1, -1), bias_after_cast=True, residual=x, out_scale=0.1767766952966369)
+    h2, _ = F.rmsnorm_proj(x2, scale, 1e-5)
+    assert torch.equal(x1, x2) and torch.equal(h1, h2)
+
+
 @pytest.mark.parametrize("T,topk,C,n,gate", [(64, 4, 2048, 16, True), (64, 4, 2048, 15, False), (3, 2, 256, 0, False), (17, 16, 4096, 7, False)])
 def test_uncombined_moe_layer_end_equals_combine_then_norm(T, topk, C, n, gate):
     """Leaving the combine step of a MoE layer to the norm that follows must give bit for bit what combining first gives,
