@@ -55,6 +55,7 @@ struct NormProjParams {
     // with `partials`: the projection's bias [C] (bf16 values as float32), added to the bf16-rounded sum in bf16 before the
     // scale / residual step (lyra/model.py:367-368, 629-630), or null
     const float* sum_bias;
+    int per_share;  // projection outputs per workgroup of a row: ceil(n / shares), set by the launch
 };
 
 constexpr int kNormThreads = 1024;
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
     // The weights of the first projection output of this wavefront do not depend on the row: they are requested before
     // anything else, so that they arrive while the row is being read and normalised (otherwise the projection is a
     // second memory round trip behind the norm: 1.4 us of a 4.7 us launch).
-    const int per_share = (p.n + shares - 1) / shares, j_end = min(p.n, (share + 1) * per_share);
+    const int per_share = p.per_share, j_end = min(p.n, (share + 1) * per_share);  // (ceil(n / shares), divided on the host)
     const int j_first = share * per_share + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // (the same in every lane)
     u32x4 w_first[8];
     if (p.proj_t && j_first < j_end) {  // (only the wavefronts that have an output: a load that fetches nothing still takes its
@@ -1020,10 +1021,12 @@ __global__ __launch_bounds__(256) void sample_tiles_kernel(TileSampleParams p) {
 }  // namespace lyra
 
 namespace lyra {
-static int launch_rmsnorm_proj(const NormProjParams& p, int B, lyra_stream_t stream) {
+static int launch_rmsnorm_proj(const NormProjParams& p0, int B, lyra_stream_t stream) {
+    NormProjParams p = p0;
     const size_t lds = ((size_t)p.C + 16) * sizeof(float);
     static const int shares_env = [] { const char* e = getenv("LYRA_NORM_SHARES"); return e ? atoi(e) : 4; }();  // tuning override
     const int shares = (p.proj_t && p.n >= 8 && B <= 256) ? std::max(1, std::min(shares_env, p.n)) : 1;
+    p.per_share = (p.n + shares - 1) / shares;
     if (p.comb_rows) hipLaunchKernelGGL(rmsnorm_proj_kernel<true>, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     else hipLaunchKernelGGL(rmsnorm_proj_kernel<false>, dim3(B, shares), dim3(kNormThreads), lds, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
