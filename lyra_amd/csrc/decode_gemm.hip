@@ -13,11 +13,21 @@
 // (x = lane & 15, kb = lane >> 4) reads 8 consecutive columns of the 8 rows 8*kb .. 8*kb+7; pairing two
 // rows in the bf16 pack step yields the K-major B operand, so the transposition costs nothing.
 //   D[16 rows, 16 cols] += X[16 rows x 32 k] . W[32 k x 16 cols]   for each of the 8 column phases.
+//
+// This file is compiled twice.  With LYRA_GEMM_SPLITK_PART it yields only the K-split kernel and its launcher,
+// built with the compiler's option that keeps matrix-core accumulators in ordinary vector registers: those
+// kernels do one or two matrix instructions per accumulator and the copies to and from the accumulator file were
+// a sixth of their instructions.  With LYRA_GEMM_MAIN_PART it yields everything else (the option makes the expert
+// kernel spill registers).  With neither macro it is one complete translation unit.
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
 #include "lyra_device.h"
+
+#if defined(LYRA_GEMM_SPLITK_PART) && defined(LYRA_GEMM_MAIN_PART)
+#error "LYRA_GEMM_SPLITK_PART and LYRA_GEMM_MAIN_PART select different halves of this file"
+#endif
 
 namespace lyra {
 
@@ -457,6 +467,7 @@ void decode_gemm_kernel(GemmParams p) {
     }
 }
 
+#ifndef LYRA_GEMM_SPLITK_PART
 // Second pass when K was split across workgroups: sum the partials, then bias / SwiGLU / cast.
 // One thread per 4 output columns.
 __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
@@ -526,7 +537,7 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
     }
     }
 }
-
+#endif  // !LYRA_GEMM_SPLITK_PART
 
 // ---- small weight sets: one group, a few MB of weights (the dense projections of a decode layer) -----------------
 // Such a product is bound by latency, not bandwidth: what counts is how many weight rows are in flight.  A workgroup
@@ -1601,6 +1612,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 // ---- span-major copy of a weight array (done once, when the weights are loaded) ---------------------------------------
 // One thread moves 8 consecutive elements of a packed row: they come from 8 consecutive columns of the reference's array
 // (widths are multiples of 8, or 16 with gate and linear halves) or are zeros where the span runs past the last column.
+#ifndef LYRA_GEMM_SPLITK_PART
 struct PackParams {
     const uint8_t* src;
     uint8_t* dst;
@@ -1634,6 +1646,7 @@ __global__ __launch_bounds__(256) void gemm_pack_kernel(PackParams p) {
         }
     }
 }
+#endif  // !LYRA_GEMM_SPLITK_PART
 
 static int packed_spans(int N, int layout) { return layout == 2 ? (N / 2 + 63) / 64 : (N + 127) / 128; }
 
@@ -1742,7 +1755,9 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
 }
 
 // Launches the K-split kernel of a plan with split_k set; p.part receives [ksplit, M, N] float32 slices.
-static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st) {
+int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st);
+#ifndef LYRA_GEMM_MAIN_PART
+int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st) {
     const dim3 grid(pl.spans, pl.ksplit, pl.row_par), block(kSplitWaves * 64);
     const size_t lds = (size_t)kSplitWaves * 64 * kSplitPitch * sizeof(float);
     const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4 steps per wavefront, or more: the looping variant
@@ -1791,8 +1806,11 @@ static int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hip
 #undef LYRA_SPLITK_M
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
+#endif  // !LYRA_GEMM_MAIN_PART
 
 }  // namespace lyra
+
+#ifndef LYRA_GEMM_SPLITK_PART
 
 namespace lyra {
 // Bytes of float32 partials (behind the counters) that the launch of `pl` writes.
@@ -2170,3 +2188,4 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     p.lhs_tiled = lhs_tiled;
     return launch_split_k(p, pl, fp8, (hipStream_t)stream);
 }
+#endif  // !LYRA_GEMM_SPLITK_PART
