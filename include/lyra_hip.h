@@ -18,12 +18,13 @@
 extern "C" {
 #endif
 
-#define LYRA_ABI_VERSION 14
+#define LYRA_ABI_VERSION 15
 
 /* element types of buffers that cross the ABI */
 #define LYRA_DTYPE_BF16 0   /* bfloat16, 2 bytes */
 #define LYRA_DTYPE_E4M3FN 1 /* OCP FP8 E4M3 (finite, max 448), 1 byte; needs scales */
 #define LYRA_DTYPE_F32 2    /* float32 (outputs only) */
+#define LYRA_DTYPE_E5M2 3   /* OCP FP8 E5M2 (max 57344), 1 byte; needs scales; accepted wherever e4m3fn is */
 /* OR-ed into rhs_dtype of lyra_decode_gemm_ex / lyra_decode_gemm_partials: rhs is not the reference's [G,K,N] array but
  * the span-major copy of it that lyra_gemm_pack writes (layout 1 or 2 below). */
 #define LYRA_RHS_SPAN_MAJOR 0x100     /* layout 1: spans of 128 consecutive columns */
@@ -57,7 +58,7 @@ const char* lyra_strerror(int code);
  * and sliding_decode :263-308).
  *
  *   q        [B,N,H] bf16                      (the reference's [B,N,1,H])
- *   k, v     [B,K,S,H] bf16 or e4m3fn, contiguous; kv head of query head n is n / (N/K)
+ *   k, v     [B,K,S,H] bf16, e4m3fn or e5m2 (both FP8_DTYPES of lyra/nn/quant.py:10), contiguous; kv head of query head n is n / (N/K)
  *   k_scale, v_scale   [B,K,S] float32, one per cached token and kv head (QArray block (1,H),
  *            lyra/model.py:225); NULL iff kv_dtype == LYRA_DTYPE_BF16
  *   sinks    [N] float32 learned sink logits (a virtual key with value 0)
@@ -186,7 +187,7 @@ int lyra_workspace_init(void* workspace, size_t workspace_bytes, lyra_stream_t s
  * lyra.nn.quant.dot for the dense projections (lyra/nn/quant.py:106-108).
  *
  *   lhs         [M,K] bf16
- *   rhs         [G,K,N] bf16 or e4m3fn, contiguous
+ *   rhs         [G,K,N] bf16, e4m3fn or e5m2, contiguous
  *   rhs_scale   [G,K/bk,N/bn] float32 block scales (QArray block (bk,bn)); NULL iff rhs is bf16.
  *               bk == K, bn == 1 is the per-output-channel layout.
  *   group_sizes [G] int32 on the device; rows of group g are [sum(sizes[:g]), +sizes[g]).
@@ -254,7 +255,7 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
  * LYRA_E_UNSUPPORTED for any other combination; lyra_decode_gemm_partials takes layout 1.  Results are the same
  * function of the same weights; the float32 summation order over K may differ from the row-major call's.
  *   lyra_gemm_packed_bytes  size of the packed copy (0 for bad arguments)
- *   lyra_gemm_pack          rhs [G,K,N] (rhs_dtype bf16 or e4m3fn) -> packed; layout 1 or 2; N % 8 == 0 (16 for layout 2)
+ *   lyra_gemm_pack          rhs [G,K,N] (rhs_dtype bf16, e4m3fn or e5m2) -> packed; layout 1 or 2; N % 8 == 0 (16 for layout 2)
  */
 size_t lyra_gemm_packed_bytes(int G, int K, int N, int rhs_dtype, int layout);
 int lyra_gemm_pack(const void* rhs, void* packed, int G, int K, int N, int rhs_dtype, int layout, lyra_stream_t stream);
@@ -322,7 +323,7 @@ int lyra_rmsnorm_proj_combine(const void* rows, const float* scores, const int32
  *   qkv [B,(N+2K)*H] bf16 -> per head rms_norm (qnorm/knorm [H] float32, both NULL = no QK norm) -> half-split
  *   rotary embedding with row position[b] of cos_t/sin_t [rope_rows, H/2] float32 (model.py:183-186) -> q_out
  *   [B,N,H] bf16; k and v rows are appended to the caches [B,K,S,H] at index position[b]: copied (bf16) or
- *   quantised with one scale per row, scale = amax/448 (1 for a zero row), code = e4m3fn_rne(clip(x/scale))
+ *   quantised with one scale per row, scale = amax/fmax (1 for a zero row; fmax 448 for e4m3fn, 57344 for e5m2), code = fp8_rne(clip(x/scale))
  *   (lyra/nn/quant.py:68-72, 213-231), scales into k_scale/v_scale [B,K,S].  Rows with position outside [0,S)
  *   are not appended.  H in {64,128}.
  *   v_unit [B,K,H] bf16 or NULL: receives the new value rows scaled to unit length, bf16(v * rsqrt(sum(v^2) + 1e-10))

@@ -7,11 +7,22 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
 
-DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32 = 0, 1, 2
+DTYPE_BF16, DTYPE_E4M3FN, DTYPE_F32, DTYPE_E5M2 = 0, 1, 2, 3
 RHS_SPAN_MAJOR, RHS_SPAN_MAJOR_GLU = 0x100, 0x200  # LYRA_RHS_SPAN_MAJOR(_GLU): OR-ed into a matmul's rhs_dtype
 LHS_TILED16, OUT_TILED16 = 0x400, 0x800  # LYRA_LHS_TILED16 / LYRA_OUT_TILED16, likewise
-ABI_VERSION = 14
+ABI_VERSION = 15
 E_UNSUPPORTED = -2  # LYRA_E_UNSUPPORTED: a shape or dtype the kernels do not cover
+
+
+def fp8_code(dtype) -> int:
+    """The C ABI's dtype code of a torch FP8 dtype (the two the reference's ``FP8_DTYPES`` names, lyra/nn/quant.py:10)."""
+    import torch
+
+    if dtype == torch.float8_e4m3fn:
+        return DTYPE_E4M3FN
+    if dtype == torch.float8_e5m2:
+        return DTYPE_E5M2
+    raise ValueError(f"no kernel reads {dtype}")
 
 _c = ctypes
 SIGNATURES = {

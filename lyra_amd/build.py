@@ -10,14 +10,17 @@ import tempfile
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "liblyra_hip.so")
-# (object name, source, extra flags).  decode_gemm.hip is compiled in two parts: its K-split kernels with the option
-# that keeps matrix-core accumulators in ordinary vector registers (fewer instructions there), the rest without it
-# (the expert kernel would spill registers with it).
+# (object name, source, extra flags).  decode_gemm.hip is compiled in four passes that run in parallel: the K-split kernels
+# with the option that keeps matrix-core accumulators in ordinary vector registers (fewer instructions there), the rest
+# without it (the expert kernel would spill registers with it); the kernels for e5m2 weights in passes of their own.
+_VGPR_FORM = ("-mllvm", "-amdgpu-mfma-vgpr-form")
 UNITS = (
     ("abi", "abi.hip", ()),
     ("decode_attention", "decode_attention.hip", ()),
-    ("decode_gemm", "decode_gemm.hip", ("-DLYRA_GEMM_MAIN_PART",)),
-    ("decode_gemm_splitk", "decode_gemm.hip", ("-DLYRA_GEMM_SPLITK_PART", "-mllvm", "-amdgpu-mfma-vgpr-form")),
+    ("decode_gemm", "decode_gemm.hip", ("-DLYRA_GEMM_PART=1",)),
+    ("decode_gemm_splitk", "decode_gemm.hip", ("-DLYRA_GEMM_PART=2", *_VGPR_FORM)),
+    ("decode_gemm_e5m2", "decode_gemm.hip", ("-DLYRA_GEMM_PART=3",)),
+    ("decode_gemm_splitk_e5m2", "decode_gemm.hip", ("-DLYRA_GEMM_PART=4", *_VGPR_FORM)),
     ("decode_fused", "decode_fused.hip", ()),
 )
 HIPCC_FLAGS = (

@@ -12,6 +12,15 @@ __device__ float e4m3fn_by_definition(int code) {
     return sign * ldexpf(1.f + (float)m / 8.f, e - 7);
 }
 
+// e5m2 code -> float by the format's definition (s.eeeee.mm, bias 15, exponent 31 = infinity / NaN)
+__device__ float e5m2_by_definition(int code) {
+    const float sign = (code & 0x80) ? -1.f : 1.f;
+    const int e = (code >> 2) & 0x1F, m = code & 3;
+    if (e == 0x1F) return m ? __builtin_nanf("") : sign * __builtin_inff();
+    if (e == 0) return sign * ldexpf((float)m / 4.f, -14);
+    return sign * ldexpf(1.f + (float)m / 4.f, e - 15);
+}
+
 __global__ __launch_bounds__(64) void selftest_kernel(int32_t* report) {
     const int lane = threadIdx.x;
     const int x = lane & 15, kb = lane >> 4;
@@ -54,6 +63,15 @@ __global__ __launch_bounds__(64) void selftest_kernel(int32_t* report) {
         const uint32_t blo = fp8x2_to_bf16x2(w, false), bhi = fp8x2_to_bf16x2(w, true);
         auto bf = [](uint32_t v, int h) { return __uint_as_float((h ? (v >> 16) : (v & 0xFFFFu)) << 16); };
         bad_cvt_bf16 += !same(bf(blo, 0), e0) + !same(bf(blo, 1), e1) + !same(bf(bhi, 0), e0) + !same(bf(bhi, 1), e1);
+        // the same for e5m2 (the finite codes: quantised data holds no others)
+        const float f0 = e5m2_by_definition(c0), f1 = e5m2_by_definition(255 - c0);
+        const bool fin0 = ((c0 >> 2) & 0x1F) != 0x1F, fin1 = (((255 - c0) >> 2) & 0x1F) != 0x1F;
+        const f32x2 lo5 = codes2_to_f32<2>(w, false), hi5 = codes2_to_f32<2>(w, true);
+        bad_cvt += (fin0 && (!same(lo5[0], f0) || !same(hi5[0], f0))) + (fin1 && (!same(lo5[1], f1) || !same(hi5[1], f1)));
+        const uint32_t blo5 = codes2_to_bf16x2<2>(w, false), bhi5 = codes2_to_bf16x2<2>(w, true);
+        bad_cvt_bf16 += (fin0 && (!same(bf(blo5, 0), f0) || !same(bf(bhi5, 0), f0))) + (fin1 && (!same(bf(blo5, 1), f1) || !same(bf(bhi5, 1), f1)));
+        // and the float32 -> code direction on every finite code's own value (exact round trip)
+        bad_cvt += (fin0 && f32_to_e5m2(f0) != (uint8_t)c0 && f0 != 0.f) + (c0 != 0x7F && c0 != 0xFF && e0 != 0.f && f32_to_e4m3fn(e0) != (uint8_t)c0);
     }
     // [3] float32 -> bf16 packing rounds to nearest even
     {

@@ -135,7 +135,7 @@ __device__ __forceinline__ void xsa_finish(const AttnParams& p, float* sm_t, flo
 }
 
 // Raw (still quantised) operands of one 32-token tile as this lane holds them.
-template <int H, bool FP8>
+template <int H, int FP8>
 struct RawK {
     static constexpr int ES = FP8 ? 1 : 2;
     static constexpr int KW = ES * H / 16;  // dwords of one K row held by a lane: 16-byte pieces at p * 64 + kb * 16
@@ -145,7 +145,7 @@ struct RawS {  // per-token scales of the 8 tokens whose logits this lane holds
     float ks[8];
     float vs[8];
 };
-template <int H, bool FP8>
+template <int H, int FP8>
 struct RawV {
     static constexpr int ES = FP8 ? 1 : 2;
     static constexpr int VW = ES * H / 64;  // dwords of one V row held by a lane (H/16 columns)
@@ -163,7 +163,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
-template <int H, bool FP8>
+template <int H, int FP8>
 __device__ __forceinline__ void load_k(RawK<H, FP8>& t, const Slab& sl, int base, bool live) {
     constexpr int ES = RawK<H, FP8>::ES;
     constexpr int KW = RawK<H, FP8>::KW;
@@ -206,7 +206,7 @@ __device__ __forceinline__ void load_s(RawS& t, const Slab& sl, int base, bool l
     }
 }
 
-template <int H, bool FP8>
+template <int H, int FP8>
 __device__ __forceinline__ void load_v(RawV<H, FP8>& t, const Slab& sl, int base, bool live) {
     constexpr int ES = RawV<H, FP8>::ES;
     constexpr int VW = RawV<H, FP8>::VW;
@@ -241,7 +241,7 @@ struct Acc {
 };
 
 // First third of a tile: S^T = K Q^T on the matrix cores (raw FP8 values, scales applied later).
-template <int H, bool FP8>
+template <int H, int FP8>
 __device__ __forceinline__ void tile_logits(const RawK<H, FP8>& t, const uint16_t* sm_q, int lane, f32x4 (&s)[2]) {
     constexpr int NC = H / 32;
     constexpr int QP = H + 8;  // LDS pitch of a q row in bf16 elements
@@ -261,7 +261,7 @@ __device__ __forceinline__ void tile_logits(const RawK<H, FP8>& t, const uint16_
         for (int c = 0; c < NC; ++c) {
             bf16x8 a;
             if constexpr (FP8) {
-                a = fp8x8_to_bf16x8(t.k[j][2 * c], t.k[j][2 * c + 1]);
+                a = fp8x8_to_bf16x8<FP8>(t.k[j][2 * c], t.k[j][2 * c + 1]);
             } else {
                 Pack8 pk;
                 pk.u[0] = t.k[j][4 * c];
@@ -278,7 +278,7 @@ __device__ __forceinline__ void tile_logits(const RawK<H, FP8>& t, const uint16_
 // Second third: the online-softmax update, producing the probability operand (already multiplied by the
 // V scales).  MASKED tiles straddle the ends of the visible range: logits of invisible keys become -inf
 // and their probabilities exactly 0.
-template <int H, bool FP8, bool MASKED>
+template <int H, int FP8, bool MASKED>
 __device__ __forceinline__ bf16x8 tile_softmax(const f32x4 (&s)[2], const RawS& t, int base, int lo, int hi, float scale_log2,
                                                int lane, Acc<H>& acc, uint32_t& vis_bits) {
     constexpr int CB = H / 16;
@@ -335,7 +335,7 @@ __device__ __forceinline__ bf16x8 tile_softmax(const f32x4 (&s)[2], const RawS& 
 // Last third of a tile: O^T += V^T P^T.  Element i of column c of the V^T operand is V[token i, c]; the
 // bf16 pack step pairs two tokens, which transposes the row-major cache for free.  In MASKED tiles the
 // rows of invisible keys are zeroed first so unwritten cache memory (possibly NaN) cannot reach O.
-template <int H, bool FP8, bool MASKED>
+template <int H, int FP8, bool MASKED>
 __device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_t vis_bits, Acc<H>& acc) {
     constexpr int CB = H / 16;
     if constexpr (MASKED) {
@@ -351,8 +351,8 @@ __device__ __forceinline__ void tile_values(RawV<H, FP8>& t, bf16x8 pop, uint32_
             Pack8 v0, v1;
 #pragma unroll
             for (int i = 0; i < 8; i += 2) {
-                const f32x2 fa = fp8x2_to_f32(t.v[i][c >> 2], (c & 2) != 0);
-                const f32x2 fb = fp8x2_to_f32(t.v[i + 1][c >> 2], (c & 2) != 0);
+                const f32x2 fa = codes2_to_f32<FP8>(t.v[i][c >> 2], (c & 2) != 0);
+                const f32x2 fb = codes2_to_f32<FP8>(t.v[i + 1][c >> 2], (c & 2) != 0);
                 v0.u[i >> 1] = pack_bf16(fa[0], fb[0]);
                 v1.u[i >> 1] = pack_bf16(fa[1], fb[1]);
             }
@@ -462,18 +462,20 @@ __device__ __forceinline__ void sum_head(const AttnParams& p, __amdgpu_buffer_rs
 
 // The cache bytes of one finished row (this lane's elements a, c) of the key (slot 0) or value (slot 1) head, left in
 // LDS: H codes and the row's scale for an FP8 cache, H bf16 values otherwise.  stage: [2][H * ES] bytes, then 2 floats.
-template <int H, bool FP8>
+template <int H, int FP8>
 __device__ __forceinline__ void stage_row(uint8_t* stage, int slot, int lane, float a, float c) {
     constexpr int half = H / 2, ES = FP8 ? 1 : 2;
     const bool active = lane < half;
     if constexpr (FP8) {
         const float amax = wave_max(fmaxf(fabsf(a), fabsf(c)));
-        const float scale = amax > 0.f ? amax / 448.f : 1.f;
+        constexpr bool e5m2 = FP8 == 2;
+        const float fmax = fp8_format_max(e5m2);
+        const float scale = amax > 0.f ? amax / fmax : 1.f;
         const float inv = 1.0f / scale;
         if (active) {
             uint8_t* dst = stage + slot * H;
-            dst[lane] = f32_to_e4m3fn(fminf(fmaxf(a * inv, -448.f), 448.f));
-            dst[lane + half] = f32_to_e4m3fn(fminf(fmaxf(c * inv, -448.f), 448.f));
+            dst[lane] = f32_to_fp8_code(fminf(fmaxf(a * inv, -fmax), fmax), e5m2);
+            dst[lane + half] = f32_to_fp8_code(fminf(fmaxf(c * inv, -fmax), fmax), e5m2);
         }
         if (lane == 0) ((float*)(stage + 2 * H * ES))[slot] = scale;
     } else if (active) {
@@ -488,7 +490,7 @@ __device__ __forceinline__ void stage_row(uint8_t* stage, int slot, int lane, fl
 // written (`live` false: not the wavefront that owns the new key), so that no memory operation sits inside a branch:
 // behind a branch the compiler no longer knows how many operations are in flight and makes the tile loop wait for all of
 // them in every pass.
-template <int H, bool FP8>
+template <int H, int FP8>
 __device__ __forceinline__ void append_staged(const Slab& sl, const uint8_t* stage, int pos, bool live, int lane) {
     constexpr int ES = FP8 ? 1 : 2, DW = H * ES / 4;  // dwords per row (16 to 64)
     const bool on = live && lane < DW;
@@ -505,7 +507,7 @@ __device__ __forceinline__ void append_staged(const Slab& sl, const uint8_t* sta
 }
 
 // QKV: the launch also does the step in front of the attention (lyra_decode_attention_qkv).
-template <int H, bool FP8, bool VEC4, int WAVES, bool EARLY, int DEPTH, bool QKV = false>
+template <int H, int FP8, bool VEC4, int WAVES, bool EARLY, int DEPTH, bool QKV = false>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(DEPTH > 1 ? 2 : (WAVES >= 8 ? 4 : 3))))
 void decode_attention_kernel(AttnParams p) {
     static_assert(!QKV || DEPTH == 1, "the fused front step knows one register set per wavefront");
@@ -893,7 +895,7 @@ void decode_attention_kernel(AttnParams p) {
 // rows that land on the same compute unit set the time of the launch (gpt-oss shape, lengths 256...4096: 39 us, of which
 // only 24 us are the average unit's share).  The first tile of the next pair is requested before the current pair's
 // wavefronts are merged, so a compute unit keeps streaming across pairs.
-template <int H, bool FP8>
+template <int H, int FP8>
 struct PairState {
     Slab sl;
     int b, kh, pos;
@@ -902,7 +904,7 @@ struct PairState {
     uint16_t gate_raw;
 };
 
-template <int H, bool FP8, bool VEC4>
+template <int H, int FP8, bool VEC4>
 __device__ __forceinline__ void request_pair(const AttnParams& p, int pair, bool live_pair, const int* sm_pos, const int* sm_order,
                                              int tid, int lane, int wave, PairState<H, FP8>& st, RawK<H, FP8>& rk, RawS& rs,
                                              RawV<H, FP8>& rv) {
@@ -937,7 +939,7 @@ __device__ __forceinline__ void request_pair(const AttnParams& p, int pair, bool
     load_v<H, FP8>(rv, st.sl, wave * kTile, live);
 }
 
-template <int H, bool FP8, bool VEC4, int WAVES>
+template <int H, int FP8, bool VEC4, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4)))  // one workgroup per compute unit
 void decode_attention_rows_kernel(AttnParams p) {
     constexpr int CB = H / 16;
@@ -1185,9 +1187,9 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || H <= 0 || N % K || sliding_window < 0) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
     if ((xsa_v == nullptr) != (xsa_alpha == nullptr)) return LYRA_E_BADARG;
-    if (kv_dtype != LYRA_DTYPE_BF16 && kv_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    if (kv_dtype != LYRA_DTYPE_BF16 && kv_dtype != LYRA_DTYPE_E4M3FN && kv_dtype != LYRA_DTYPE_E5M2) return LYRA_E_UNSUPPORTED;
     if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
-    const bool fp8 = kv_dtype == LYRA_DTYPE_E4M3FN;
+    const bool fp8 = kv_dtype != LYRA_DTYPE_BF16, e5m2 = kv_dtype == LYRA_DTYPE_E5M2;
     if (fp8 != (k_scale != nullptr) || fp8 != (v_scale != nullptr)) return LYRA_E_BADARG;
     const int G = N / K;
     if ((H != 64 && H != 128) || G > 16) return LYRA_E_UNSUPPORTED;
@@ -1303,14 +1305,19 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
         if (waves == 4) LYRA_LAUNCH_ATTN_R(HH, F, V, 4); \
         else LYRA_LAUNCH_ATTN_R(HH, F, V, 8);            \
     } while (0)
+        // (the second argument is the cache format: 0 bf16, 1 e4m3fn, 2 e5m2)
         if (H == 128) {
-            if (!fp8) LYRA_LAUNCH_ATTN_RW(128, false, false);
-            else if (vec4) LYRA_LAUNCH_ATTN_RW(128, true, true);
-            else LYRA_LAUNCH_ATTN_RW(128, true, false);
+            if (!fp8) LYRA_LAUNCH_ATTN_RW(128, 0, false);
+            else if (e5m2 && vec4) LYRA_LAUNCH_ATTN_RW(128, 2, true);
+            else if (e5m2) LYRA_LAUNCH_ATTN_RW(128, 2, false);
+            else if (vec4) LYRA_LAUNCH_ATTN_RW(128, 1, true);
+            else LYRA_LAUNCH_ATTN_RW(128, 1, false);
         } else {
-            if (!fp8) LYRA_LAUNCH_ATTN_RW(64, false, false);
-            else if (vec4) LYRA_LAUNCH_ATTN_RW(64, true, true);
-            else LYRA_LAUNCH_ATTN_RW(64, true, false);
+            if (!fp8) LYRA_LAUNCH_ATTN_RW(64, 0, false);
+            else if (e5m2 && vec4) LYRA_LAUNCH_ATTN_RW(64, 2, true);
+            else if (e5m2) LYRA_LAUNCH_ATTN_RW(64, 2, false);
+            else if (vec4) LYRA_LAUNCH_ATTN_RW(64, 1, true);
+            else LYRA_LAUNCH_ATTN_RW(64, 1, false);
         }
 #undef LYRA_LAUNCH_ATTN_RW
 #undef LYRA_LAUNCH_ATTN_R
@@ -1332,13 +1339,17 @@ static int run_attention(const void* q, const void* k, const void* v, const floa
         else LYRA_LAUNCH_ATTN_W(HH, F, V, 16);                  \
     } while (0)
     if (H == 128) {
-        if (!fp8) LYRA_LAUNCH_ATTN(128, false, false);
-        else if (vec4) LYRA_LAUNCH_ATTN(128, true, true);
-        else LYRA_LAUNCH_ATTN(128, true, false);
+        if (!fp8) LYRA_LAUNCH_ATTN(128, 0, false);
+        else if (e5m2 && vec4) LYRA_LAUNCH_ATTN(128, 2, true);
+        else if (e5m2) LYRA_LAUNCH_ATTN(128, 2, false);
+        else if (vec4) LYRA_LAUNCH_ATTN(128, 1, true);
+        else LYRA_LAUNCH_ATTN(128, 1, false);
     } else {
-        if (!fp8) LYRA_LAUNCH_ATTN(64, false, false);
-        else if (vec4) LYRA_LAUNCH_ATTN(64, true, true);
-        else LYRA_LAUNCH_ATTN(64, true, false);
+        if (!fp8) LYRA_LAUNCH_ATTN(64, 0, false);
+        else if (e5m2 && vec4) LYRA_LAUNCH_ATTN(64, 2, true);
+        else if (e5m2) LYRA_LAUNCH_ATTN(64, 2, false);
+        else if (vec4) LYRA_LAUNCH_ATTN(64, 1, true);
+        else LYRA_LAUNCH_ATTN(64, 1, false);
     }
 #undef LYRA_LAUNCH_ATTN
 #undef LYRA_LAUNCH_ATTN_W

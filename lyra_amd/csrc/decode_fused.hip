@@ -222,7 +222,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_proj_kernel(NormProjPara
 // half-split rotary embedding mixes (lyra/model.py:183-186).
 //   q, k: rms_norm over the head (model.py:315-320) -> bf16 -> rotate -> bf16
 //   k, v: written at `position` into the cache; FP8 caches quantise the row with block (1, H):
-//         scale = amax / 448 (1 if the row is zero), code = fp8_rne(clip(x / scale))   (lyra/nn/quant.py:68-72)
+//         scale = amax / fmax (1 if the row is zero; fmax = 448 for e4m3fn, 57344 for e5m2), code = fp8_rne(clip(x / scale))
+//         (lyra/nn/quant.py:68-72)
 struct QkvPostParams {
     const uint16_t* qkv;  // [B, (N + 2K) * H]
     const float* qnorm;   // [H] or null
@@ -241,6 +242,7 @@ struct QkvPostParams {
     float eps;
     const float* partials;  // [splits, B, (N + 2K) * H] K slices of the projection not summed yet, or null (then qkv)
     int splits;
+    bool e5m2;  // the 1-byte format of a quantised cache: e5m2 instead of e4m3fn
 };
 
 __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
@@ -318,12 +320,13 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
     float* scales = is_k ? p.k_scale : p.v_scale;
     if (scales) {
         const float amax = wave_max(fmaxf(fabsf(a), fabsf(c)));
-        const float scale = amax > 0.f ? amax / 448.f : 1.f;
+        const float fmax = fp8_format_max(p.e5m2);
+        const float scale = amax > 0.f ? amax / fmax : 1.f;
         const float inv = 1.0f / scale;
         if (active) {
             uint8_t* dst = (uint8_t*)cache + row * p.H;
-            dst[lane] = f32_to_e4m3fn(fminf(fmaxf(a * inv, -448.f), 448.f));
-            dst[lane + half] = f32_to_e4m3fn(fminf(fmaxf(c * inv, -448.f), 448.f));
+            dst[lane] = f32_to_fp8_code(fminf(fmaxf(a * inv, -fmax), fmax), p.e5m2);
+            dst[lane + half] = f32_to_fp8_code(fminf(fmaxf(c * inv, -fmax), fmax), p.e5m2);
         }
         if (lane == 0) scales[row] = scale;
     } else if (active) {
@@ -1109,12 +1112,13 @@ extern "C" int lyra_qkv_post_sum(const void* qkv, const float* partials, int spl
     if (B <= 0 || N <= 0 || K <= 0 || S <= 0 || rope_rows <= 0) return LYRA_E_BADARG;
     if (H != 64 && H != 128) return LYRA_E_UNSUPPORTED;
     if ((qnorm == nullptr) != (knorm == nullptr)) return LYRA_E_BADARG;
-    const bool fp8 = kv_dtype == LYRA_DTYPE_E4M3FN;
+    const bool fp8 = kv_dtype == LYRA_DTYPE_E4M3FN || kv_dtype == LYRA_DTYPE_E5M2;
     if (!fp8 && kv_dtype != LYRA_DTYPE_BF16) return LYRA_E_UNSUPPORTED;
     if (fp8 != (k_scale != nullptr) || fp8 != (v_scale != nullptr)) return LYRA_E_BADARG;
     if (position_stride != 0 && position_stride != 1) return LYRA_E_BADARG;
     QkvPostParams p{(const uint16_t*)qkv, qnorm, knorm, cos_t, sin_t, position, position_stride, (uint16_t*)q_out,
-                    k_cache, v_cache, k_scale, v_scale, (uint16_t*)v_unit, B, N, K, S, H, rope_rows, eps, partials, splits};
+                    k_cache, v_cache, k_scale, v_scale, (uint16_t*)v_unit, B, N, K, S, H, rope_rows, eps, partials, splits,
+                    kv_dtype == LYRA_DTYPE_E5M2};
     const int items = B * (N + 2 * K);
     hipLaunchKernelGGL(qkv_post_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, p);
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;

@@ -14,22 +14,34 @@
 // rows in the bf16 pack step yields the K-major B operand, so the transposition costs nothing.
 //   D[16 rows, 16 cols] += X[16 rows x 32 k] . W[32 k x 16 cols]   for each of the 8 column phases.
 //
-// This file is compiled twice.  With LYRA_GEMM_SPLITK_PART it yields only the K-split kernel and its launcher,
-// built with the compiler's option that keeps matrix-core accumulators in ordinary vector registers: those
-// kernels do one or two matrix instructions per accumulator and the copies to and from the accumulator file were
-// a sixth of their instructions.  With LYRA_GEMM_MAIN_PART it yields everything else (the option makes the expert
-// kernel spill registers).  With neither macro it is one complete translation unit.
+// This file is compiled in several passes, selected by LYRA_GEMM_PART, and the objects are linked:
+//   1  the C entry points, the planning, the finish and pack kernels and the launches of the bf16 and e4m3fn kernels
+//   2  the K-split kernels for bf16 and e4m3fn weights, built with the compiler's option that keeps matrix-core
+//      accumulators in ordinary vector registers: those kernels do one or two matrix instructions per accumulator and the
+//      copies to and from the accumulator file were a sixth of their instructions (the option makes the expert kernel
+//      spill registers, so the other passes are built without it)
+//   3  the launches of pass 1 for e5m2 weights;  4  the kernels of pass 2 for e5m2 weights
+// Without the macro the file is one complete translation unit.
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
 #include "lyra_device.h"
 
-#if defined(LYRA_GEMM_SPLITK_PART) && defined(LYRA_GEMM_MAIN_PART)
-#error "LYRA_GEMM_SPLITK_PART and LYRA_GEMM_MAIN_PART select different halves of this file"
+#ifndef LYRA_GEMM_PART
+#define LYRA_GEMM_PART 0
 #endif
+#if LYRA_GEMM_PART < 0 || LYRA_GEMM_PART > 4
+#error "LYRA_GEMM_PART: 0 (everything) or one of the passes 1-4"
+#endif
+#define LYRA_GEMM_HAS_ENTRY (LYRA_GEMM_PART == 0 || LYRA_GEMM_PART == 1)
+#define LYRA_GEMM_HAS_LAUNCH (LYRA_GEMM_PART == 0 || LYRA_GEMM_PART == 1 || LYRA_GEMM_PART == 3)
+#define LYRA_GEMM_HAS_SPLITK (LYRA_GEMM_PART == 0 || LYRA_GEMM_PART == 2 || LYRA_GEMM_PART == 4)
 
 namespace lyra {
+
+// the weight formats of one byte per element (block-scaled)
+static inline bool one_byte_format(int dtype) { return dtype == LYRA_DTYPE_E4M3FN || dtype == LYRA_DTYPE_E5M2; }
 
 struct GemmParams {
     const uint16_t* lhs;
@@ -120,7 +132,9 @@ __device__ __forceinline__ float swiglu_one(float glu, float lin, float beta, fl
 
 constexpr int kGemmWaves = 4;  // wavefronts per workgroup, each on its own 128-column span
 
-template <bool FP8>
+// The template argument FP8 of everything below is the weight format: 0 bf16, 1 e4m3fn, 2 e5m2 (both 1-byte formats go the
+// same way - codes converted exactly to bf16, block scales on the float32 accumulators - and differ in one instruction).
+template <int FP8>
 struct RawW {
     static constexpr int WW = FP8 ? 2 : 4;  // dwords per lane per weight row (8 columns)
     uint32_t w[8][WW];
@@ -128,7 +142,7 @@ struct RawW {
 
 // Two of the 8 weight rows of this lane (rows kk + 8*kb + 2*pair, +1), 8 columns each.  The lane part of the
 // address is fixed (voff); the row part is uniform and travels in a scalar register.
-template <bool FP8>
+template <int FP8>
 __device__ __forceinline__ void load_w_pair(RawW<FP8>& t, int pair, __amdgpu_buffer_rsrc_t rsrc, int voff, int kk, int row_bytes) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -153,7 +167,7 @@ __device__ __forceinline__ void load_w_pair(RawW<FP8>& t, int pair, __amdgpu_buf
 // that the number of loads in flight is the same on every path and each wait covers exactly the loads it needs
 // (a load inside a branch makes the compiler wait for every outstanding load at the next use).
 
-template <bool FP8>
+template <int FP8>
 __device__ __forceinline__ void load_w_pair_if(bool live, RawW<FP8>& t, int pair, __amdgpu_buffer_rsrc_t rsrc, int voff, int kk,
                                                int row_bytes) {
     load_w_pair<FP8>(t, pair, rsrc, live ? voff : kNoLoad, live ? kk : 0, live ? row_bytes : 0);
@@ -161,7 +175,7 @@ __device__ __forceinline__ void load_w_pair_if(bool live, RawW<FP8>& t, int pair
 
 // Element `pair` of the K-major B operands of all 8 column phases: pairing two weight rows in the bf16 pack
 // step transposes the row-major weights for free.
-template <bool FP8>
+template <int FP8>
 __device__ __forceinline__ void convert_pair(const RawW<FP8>& t, int pair, Pack8 (&bop)[8]) {
     const int i = 2 * pair;
 #pragma unroll
@@ -170,8 +184,8 @@ __device__ __forceinline__ void convert_pair(const RawW<FP8>& t, int pair, Pack8
             // the two rows' codes of columns c, c + 1 side by side (row i, row i + 1, row i, row i + 1), then one exact
             // conversion per pair: 3 instructions for 4 weights
             const uint32_t both = __builtin_amdgcn_perm(t.w[i + 1][c >> 2], t.w[i][c >> 2], (c & 2) ? 0x07030602u : 0x05010400u);
-            bop[c].u[pair] = fp8x2_to_bf16x2(both, false);
-            bop[c + 1].u[pair] = fp8x2_to_bf16x2(both, true);
+            bop[c].u[pair] = codes2_to_bf16x2<FP8>(both, false);
+            bop[c + 1].u[pair] = codes2_to_bf16x2<FP8>(both, true);
         } else {
             const uint32_t a = t.w[i][c >> 1], b = t.w[i + 1][c >> 1];
             bop[c].u[pair] = __builtin_amdgcn_perm(b, a, 0x05040100u);
@@ -184,7 +198,7 @@ __device__ __forceinline__ void convert_pair(const RawW<FP8>& t, int pair, Pack8
 // one row pair and all phases, done for all row pairs and one pair of phases).
 // SCALED: every value is multiplied by `scale` in float32 before it is rounded to bf16 - the dequantisation of the plain-JAX
 // path, bit for bit: dequantize() forms f32(code) * scale and casts to the activation dtype (lyra/nn/quant.py:82-85).
-template <bool FP8, bool SCALED = false>
+template <int FP8, bool SCALED = false>
 __device__ __forceinline__ void convert_colpair(const RawW<FP8>& t, int cp, Pack8& b0, Pack8& b1, float scale = 1.f) {
     const int c = 2 * cp;
 #pragma unroll
@@ -194,8 +208,8 @@ __device__ __forceinline__ void convert_colpair(const RawW<FP8>& t, int cp, Pack
             // (the byte shuffle + single conversion of convert_pair - 3 instead of 4 instructions for 4 weights - was
             // measured here too: no faster, the lyra-max down projection 1.3 % slower; this loop hides its conversions
             // behind matrix instructions already)
-            f32x2 fa = fp8x2_to_f32(t.w[i][c >> 2], (c & 2) != 0);
-            f32x2 fb = fp8x2_to_f32(t.w[i + 1][c >> 2], (c & 2) != 0);
+            f32x2 fa = codes2_to_f32<FP8>(t.w[i][c >> 2], (c & 2) != 0);
+            f32x2 fb = codes2_to_f32<FP8>(t.w[i + 1][c >> 2], (c & 2) != 0);
             if constexpr (SCALED) {
                 fa[0] *= scale;
                 fa[1] *= scale;
@@ -270,7 +284,7 @@ __device__ __forceinline__ void store_tile_max(const GemmParams& p, const float 
 
 constexpr int kTileMaxPitch = 20;  // floats per row of a wavefront's tile-maximum staging area (conflict-free for 4 rows x 16 lanes)
 
-template <bool FP8, int MT, bool TMAX = false>
+template <int FP8, int MT, bool TMAX = false>
 __global__ __launch_bounds__(MT == 1 ? 768 : 512) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 3 : 2)))
 void decode_gemm_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
@@ -467,7 +481,7 @@ void decode_gemm_kernel(GemmParams p) {
     }
 }
 
-#ifndef LYRA_GEMM_SPLITK_PART
+#if LYRA_GEMM_HAS_ENTRY
 // Second pass when K was split across workgroups: sum the partials, then bias / SwiGLU / cast.
 // One thread per 4 output columns.
 __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
@@ -537,7 +551,7 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
     }
     }
 }
-#endif  // !LYRA_GEMM_SPLITK_PART
+#endif  // LYRA_GEMM_HAS_ENTRY
 
 // ---- small weight sets: one group, a few MB of weights (the dense projections of a decode layer) -----------------
 // Such a product is bound by latency, not bandwidth: what counts is how many weight rows are in flight.  A workgroup
@@ -547,7 +561,7 @@ __global__ __launch_bounds__(256) void decode_gemm_finish_kernel(GemmParams p) {
 // pass, no workspace.  Rows at or beyond group_sizes[0] multiply zeros (epilogue(0), lax.ragged_dot semantics).
 constexpr int kSmallWaves = 8;
 
-template <bool FP8, int DEPTH, bool STEP_SCALES, bool ONE_ROUND>
+template <int FP8, int DEPTH, bool STEP_SCALES, bool ONE_ROUND>
 __global__ __launch_bounds__(kSmallWaves * 64) void decode_gemm_small_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSmallWaves][16][128]
@@ -760,7 +774,7 @@ constexpr int kSplitPitch = 132;  // floats per row of a partial tile in LDS (12
 // the DEPTH register sets are refilled as they are used, wavefronts interleave, STEP_SCALES is 0 or 2.
 // MT: 16-row tiles the instantiation holds (1, 2 or 4 = row blocks of 16, 32, 64 rows): a launch with smaller blocks runs
 // less code - these launches are bound by the instructions one wavefront per SIMD gets through, not by arithmetic.
-template <bool FP8, int DEPTH, int STEP_SCALES, bool LOOP, int MT = 4>
+template <int FP8, int DEPTH, int STEP_SCALES, bool LOOP, int MT = 4>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_splitk_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     extern __shared__ float sm_part[];  // [kSplitWaves][64][kSplitPitch]
@@ -1066,7 +1080,7 @@ __device__ __forceinline__ unsigned long long wg_scan_exclusive4(unsigned long l
 // weights.  With SwiGLU a span then holds 64 gate columns and their 64 linear columns, so a unit of one span is half as
 // wide as without the copy and a launch has twice the units to deal out; whether wavefront pairs take two spans (as many
 // rounds as before) or all four wavefronts one span (short lists: finer shares) is decided once the unit list is known.
-template <bool FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false, bool PACKED = false>
+template <int FP8, bool STEP_SCALES, int ROUNDS, bool SLICED, bool WIDE_DYN = false, bool PACKED = false>
 __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(GemmParams p) {
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int DEPTH = FP8 ? 4 : 2;
@@ -1612,7 +1626,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 // ---- span-major copy of a weight array (done once, when the weights are loaded) ---------------------------------------
 // One thread moves 8 consecutive elements of a packed row: they come from 8 consecutive columns of the reference's array
 // (widths are multiples of 8, or 16 with gate and linear halves) or are zeros where the span runs past the last column.
-#ifndef LYRA_GEMM_SPLITK_PART
+#if LYRA_GEMM_HAS_ENTRY
 struct PackParams {
     const uint8_t* src;
     uint8_t* dst;
@@ -1646,7 +1660,7 @@ __global__ __launch_bounds__(256) void gemm_pack_kernel(PackParams p) {
         }
     }
 }
-#endif  // !LYRA_GEMM_SPLITK_PART
+#endif  // LYRA_GEMM_HAS_ENTRY
 
 static int packed_spans(int N, int layout) { return layout == 2 ? (N / 2 + 63) / 64 : (N + 127) / 128; }
 
@@ -1754,65 +1768,234 @@ static GemmPlan plan_gemm(int M, int G, int K, int N, int bk, int fused_swiglu, 
     return pl;
 }
 
-// Launches the K-split kernel of a plan with split_k set; p.part receives [ksplit, M, N] float32 slices.
-int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st);
-#ifndef LYRA_GEMM_MAIN_PART
-int launch_split_k(const GemmParams& p, const GemmPlan& pl, bool fp8, hipStream_t st) {
+// Launches the K-split kernel of a plan with split_k set for weights of format WT (0 bf16, 1 e4m3fn, 2 e5m2); p.part
+// receives [ksplit, M, N] float32 slices.
+template <int WT>
+int launch_split_k_fmt(const GemmParams& p, const GemmPlan& pl, hipStream_t st);
+// Sums the K slices in p.part and applies the epilogue (the finish kernel lives in the pass with the entry points).
+int launch_finish(const GemmParams& p, hipStream_t st);
+
+#if LYRA_GEMM_HAS_SPLITK
+template <int WT>
+int launch_split_k_fmt(const GemmParams& p, const GemmPlan& pl, hipStream_t st) {
     const dim3 grid(pl.spans, pl.ksplit, pl.row_par), block(kSplitWaves * 64);
     const size_t lds = (size_t)kSplitWaves * 64 * kSplitPitch * sizeof(float);
     const int depth = (pl.kpart / 32 + kSplitWaves - 1) / kSplitWaves;  // 1..4 steps per wavefront, or more: the looping variant
     const bool loop = depth > 4;
     // scales that change along K: free when every wavefront's rows (32 * depth) lie within one scale block
     const int step_scales =
-        !(fp8 && p.scale_mode == 1 && p.bk < p.K) ? 0 : ((!loop && p.bk % (32 * std::max(1, std::min(depth, 4))) == 0) ? 1 : 2);
-#define LYRA_SPLITK_M(F, D, S, M_)                                                                                    \
+        !(WT != 0 && p.scale_mode == 1 && p.bk < p.K) ? 0 : ((!loop && p.bk % (32 * std::max(1, std::min(depth, 4))) == 0) ? 1 : 2);
+#define LYRA_SPLITK_M(D, S, M_)                                                                                        \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, D, S, false, M_>, \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<WT, D, S, false, M_>, \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, D, S, false, M_>), grid, block, lds, st, p);                 \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<WT, D, S, false, M_>), grid, block, lds, st, p);                \
     } while (0)
-#define LYRA_SPLITK(F, D, S)                              \
-    do {                                                  \
-        if (pl.row_block <= 16) LYRA_SPLITK_M(F, D, S, 1); \
-        else if (pl.row_block <= 32) LYRA_SPLITK_M(F, D, S, 2); \
-        else LYRA_SPLITK_M(F, D, S, 4);                   \
+#define LYRA_SPLITK(D, S)                              \
+    do {                                               \
+        if (pl.row_block <= 16) LYRA_SPLITK_M(D, S, 1); \
+        else if (pl.row_block <= 32) LYRA_SPLITK_M(D, S, 2); \
+        else LYRA_SPLITK_M(D, S, 4);                   \
     } while (0)
-#define LYRA_SPLITK_LOOP(F, S)                                                                                        \
+#define LYRA_SPLITK_LOOP(S)                                                                                            \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<F, (F ? 4 : 2), S, true>, \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_splitk_kernel<WT, (WT ? 4 : 2), S, true>, \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
         if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_splitk_kernel<F, (F ? 4 : 2), S, true>), grid, block, lds, st, p);            \
+        hipLaunchKernelGGL((decode_gemm_splitk_kernel<WT, (WT ? 4 : 2), S, true>), grid, block, lds, st, p);           \
     } while (0)
-#define LYRA_SPLITK_D(F, S)                   \
-    do {                                      \
-        if (depth <= 1) LYRA_SPLITK(F, 1, S); \
-        else if (depth == 2) LYRA_SPLITK(F, 2, S); \
-        else if (depth == 3) LYRA_SPLITK(F, 3, S); \
-        else LYRA_SPLITK(F, 4, S);            \
+#define LYRA_SPLITK_D(S)                   \
+    do {                                   \
+        if (depth <= 1) LYRA_SPLITK(1, S); \
+        else if (depth == 2) LYRA_SPLITK(2, S); \
+        else if (depth == 3) LYRA_SPLITK(3, S); \
+        else LYRA_SPLITK(4, S);            \
     } while (0)
-    if (loop) {
-        if (step_scales == 2) LYRA_SPLITK_LOOP(true, 2);
-        else if (fp8) LYRA_SPLITK_LOOP(true, 0);
-        else LYRA_SPLITK_LOOP(false, 0);
-    } else if (step_scales == 1) LYRA_SPLITK_D(true, 1);
-    else if (step_scales == 2) LYRA_SPLITK_D(true, 2);
-    else if (fp8) LYRA_SPLITK_D(true, 0);
-    else LYRA_SPLITK_D(false, 0);
+    if constexpr (WT != 0) {
+        if (loop) {
+            if (step_scales == 2) LYRA_SPLITK_LOOP(2);
+            else LYRA_SPLITK_LOOP(0);
+        } else if (step_scales == 1) LYRA_SPLITK_D(1);
+        else if (step_scales == 2) LYRA_SPLITK_D(2);
+        else LYRA_SPLITK_D(0);
+    } else {
+        if (loop) LYRA_SPLITK_LOOP(0);
+        else LYRA_SPLITK_D(0);
+    }
 #undef LYRA_SPLITK_D
 #undef LYRA_SPLITK_LOOP
 #undef LYRA_SPLITK
 #undef LYRA_SPLITK_M
     return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
 }
-#endif  // !LYRA_GEMM_MAIN_PART
+#if LYRA_GEMM_PART == 2
+template int launch_split_k_fmt<0>(const GemmParams&, const GemmPlan&, hipStream_t);
+template int launch_split_k_fmt<1>(const GemmParams&, const GemmPlan&, hipStream_t);
+#elif LYRA_GEMM_PART == 4
+template int launch_split_k_fmt<2>(const GemmParams&, const GemmPlan&, hipStream_t);
+#endif
+#endif  // LYRA_GEMM_HAS_SPLITK
+
 
 }  // namespace lyra
 
-#ifndef LYRA_GEMM_SPLITK_PART
+namespace lyra {
+// Launches the kernels of a plan for weights of format WT (0 bf16, 1 e4m3fn, 2 e5m2); p is complete except even_spans.
+template <int WT>
+int launch_planned(GemmParams p, const GemmPlan& pl, int layout, int fused_swiglu, float* tile_max, hipStream_t st);
+
+#if LYRA_GEMM_HAS_LAUNCH
+template <int WT>
+int launch_planned(GemmParams p, const GemmPlan& pl, int layout, int fused_swiglu, float* tile_max, hipStream_t st) {
+    constexpr bool fp8 = WT != 0;
+    const int M = p.M, G = p.G, K = p.K, N = p.N;
+    if (pl.grouped) {
+        // one workgroup per compute unit (more would only queue behind the LDS tiles), fewer when there is less work
+        const long most_blocks = std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
+        // (packed: units of one span unless the list is long enough for units of two - the kernel's own rule, on the most
+        // row blocks the shapes allow)
+        const bool packed_wide = layout && 4 * most_blocks * ((p.pspans + 1) / 2) >= 7 * (long)kGroupMaxWgs;
+        const long most_units = (layout ? (long)p.pspans : (long)pl.spans) * most_blocks;
+        const int gkw = layout ? (packed_wide ? 2 : kSplitWaves) : ((fused_swiglu || pl.wide) ? 2 : kSplitWaves);
+        const long trips_least = std::max(1, ((K / 32 + gkw - 1) / gkw + 7) / 8);  // trips per unit (at least)
+        const dim3 ggrid((unsigned)std::max(1L, std::min((long)kGroupMaxWgs, most_units * trips_least))), gblock(kSplitWaves * 64);
+        const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
+        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+#define LYRA_GROUP_RS(F, S, R, C)                                                                                     \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C>,        \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C>), ggrid, gblock, glds, st, p);                       \
+    } while (0)
+    // fewer units than workgroups whatever the group sizes: the variant that cuts units into K slices
+    // without SwiGLU, when the shapes allow 1.75 rounds of 256-column units: the variant that decides on them on the device
+    static const bool no_wide_dyn = getenv("LYRA_GEMM_NO_WIDE_IF_MANY") != nullptr;  // tuning override
+    const bool wide_dyn = !no_wide_dyn && !fused_swiglu && !pl.wide && N % 256 == 0 &&
+                          4 * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M)) * (N / 256) >= 7 * (long)kGroupMaxWgs;
+#define LYRA_GROUP_RSW(F, S, R)                                                                                       \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, false, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, false, true>), ggrid, gblock, glds, st, p);             \
+    } while (0)
+#define LYRA_GROUP_P(F, S, R, C, W)                                                                                   \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C, W, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
+        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
+        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C, W, true>), ggrid, gblock, glds, st, p);              \
+    } while (0)
+#define LYRA_GROUP_R(F, S, R)                                               \
+    do {                                                                    \
+        if (layout) {                                                       \
+            if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_P(F, S, R, true, false); \
+            else LYRA_GROUP_P(F, S, R, false, true);                        \
+        } else if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
+        else if (wide_dyn) LYRA_GROUP_RSW(F, S, R);                         \
+        else LYRA_GROUP_RS(F, S, R, false);                                 \
+    } while (0)
+#define LYRA_GROUP(F, S, DEPTH_)                                                          \
+    do {                                                                                  \
+        const int kw = gkw;                                                               \
+        const int per_wave = (K / 32 + kw - 1) / kw;                                      \
+        const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
+        if (K % (kw * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);                 \
+        else LYRA_GROUP_R(F, S, 1);                                                       \
+    } while (0)
+        if constexpr (WT != 0) {
+            if (step_scales) LYRA_GROUP(WT, true, 4);
+            else LYRA_GROUP(WT, false, 4);
+        } else {
+            LYRA_GROUP(0, false, 2);
+        }
+#undef LYRA_GROUP
+#undef LYRA_GROUP_R
+#undef LYRA_GROUP_P
+#undef LYRA_GROUP_RSW
+#undef LYRA_GROUP_RS
+        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+    }
+    if (pl.split_k) {
+        const int rc = launch_split_k_fmt<WT>(p, pl, st);
+        if (rc != LYRA_OK) return rc;
+        return launch_finish(p, st);
+    }
+    if (pl.one_pass) {
+        const dim3 sgrid(pl.spans, pl.row_par), sblock(kSmallWaves * 64);
+        const size_t slds = (size_t)kSmallWaves * 16 * 128 * sizeof(float);
+        const int per_wave = (K / 32 + kSmallWaves - 1) / kSmallWaves;  // steps of 32 rows each wavefront walks
+        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
+#define LYRA_SMALL(F, D, S, O) hipLaunchKernelGGL((decode_gemm_small_kernel<F, D, S, O>), sgrid, sblock, slds, st, p)
+        if constexpr (WT != 0) {
+            if (step_scales) {
+                if (per_wave <= 4) LYRA_SMALL(WT, 4, true, true);
+                else LYRA_SMALL(WT, 4, true, false);
+            } else {
+                if (per_wave <= 2) LYRA_SMALL(WT, 2, false, true);
+                else if (per_wave <= 4) LYRA_SMALL(WT, 4, false, true);
+                else if (per_wave <= 6) LYRA_SMALL(WT, 6, false, true);
+                else if (per_wave <= 8) LYRA_SMALL(WT, 8, false, true);
+                else LYRA_SMALL(WT, 6, false, false);
+            }
+        } else {
+            if (per_wave <= 2) LYRA_SMALL(0, 2, false, true);
+            else if (per_wave <= 4) LYRA_SMALL(0, 4, false, true);
+            else LYRA_SMALL(0, 4, false, false);
+        }
+#undef LYRA_SMALL
+        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+    }
+    dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
+    // a very wide single projection (the LM head): one workgroup per compute unit with as many wavefronts as its share of spans
+    static const bool no_even = getenv("LYRA_GEMM_NO_EVEN_SPANS") != nullptr;  // tuning override
+    const int per_cu = (pl.spans + kGroupMaxWgs - 1) / kGroupMaxWgs;
+    if (!no_even && G == 1 && pl.ksplit == 1 && pl.row_par == 1 && pl.spans >= 4 * kGroupMaxWgs && per_cu <= (pl.mt == 1 ? 12 : 8)) {
+        p.even_spans = 1;
+        grid = dim3(kGroupMaxWgs, 1, 1);
+        block = dim3(per_cu * 64);
+    }
+    const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t) +
+                       (tile_max ? (size_t)(block.x / 64) * 16 * pl.mt * kTileMaxPitch * sizeof(float) : 0);
+#define LYRA_LAUNCH_GEMM(F, T)                                                                                         \
+    do {                                                                                                               \
+        if (tile_max) {                                                                                                \
+            static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_kernel<F, T, true>,            \
+                                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                              \
+            hipLaunchKernelGGL((decode_gemm_kernel<F, T, true>), grid, block, lds, st, p);                             \
+        } else {                                                                                                       \
+            hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p);                                   \
+        }                                                                                                              \
+    } while (0)
+    if (pl.mt == 1) LYRA_LAUNCH_GEMM(WT, 1);
+    else if (pl.mt == 2) LYRA_LAUNCH_GEMM(WT, 2);
+    else LYRA_LAUNCH_GEMM(WT, 4);
+#undef LYRA_LAUNCH_GEMM
+    if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
+    if (pl.ksplit > 1) return launch_finish(p, st);
+    return LYRA_OK;
+}
+#if LYRA_GEMM_PART == 1
+template int launch_planned<0>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);
+template int launch_planned<1>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);
+#elif LYRA_GEMM_PART == 3
+template int launch_planned<2>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);
+#endif
+#endif  // LYRA_GEMM_HAS_LAUNCH
+}  // namespace lyra
+
+#if LYRA_GEMM_HAS_ENTRY
 
 namespace lyra {
+int launch_finish(const GemmParams& p, hipStream_t st) {
+    const int NO = p.swiglu ? p.N / 2 : p.N;
+    hipLaunchKernelGGL(decode_gemm_finish_kernel, dim3((unsigned)((NO / 4 + 255) / 256), (unsigned)std::min(p.M, 65535)), dim3(256), 0, st, p);
+    return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
+}
+
 // Bytes of float32 partials (behind the counters) that the launch of `pl` writes.
 static size_t gemm_partial_bytes(const GemmPlan& pl, int M, int N) {
     if (pl.grouped)  // one tile slot of 64 rows x 256 columns per workgroup
@@ -1824,18 +2007,18 @@ static size_t gemm_partial_bytes(const GemmPlan& pl, int M, int N) {
 
 extern "C" size_t lyra_gemm_packed_bytes(int G, int K, int N, int rhs_dtype, int layout) {
     if (G <= 0 || K <= 0 || N <= 0 || (layout != 1 && layout != 2)) return 0;
-    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return 0;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && !lyra::one_byte_format(rhs_dtype)) return 0;
     if (N % 8 || (layout == 2 && N % 16)) return 0;
-    return (size_t)G * lyra::packed_spans(N, layout) * K * 128 * (rhs_dtype == LYRA_DTYPE_E4M3FN ? 1 : 2);
+    return (size_t)G * lyra::packed_spans(N, layout) * K * 128 * (lyra::one_byte_format(rhs_dtype) ? 1 : 2);
 }
 
 extern "C" int lyra_gemm_pack(const void* rhs, void* packed, int G, int K, int N, int rhs_dtype, int layout, lyra_stream_t stream) {
     using namespace lyra;
     if (!rhs || !packed || G <= 0 || K <= 0 || N <= 0 || (layout != 1 && layout != 2)) return LYRA_E_BADARG;
-    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && !lyra::one_byte_format(rhs_dtype)) return LYRA_E_UNSUPPORTED;
     if (N % 8 || (layout == 2 && N % 16)) return LYRA_E_UNSUPPORTED;
     if (((uintptr_t)rhs | (uintptr_t)packed) % 16) return LYRA_E_BADARG;
-    PackParams p{(const uint8_t*)rhs, (uint8_t*)packed, G, K, N, rhs_dtype == LYRA_DTYPE_E4M3FN ? 1 : 2, layout == 2, packed_spans(N, layout)};
+    PackParams p{(const uint8_t*)rhs, (uint8_t*)packed, G, K, N, lyra::one_byte_format(rhs_dtype) ? 1 : 2, layout == 2, packed_spans(N, layout)};
     const size_t pieces = (size_t)G * p.pspans * K * 16;
     const unsigned blocks = (unsigned)std::min<size_t>((pieces + 255) / 256, 65536);
     hipLaunchKernelGGL(gemm_pack_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, p);
@@ -1911,9 +2094,9 @@ static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const vo
     if (bias_post && (G != 1 || fused_swiglu)) return LYRA_E_UNSUPPORTED;
     if (!lhs || !rhs || !group_sizes || !out) return LYRA_E_BADARG;
     if (M <= 0 || G <= 0 || K <= 0 || N <= 0) return LYRA_E_BADARG;
-    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && !lyra::one_byte_format(rhs_dtype)) return LYRA_E_UNSUPPORTED;
     if (out_dtype != LYRA_DTYPE_BF16 && out_dtype != LYRA_DTYPE_F32) return LYRA_E_UNSUPPORTED;
-    const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
+    const bool fp8 = one_byte_format(rhs_dtype);
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
     if (K % 32 || N % 8 || (fused_swiglu && N % 16) || G > 8191) return LYRA_E_UNSUPPORTED;  // (a lane holds 8 columns)
     if ((size_t)M * N * 4 >= (1ull << 31)) return LYRA_E_UNSUPPORTED;  // results are stored through 31-bit buffer offsets
@@ -1998,141 +2181,9 @@ static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const vo
     }
 
     hipStream_t st = (hipStream_t)stream;
-    if (pl.grouped) {
-        // one workgroup per compute unit (more would only queue behind the LDS tiles), fewer when there is less work
-        const long most_blocks = std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M));
-        // (packed: units of one span unless the list is long enough for units of two - the kernel's own rule, on the most
-        // row blocks the shapes allow)
-        const bool packed_wide = layout && 4 * most_blocks * ((p.pspans + 1) / 2) >= 7 * (long)kGroupMaxWgs;
-        const long most_units = (layout ? (long)p.pspans : (long)pl.spans) * most_blocks;
-        const int gkw = layout ? (packed_wide ? 2 : kSplitWaves) : ((fused_swiglu || pl.wide) ? 2 : kSplitWaves);
-        const long trips_least = std::max(1, ((K / 32 + gkw - 1) / gkw + 7) / 8);  // trips per unit (at least)
-        const dim3 ggrid((unsigned)std::max(1L, std::min((long)kGroupMaxWgs, most_units * trips_least))), gblock(kSplitWaves * 64);
-        const size_t glds = (size_t)kSplitWaves * 16 * kGroupTiles * kSplitPitch * sizeof(float);
-        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
-#define LYRA_GROUP_RS(F, S, R, C)                                                                                     \
-    do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C>,        \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
-        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C>), ggrid, gblock, glds, st, p);                       \
-    } while (0)
-    // fewer units than workgroups whatever the group sizes: the variant that cuts units into K slices
-    // without SwiGLU, when the shapes allow 1.75 rounds of 256-column units: the variant that decides on them on the device
-    static const bool no_wide_dyn = getenv("LYRA_GEMM_NO_WIDE_IF_MANY") != nullptr;  // tuning override
-    const bool wide_dyn = !no_wide_dyn && !fused_swiglu && !pl.wide && N % 256 == 0 &&
-                          4 * std::min((long)G + M / (16 * kGroupTiles), (long)std::max(1, M)) * (N / 256) >= 7 * (long)kGroupMaxWgs;
-#define LYRA_GROUP_RSW(F, S, R)                                                                                       \
-    do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, false, true>, \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
-        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, false, true>), ggrid, gblock, glds, st, p);             \
-    } while (0)
-#define LYRA_GROUP_P(F, S, R, C, W)                                                                                   \
-    do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_group_kernel<F, S, R, C, W, true>, \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)glds);    \
-        if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                                 \
-        hipLaunchKernelGGL((decode_gemm_group_kernel<F, S, R, C, W, true>), ggrid, gblock, glds, st, p);              \
-    } while (0)
-#define LYRA_GROUP_R(F, S, R)                                               \
-    do {                                                                    \
-        if (layout) {                                                       \
-            if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_P(F, S, R, true, false); \
-            else LYRA_GROUP_P(F, S, R, false, true);                        \
-        } else if (most_units < (long)kGroupMaxWgs && p.max_slices > 1) LYRA_GROUP_RS(F, S, R, true); \
-        else if (wide_dyn) LYRA_GROUP_RSW(F, S, R);                         \
-        else LYRA_GROUP_RS(F, S, R, false);                                 \
-    } while (0)
-#define LYRA_GROUP(F, S, DEPTH_)                                                          \
-    do {                                                                                  \
-        const int kw = gkw;                                                               \
-        const int per_wave = (K / 32 + kw - 1) / kw;                                      \
-        const int rounds = (per_wave + (DEPTH_) - 1) / (DEPTH_);                          \
-        if (K % (kw * 32) == 0 && rounds % 2 == 0) LYRA_GROUP_R(F, S, 2);                 \
-        else LYRA_GROUP_R(F, S, 1);                                                       \
-    } while (0)
-        if (step_scales) LYRA_GROUP(true, true, 4);
-        else if (fp8) LYRA_GROUP(true, false, 4);
-        else LYRA_GROUP(false, false, 2);
-#undef LYRA_GROUP
-#undef LYRA_GROUP_R
-#undef LYRA_GROUP_P
-#undef LYRA_GROUP_RSW
-#undef LYRA_GROUP_RS
-        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
-    }
-    if (pl.split_k) {
-        const int rc = launch_split_k(p, pl, fp8, st);
-        if (rc != LYRA_OK) return rc;
-        const int NO = fused_swiglu ? N / 2 : N;
-        hipLaunchKernelGGL(decode_gemm_finish_kernel, dim3((unsigned)((NO / 4 + 255) / 256), (unsigned)std::min(M, 65535)), dim3(256), 0, st, p);
-        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
-    }
-    if (pl.one_pass) {
-        const dim3 sgrid(pl.spans, pl.row_par), sblock(kSmallWaves * 64);
-        const size_t slds = (size_t)kSmallWaves * 16 * 128 * sizeof(float);
-        const int per_wave = (K / 32 + kSmallWaves - 1) / kSmallWaves;  // steps of 32 rows each wavefront walks
-        const bool step_scales = fp8 && p.scale_mode == 1 && p.bk < p.K;
-#define LYRA_SMALL(F, D, S, O) hipLaunchKernelGGL((decode_gemm_small_kernel<F, D, S, O>), sgrid, sblock, slds, st, p)
-        if (step_scales) {
-            if (per_wave <= 4) LYRA_SMALL(true, 4, true, true);
-            else LYRA_SMALL(true, 4, true, false);
-        } else if (fp8) {
-            if (per_wave <= 2) LYRA_SMALL(true, 2, false, true);
-            else if (per_wave <= 4) LYRA_SMALL(true, 4, false, true);
-            else if (per_wave <= 6) LYRA_SMALL(true, 6, false, true);
-            else if (per_wave <= 8) LYRA_SMALL(true, 8, false, true);
-            else LYRA_SMALL(true, 6, false, false);
-        } else {
-            if (per_wave <= 2) LYRA_SMALL(false, 2, false, true);
-            else if (per_wave <= 4) LYRA_SMALL(false, 4, false, true);
-            else LYRA_SMALL(false, 4, false, false);
-        }
-#undef LYRA_SMALL
-        return hipGetLastError() == hipSuccess ? LYRA_OK : LYRA_E_LAUNCH;
-    }
-    dim3 grid((pl.spans + kGemmWaves - 1) / kGemmWaves, pl.ksplit, G * pl.row_par), block(kGemmWaves * 64);
-    // a very wide single projection (the LM head): one workgroup per compute unit with as many wavefronts as its share of spans
-    static const bool no_even = getenv("LYRA_GEMM_NO_EVEN_SPANS") != nullptr;  // tuning override
-    const int per_cu = (pl.spans + kGroupMaxWgs - 1) / kGroupMaxWgs;
-    if (!no_even && G == 1 && pl.ksplit == 1 && pl.row_par == 1 && pl.spans >= 4 * kGroupMaxWgs && per_cu <= (pl.mt == 1 ? 12 : 8)) {
-        p.even_spans = 1;
-        grid = dim3(kGroupMaxWgs, 1, 1);
-        block = dim3(per_cu * 64);
-    }
-    const size_t lds = (size_t)16 * pl.mt * (512 + 8) * sizeof(uint16_t) +
-                       (tile_max ? (size_t)(block.x / 64) * 16 * pl.mt * kTileMaxPitch * sizeof(float) : 0);
-#define LYRA_LAUNCH_GEMM(F, T)                                                                                         \
-    do {                                                                                                               \
-        if (tile_max) {                                                                                                \
-            static const hipError_t attr = hipFuncSetAttribute((const void*)decode_gemm_kernel<F, T, true>,            \
-                                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-            if (attr != hipSuccess) return LYRA_E_LAUNCH;                                                              \
-            hipLaunchKernelGGL((decode_gemm_kernel<F, T, true>), grid, block, lds, st, p);                             \
-        } else {                                                                                                       \
-            hipLaunchKernelGGL((decode_gemm_kernel<F, T>), grid, block, lds, st, p);                                   \
-        }                                                                                                              \
-    } while (0)
-    if (fp8) {
-        if (pl.mt == 1) LYRA_LAUNCH_GEMM(true, 1);
-        else if (pl.mt == 2) LYRA_LAUNCH_GEMM(true, 2);
-        else LYRA_LAUNCH_GEMM(true, 4);
-    } else {
-        if (pl.mt == 1) LYRA_LAUNCH_GEMM(false, 1);
-        else if (pl.mt == 2) LYRA_LAUNCH_GEMM(false, 2);
-        else LYRA_LAUNCH_GEMM(false, 4);
-    }
-#undef LYRA_LAUNCH_GEMM
-    if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
-    if (pl.ksplit > 1) {
-        const int NO = fused_swiglu ? N / 2 : N;
-        const dim3 fgrid((unsigned)((NO / 4 + 255) / 256), (unsigned)std::min(M, 65535)), fblock(256);
-        hipLaunchKernelGGL(decode_gemm_finish_kernel, fgrid, fblock, 0, st, p);
-        if (hipGetLastError() != hipSuccess) return LYRA_E_LAUNCH;
-    }
-    return LYRA_OK;
+    if (rhs_dtype == LYRA_DTYPE_E5M2) return launch_planned<2>(p, pl, layout, fused_swiglu, tile_max, st);
+    if (fp8) return launch_planned<1>(p, pl, layout, fused_swiglu, tile_max, st);
+    return launch_planned<0>(p, pl, layout, fused_swiglu, tile_max, st);
 }
 }  // namespace lyra
 
@@ -2153,8 +2204,8 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     if (rhs_dtype & LYRA_OUT_TILED16) return LYRA_E_UNSUPPORTED;  // (the slices are float32, row-major)
     rhs_dtype &= ~(LYRA_RHS_SPAN_MAJOR | LYRA_LHS_TILED16);
     if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
-    if (rhs_dtype != LYRA_DTYPE_BF16 && rhs_dtype != LYRA_DTYPE_E4M3FN) return LYRA_E_UNSUPPORTED;
-    const bool fp8 = rhs_dtype == LYRA_DTYPE_E4M3FN;
+    if (rhs_dtype != LYRA_DTYPE_BF16 && !lyra::one_byte_format(rhs_dtype)) return LYRA_E_UNSUPPORTED;
+    const bool fp8 = one_byte_format(rhs_dtype);
     if (fp8 != (rhs_scale != nullptr)) return LYRA_E_BADARG;
     if (K % 32 || N % 8) return LYRA_E_UNSUPPORTED;
     GemmParams p = {};
@@ -2186,6 +2237,7 @@ extern "C" int lyra_decode_gemm_partials(const void* lhs, const void* rhs, const
     p.packed = layout;
     p.pspans = layout ? packed_spans(N, layout) : 0;
     p.lhs_tiled = lhs_tiled;
-    return launch_split_k(p, pl, fp8, (hipStream_t)stream);
+    if (rhs_dtype == LYRA_DTYPE_E5M2) return launch_split_k_fmt<2>(p, pl, (hipStream_t)stream);
+    return fp8 ? launch_split_k_fmt<1>(p, pl, (hipStream_t)stream) : launch_split_k_fmt<0>(p, pl, (hipStream_t)stream);
 }
-#endif  // !LYRA_GEMM_SPLITK_PART
+#endif  // LYRA_GEMM_HAS_ENTRY

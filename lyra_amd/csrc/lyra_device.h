@@ -60,13 +60,34 @@ __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// 8 consecutive e4m3fn codes (two dwords) -> bf16x8 in the same order
+// The same for the two 1-byte formats the kernels read, picked at compile time.  FMT 1: e4m3fn; FMT 2: e5m2 (OCP FP8 E5M2:
+// 5 exponent bits, 2 mantissa bits, max 57344; its infinities and NaNs never occur in quantised data, which is clipped).
+template <int FMT>
+__device__ __forceinline__ uint32_t codes2_to_bf16x2(uint32_t w, bool hi) {
+    static_assert(FMT == 1 || FMT == 2, "1-byte formats: 1 = e4m3fn, 2 = e5m2");
+    if constexpr (FMT == 2) {
+        bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, true)
+                      : __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, false);
+        return __builtin_bit_cast(uint32_t, r);
+    } else {
+        return fp8x2_to_bf16x2(w, hi);
+    }
+}
+template <int FMT>
+__device__ __forceinline__ f32x2 codes2_to_f32(uint32_t w, bool hi) {
+    static_assert(FMT == 1 || FMT == 2, "1-byte formats: 1 = e4m3fn, 2 = e5m2");
+    if constexpr (FMT == 2) return hi ? __builtin_amdgcn_cvt_pk_f32_bf8(w, true) : __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+    else return fp8x2_to_f32(w, hi);
+}
+
+// 8 consecutive 1-byte codes (two dwords) -> bf16x8 in the same order
+template <int FMT = 1>
 __device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
     Pack8 p;
-    p.u[0] = fp8x2_to_bf16x2(w0, false);
-    p.u[1] = fp8x2_to_bf16x2(w0, true);
-    p.u[2] = fp8x2_to_bf16x2(w1, false);
-    p.u[3] = fp8x2_to_bf16x2(w1, true);
+    p.u[0] = codes2_to_bf16x2<FMT>(w0, false);
+    p.u[1] = codes2_to_bf16x2<FMT>(w0, true);
+    p.u[2] = codes2_to_bf16x2<FMT>(w1, false);
+    p.u[3] = codes2_to_bf16x2<FMT>(w1, true);
     return p.v;
 }
 
@@ -85,6 +106,16 @@ __device__ __forceinline__ uint8_t f32_to_e4m3fn(float v) {
     const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false);
     return (uint8_t)(packed & 0xFF);
 }
+
+// float32 -> e5m2 code, round to nearest even; |v| <= 57344 by construction
+__device__ __forceinline__ uint8_t f32_to_e5m2(float v) {
+    const int packed = __builtin_amdgcn_cvt_pk_bf8_f32(v, 0.f, 0, false);
+    return (uint8_t)(packed & 0xFF);
+}
+
+// Largest finite value of a 1-byte format (jnp.finfo(dtype).max in lyra/nn/quant.py:68) and the quantiser for it.
+__device__ __forceinline__ float fp8_format_max(bool e5m2) { return e5m2 ? 57344.f : 448.f; }
+__device__ __forceinline__ uint8_t f32_to_fp8_code(float v, bool e5m2) { return e5m2 ? f32_to_e5m2(v) : f32_to_e4m3fn(v); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -54,7 +54,7 @@ def select_decode_attention_config(
         return None
     if batch > _MAX_GRID_YZ or kv_heads > _MAX_GRID_YZ:  # batch rows and kv heads are grid dimensions of the launch
         return None
-    if cache_dtype is not None and cache_dtype != torch.float8_e4m3fn:
+    if cache_dtype is not None and cache_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
         return None
     if out_dtype not in (torch.bfloat16, torch.float32):
         return None
@@ -111,7 +111,7 @@ def _decode_attention(q, k, v, sinks, sm_scale, sliding_window, position, config
         k_val, v_val = k.qval, v.qval
         k_scale = k.scale.to(torch.float32).reshape(B, K, S).contiguous()
         v_scale = v.scale.to(torch.float32).reshape(B, K, S).contiguous()
-        kv_dtype = _lib.DTYPE_E4M3FN
+        kv_dtype = _lib.fp8_code(k_val.dtype)
     else:
         if isinstance(k, QArray) or isinstance(v, QArray):
             raise ValueError("dense decode attention config received QArray k/v")
@@ -237,7 +237,7 @@ def decode_attention(
     xsa_alpha: torch.Tensor | None = None,
     row_order: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """q [B,N,1,H]; k, v [B,K,S,H] tensors or QArray (e4m3fn, block (1,H)); sinks [N]; returns [B,N,1,H].
+    """q [B,N,1,H]; k, v [B,K,S,H] tensors or QArray (e4m3fn or e5m2 codes, block (1,H)); sinks [N]; returns [B,N,1,H].
 
     ``row_order`` (``rank_rows(position)``; ragged batches only): lets the kernel deal the rows out by length instead of
     ranking them in every launch.  It changes which workgroup computes which row, never a result.

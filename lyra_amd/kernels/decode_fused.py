@@ -117,7 +117,7 @@ def pack_weights(rhs, glu: bool = False) -> SpanMajor:
     assert rv.is_contiguous() and rv.ndim == 3 and (fp8 or rv.dtype == torch.bfloat16)
     G, K, N = rv.shape
     layout = 2 if glu else 1
-    dt = _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16
+    dt = _lib.fp8_code(rv.dtype) if fp8 else _lib.DTYPE_BF16
     nbytes = _L.lyra_gemm_packed_bytes(G, K, N, dt, layout)
     if nbytes == 0:
         raise ValueError(f"no span-major layout {layout} for weights {tuple(rv.shape)} {rv.dtype}")
@@ -161,11 +161,11 @@ def _rhs_args(rhs):
         fp8 = rhs.scale is not None
         flag = _lib.RHS_SPAN_MAJOR if rhs.layout == 1 else _lib.RHS_SPAN_MAJOR_GLU
         bk, bn = rhs.block if fp8 else (0, 0)
-        return rhs.data, rhs.scale, bk, bn, (_lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16) | flag, rhs.shape
+        return rhs.data, rhs.scale, bk, bn, (_lib.fp8_code(rhs.dtype) if fp8 else _lib.DTYPE_BF16) | flag, rhs.shape
     if isinstance(rhs, QArray):
         bk, bn = rhs.block
         assert rhs.qval.is_contiguous()
-        return rhs.qval, _f32(rhs.scale), bk, bn, _lib.DTYPE_E4M3FN, tuple(rhs.shape)
+        return rhs.qval, _f32(rhs.scale), bk, bn, _lib.fp8_code(rhs.qval.dtype), tuple(rhs.shape)
     assert rhs.dtype == torch.bfloat16 and rhs.is_contiguous()
     return rhs, None, 0, 0, _lib.DTYPE_BF16, tuple(rhs.shape)
 
@@ -314,7 +314,7 @@ def qkv_post(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, pos: t
     rc = _L.lyra_qkv_post_sum(None if unsummed else qkv.data_ptr(), part.data_ptr() if unsummed else None, splits if unsummed else 0,
                               _ptr(qnorm), _ptr(knorm), _f32(cos_t).data_ptr(), _f32(sin_t).data_ptr(), pos.data_ptr(),
                               0 if pos.numel() == 1 else 1, q.data_ptr(), kq.data_ptr(), vq.data_ptr(), _ptr(ks), _ptr(vs),
-                              _ptr(vn), B, N, K, S, H, cos_t.shape[0], _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16, float(eps),
+                              _ptr(vn), B, N, K, S, H, cos_t.shape[0], _lib.fp8_code(kq.dtype) if fp8 else _lib.DTYPE_BF16, float(eps),
                               _stream(dev))
     _lib.check(rc, "lyra_qkv_post_sum")
     return (q, vn) if unit_v else q
@@ -366,7 +366,7 @@ def attention_qkv(qkv, qnorm, knorm, cos_t: torch.Tensor, sin_t: torch.Tensor, p
                                       _f32(sin_t).data_ptr(), cos_t.shape[0], float(eps), kq.data_ptr(), vq.data_ptr(), _ptr(ks),
                                       _ptr(vs), sinks.data_ptr(), pos.data_ptr(), 0 if pos.numel() == 1 else 1, _ptr(gate),
                                       out.data_ptr(), ws.data_ptr(), ws.numel(), B, N, K, S, H, float(sm_scale),
-                                      int(sliding_window), _lib.DTYPE_E4M3FN if fp8 else _lib.DTYPE_BF16,
+                                      int(sliding_window), _lib.fp8_code(kq.dtype) if fp8 else _lib.DTYPE_BF16,
                                       _lib.DTYPE_F32 if out_dtype == torch.float32 else _lib.DTYPE_BF16, stream)
     if rc == _lib.E_UNSUPPORTED:
         return None

@@ -45,7 +45,7 @@ def select_decode_gemm_config(m: int, groups: int, k: int, n: int, quant_dtype=N
     if k % 32 or n % 8 or (fused_swiglu and n % 16):  # (whole 128-column spans get the streaming kernels, other widths the general one)
         return None
     if quant_dtype is not None:
-        if quant_dtype != torch.float8_e4m3fn:
+        if quant_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
             return None
         if block is not None and not _scale_layout_supported(k, n, tuple(block)):
             return None
@@ -90,7 +90,7 @@ def _decode_gemm(lhs, rhs, group_sizes, config: DecodeGEMMConfig, *, bias, fused
             raise ValueError(f"FP8 decode RHS scale must be {expected}, got {tuple(rhs.scale.shape)}")
         rhs_val = rhs.qval.contiguous()
         rhs_scale = rhs.scale.to(torch.float32).contiguous()
-        rhs_dtype = _lib.DTYPE_E4M3FN
+        rhs_dtype = _lib.fp8_code(rhs.qval.dtype)
     else:
         if isinstance(rhs, QArray):
             raise ValueError("dense decode GEMM config received a QArray RHS")

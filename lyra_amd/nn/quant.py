@@ -161,7 +161,7 @@ def dot(lhs: torch.Tensor, rhs, *, dimension_numbers=None, preferred_element_typ
     flat = _flat_weight(rhs) if inner and rhs.ndim >= 2 else None
     fp8 = isinstance(rhs, QArray)
     kernel_ok = (flat is not None and lhs.is_cuda and lhs.dtype == torch.bfloat16 and out_dtype in (torch.bfloat16, torch.float32)
-                 and (rhs.dtype == torch.float8_e4m3fn if fp8 else rhs.dtype == torch.bfloat16))
+                 and (rhs.dtype in FP8_DTYPES if fp8 else rhs.dtype == torch.bfloat16))
     if not kernel_ok:
         if implementation in ("pallas", "hip"):
             raise ValueError(f"quant.dot: no HIP kernel for lhs {tuple(lhs.shape)} {lhs.dtype} . rhs {tuple(rhs.shape)} {rhs.dtype} "

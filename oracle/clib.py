@@ -24,6 +24,14 @@ def load() -> ctypes.CDLL:
     lib.lyra_oracle_fp8_e4m3fn_to_f32.argtypes = [c.c_uint8]
     lib.lyra_oracle_f32_to_fp8_e4m3fn.restype = c.c_uint8
     lib.lyra_oracle_f32_to_fp8_e4m3fn.argtypes = [c.c_float]
+    lib.lyra_oracle_fp8_e5m2_to_f32.restype = c.c_float
+    lib.lyra_oracle_fp8_e5m2_to_f32.argtypes = [c.c_uint8]
+    lib.lyra_oracle_f32_to_fp8_e5m2.restype = c.c_uint8
+    lib.lyra_oracle_f32_to_fp8_e5m2.argtypes = [c.c_float]
+    lib.lyra_oracle_quantize_rows_fmt.restype = None
+    lib.lyra_oracle_quantize_rows_fmt.argtypes = [c.c_void_p, c.c_int64, c.c_int, c.c_void_p, c.c_void_p, c.c_int]
+    lib.lyra_oracle_quantize_blocks_fmt.restype = c.c_int
+    lib.lyra_oracle_quantize_blocks_fmt.argtypes = [c.c_void_p] + [c.c_int] * 5 + [c.c_void_p] * 2 + [c.c_int]
     lib.lyra_oracle_f32_to_bf16.restype = c.c_uint16
     lib.lyra_oracle_f32_to_bf16.argtypes = [c.c_float]
     lib.lyra_oracle_quantize_rows.restype = None
@@ -52,32 +60,34 @@ def _p(a):
     return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
 
 
-def quantize_rows(x: np.ndarray):
-    """Block (1,H) quantiser (KV cache); bit-identical to lyra_oracle.quantize(x, (1, H))."""
+def quantize_rows(x: np.ndarray, fp8_format: int = 1):
+    """Block (1,H) quantiser (KV cache); bit-identical to lyra_oracle.quantize(x, (1, H)).  fp8_format 1: e4m3fn, 2: e5m2."""
     lib = load()
     H = x.shape[-1]
     flat = np.ascontiguousarray(x.reshape(-1, H), dtype=np.float32)
     q = np.empty(flat.shape, dtype=np.uint8)
     s = np.empty(flat.shape[0], dtype=np.float32)
-    lib.lyra_oracle_quantize_rows(_p(flat), flat.shape[0], H, _p(q), _p(s))
+    lib.lyra_oracle_quantize_rows_fmt(_p(flat), flat.shape[0], H, _p(q), _p(s), int(fp8_format))
     return q.reshape(x.shape), s.reshape(*x.shape[:-1], 1)
 
 
-def quantize_blocks(w: np.ndarray, block):
-    """Block (bk,bn) quantiser of [G,K,N] weights; bit-identical to lyra_oracle.quantize(w, block)."""
+def quantize_blocks(w: np.ndarray, block, fp8_format: int = 1):
+    """Block (bk,bn) quantiser of [G,K,N] weights; bit-identical to lyra_oracle.quantize(w, block).  fp8_format 1: e4m3fn, 2: e5m2."""
     lib = load()
     G, K, N = w.shape
     bk, bn = block
     w = np.ascontiguousarray(w, dtype=np.float32)
     q = np.empty(w.shape, dtype=np.uint8)
     s = np.empty((G, K // bk, N // bn), dtype=np.float32)
-    if lib.lyra_oracle_quantize_blocks(_p(w), G, K, N, bk, bn, _p(q), _p(s)):
+    if lib.lyra_oracle_quantize_blocks_fmt(_p(w), G, K, N, bk, bn, _p(q), _p(s), int(fp8_format)):
         raise ValueError(f"block {block} does not divide {(K, N)}")
     return q, s
 
 
-def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_scale, sliding_window, *, ref_rounding=False):
-    """q_bits uint16 [B,N,1,H]; k,v uint8 (fp8) or uint16 (bf16) [B,K,S,H]; returns f32 [B,N,1,H]."""
+def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_scale, sliding_window, *, ref_rounding=False,
+                     fp8_format: int = 1):
+    """q_bits uint16 [B,N,1,H]; k,v uint8 (fp8 codes of ``fp8_format``: 1 e4m3fn, 2 e5m2) or uint16 (bf16) [B,K,S,H]; returns f32
+    [B,N,1,H]."""
     lib = load()
     B, N, _, H = q_bits.shape
     _, K, S, _ = k.shape
@@ -92,7 +102,7 @@ def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_s
     out = np.empty((B, N, 1, H), dtype=np.float32)
     rc = lib.lyra_oracle_decode_attention(
         _p(q_bits), _p(k), _p(v), _p(ks), _p(vs), _p(sinks), _p(pos), _p(g), _p(out),
-        B, N, K, S, H, float(sm_scale), int(sliding_window), int(fp8), int(ref_rounding),
+        B, N, K, S, H, float(sm_scale), int(sliding_window), int(fp8_format) if fp8 else 0, int(ref_rounding),
     )
     if rc:
         raise RuntimeError(f"lyra_oracle_decode_attention failed: {rc}")
@@ -100,8 +110,9 @@ def decode_attention(q_bits, k, v, k_scale, v_scale, sinks, position, gate, sm_s
 
 
 def decode_gemm(lhs_bits, rhs, rhs_scale, block, group_sizes, bias, *, fused_swiglu=False, beta=1.702, limit=7.0,
-                ref_rounding=False, scratch=None, dequant_bf16=False):
-    """lhs_bits uint16 [M,K]; rhs uint8 (fp8, with rhs_scale/block) or uint16 (bf16) [G,K,N]; returns f32.
+                ref_rounding=False, scratch=None, dequant_bf16=False, fp8_format: int = 1):
+    """lhs_bits uint16 [M,K]; rhs uint8 (fp8 codes of ``fp8_format``: 1 e4m3fn, 2 e5m2; with rhs_scale/block) or uint16 (bf16)
+    [G,K,N]; returns f32.
     ref_rounding: dequantised weights and outputs rounded to bf16; dequant_bf16 (without it): only the dequantised weights."""
     lib = load()
     M, K = lhs_bits.shape
@@ -117,7 +128,7 @@ def decode_gemm(lhs_bits, rhs, rhs_scale, block, group_sizes, bias, *, fused_swi
         scratch = np.empty((G, K, N), dtype=np.float32)
     rc = lib.lyra_oracle_decode_gemm(
         _p(lhs_bits), _p(rhs), _p(sc), bk, bn, _p(gs), _p(b), _p(out), _p(scratch),
-        M, G, K, N, int(fp8), int(fused_swiglu), float(beta), float(limit), 1 if ref_rounding else (2 if dequant_bf16 else 0),
+        M, G, K, N, int(fp8_format) if fp8 else 0, int(fused_swiglu), float(beta), float(limit), 1 if ref_rounding else (2 if dequant_bf16 else 0),
     )
     if rc:
         raise RuntimeError(f"lyra_oracle_decode_gemm failed: {rc}")

@@ -26,8 +26,12 @@
 #define LYRA_DECODE_BLOCK 128 /* decode_attention.py:29 */
 
 /* ---- number formats ------------------------------------------------------------- */
-static float fp8_table[256];
+/* Two 1-byte formats (lyra/nn/quant.py:10): index 1 = e4m3fn (s.eeee.mmm, bias 7, no infinities, S.1111.111 = NaN, max
+ * 448), index 2 = e5m2 (s.eeeee.mm, bias 15, IEEE-like: exponent 31 = inf / NaN, max 57344).  Wherever this file takes a
+ * flag "fp8" for an array, 0 means bf16 and 1 / 2 name the format of its codes. */
+static float fp8_tables[3][256];
 static int fp8_table_ready = 0;
+#define fp8_table fp8_tables[1]
 
 static void fp8_init(void) {
     if (fp8_table_ready) return;
@@ -38,9 +42,44 @@ static void fp8_init(void) {
         if (e == 0xF && m == 7) v = NAN;
         else if (e == 0) v = sign * ldexpf((float)m / 8.0f, -6);
         else v = sign * ldexpf(1.0f + (float)m / 8.0f, e - 7);
-        fp8_table[code] = v;
+        fp8_tables[1][code] = v;
+        int e5 = (code >> 2) & 0x1F, m5 = code & 3;
+        if (e5 == 0x1F) v = m5 ? NAN : sign * INFINITY;
+        else if (e5 == 0) v = sign * ldexpf((float)m5 / 4.0f, -14);
+        else v = sign * ldexpf(1.0f + (float)m5 / 4.0f, e5 - 15);
+        fp8_tables[2][code] = v;
     }
     fp8_table_ready = 1;
+}
+
+static inline float fp8_format_max(int fmt) { return fmt == 2 ? 57344.0f : 448.0f; }
+
+float lyra_oracle_fp8_e5m2_to_f32(uint8_t code) {
+    fp8_init();
+    return fp8_tables[2][code];
+}
+
+/* float32 -> e5m2, round to nearest even; magnitudes that round above 57344 -> inf (0x7c), NaN -> 0x7f. */
+uint8_t lyra_oracle_f32_to_fp8_e5m2(float x) {
+    uint8_t sign = signbit(x) ? 0x80 : 0;
+    if (isnan(x)) return sign | 0x7F;
+    double a = fabs((double)x);
+    if (a == 0.0) return sign;
+    if (isinf(a)) return sign | 0x7C;
+    int e;
+    frexp(a, &e);
+    e -= 1;
+    if (e < -14) e = -14;
+    if (e > 15) e = 15;
+    double ulp = ldexp(1.0, e - 2);
+    double val = nearbyint(a / ulp) * ulp; /* ties to even */
+    if (val > 57344.0) return sign | 0x7C;
+    if (val < ldexp(1.0, -14)) return sign | (uint8_t)nearbyint(val / ldexp(1.0, -16));
+    int e2;
+    frexp(val, &e2);
+    e2 -= 1;
+    int mant = (int)nearbyint((val / ldexp(1.0, e2) - 1.0) * 4.0);
+    return sign | (uint8_t)(((e2 + 15) << 2) | mant);
 }
 
 float lyra_oracle_fp8_e4m3fn_to_f32(uint8_t code) {
@@ -71,6 +110,9 @@ uint8_t lyra_oracle_f32_to_fp8_e4m3fn(float x) {
     return sign | (uint8_t)(((e2 + 7) << 3) | mant);
 }
 
+uint8_t lyra_oracle_f32_to_fp8_e4m3fn(float x);
+static inline uint8_t f32_to_fp8(float x, int fmt) { return fmt == 2 ? lyra_oracle_f32_to_fp8_e5m2(x) : lyra_oracle_f32_to_fp8_e4m3fn(x); }
+
 static inline float bf16_to_f32(uint16_t b) {
     uint32_t u = (uint32_t)b << 16;
     float f;
@@ -92,28 +134,34 @@ static inline float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 uint16_t lyra_oracle_f32_to_bf16(float f) { return f32_to_bf16(f); }
 
 /* ---- quantise one block-row (KV cache block (1,H)): quant.py:68-72 ------------------ */
-void lyra_oracle_quantize_rows(const float* x, int64_t rows, int H, uint8_t* qval, float* scale) {
+void lyra_oracle_quantize_rows_fmt(const float* x, int64_t rows, int H, uint8_t* qval, float* scale, int fmt) {
     fp8_init();
+    const float fmax = fp8_format_max(fmt);
 #pragma omp parallel for schedule(static)
     for (int64_t r = 0; r < rows; ++r) {
         const float* xr = x + r * H;
         float amax = 0.0f;
         for (int h = 0; h < H; ++h) amax = fmaxf(amax, fabsf(xr[h]));
-        float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+        float s = amax > 0.0f ? amax / fmax : 1.0f;
         float inv = 1.0f / s;
         scale[r] = s;
         for (int h = 0; h < H; ++h) {
             float t = xr[h] * inv;
-            t = fminf(fmaxf(t, -448.0f), 448.0f);
-            qval[r * H + h] = lyra_oracle_f32_to_fp8_e4m3fn(t);
+            t = fminf(fmaxf(t, -fmax), fmax);
+            qval[r * H + h] = f32_to_fp8(t, fmt);
         }
     }
 }
 
+void lyra_oracle_quantize_rows(const float* x, int64_t rows, int H, uint8_t* qval, float* scale) {
+    lyra_oracle_quantize_rows_fmt(x, rows, H, qval, scale, 1);
+}
+
 /* ---- quantise [G,K,N] weights with block (bk,bn): quant.py:48-75; scale is [G,K/bk,N/bn] ------- */
-int lyra_oracle_quantize_blocks(const float* x, int G, int K, int N, int bk, int bn, uint8_t* qval, float* scale) {
+int lyra_oracle_quantize_blocks_fmt(const float* x, int G, int K, int N, int bk, int bn, uint8_t* qval, float* scale, int fmt) {
     if (G <= 0 || K <= 0 || N <= 0 || bk <= 0 || bn <= 0 || K % bk || N % bn) return -1;
     fp8_init();
+    const float fmax = fp8_format_max(fmt);
     const int KB = K / bk, NB = N / bn;
 #pragma omp parallel for collapse(3) schedule(static)
     for (int g = 0; g < G; ++g) {
@@ -123,19 +171,23 @@ int lyra_oracle_quantize_blocks(const float* x, int G, int K, int N, int bk, int
                 float amax = 0.0f;
                 for (int i = 0; i < bk; ++i)
                     for (int j = 0; j < bn; ++j) amax = fmaxf(amax, fabsf(x[base + (size_t)i * N + j]));
-                const float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+                const float s = amax > 0.0f ? amax / fmax : 1.0f;
                 const float inv = 1.0f / s;
                 scale[((size_t)g * KB + kb) * NB + nb] = s;
                 for (int i = 0; i < bk; ++i)
                     for (int j = 0; j < bn; ++j) {
                         float t = x[base + (size_t)i * N + j] * inv;
-                        t = fminf(fmaxf(t, -448.0f), 448.0f);
-                        qval[base + (size_t)i * N + j] = lyra_oracle_f32_to_fp8_e4m3fn(t);
+                        t = fminf(fmaxf(t, -fmax), fmax);
+                        qval[base + (size_t)i * N + j] = f32_to_fp8(t, fmt);
                     }
             }
         }
     }
     return 0;
+}
+
+int lyra_oracle_quantize_blocks(const float* x, int G, int K, int N, int bk, int bn, uint8_t* qval, float* scale) {
+    return lyra_oracle_quantize_blocks_fmt(x, G, K, N, bk, bn, qval, scale, 1);
 }
 
 /* ---- window arithmetic: decode_attention.py:63-69, :277-280 -------------------------- */
@@ -200,8 +252,8 @@ int lyra_oracle_decode_attention(const uint16_t* q, const void* k, const void* v
                 for (int h = 0; h < H; ++h) {
                     float kv_, vv_;
                     if (kv_fp8) {
-                        kv_ = fp8_table[((const uint8_t*)k)[row * H + h]] * k_scale[row];
-                        vv_ = fp8_table[((const uint8_t*)v)[row * H + h]] * v_scale[row];
+                        kv_ = fp8_tables[kv_fp8 == 2 ? 2 : 1][((const uint8_t*)k)[row * H + h]] * k_scale[row];
+                        vv_ = fp8_tables[kv_fp8 == 2 ? 2 : 1][((const uint8_t*)v)[row * H + h]] * v_scale[row];
                         if (ref_rounding) { kv_ = bf16_round(kv_); vv_ = bf16_round(vv_); }
                     } else {
                         kv_ = bf16_to_f32(((const uint16_t*)k)[row * H + h]);
@@ -288,7 +340,7 @@ int lyra_oracle_decode_gemm(const uint16_t* lhs, const void* rhs, const float* r
             for (int n = 0; n < N; ++n) {
                 float w;
                 if (rhs_fp8) {
-                    w = fp8_table[((const uint8_t*)rhs)[row + n]] * rhs_scale[((size_t)g * KB + kk / bk) * NB + n / bn];
+                    w = fp8_tables[rhs_fp8 == 2 ? 2 : 1][((const uint8_t*)rhs)[row + n]] * rhs_scale[((size_t)g * KB + kk / bk) * NB + n / bn];
                     if (ref_rounding) w = bf16_round(w);
                 } else {
                     w = bf16_to_f32(((const uint16_t*)rhs)[row + n]);

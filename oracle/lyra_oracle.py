@@ -16,8 +16,8 @@ path and cites the reference file:line it follows.  Two arithmetic modes:
 Pinning status (what fixes each function independently of this file's own
 formulas; the checks live in tests/test_oracle_*.py):
 
-* fp8 e4m3fn decode/encode ......... all 256 codes and all rounding midpoints
-                                     against ``torch.float8_e4m3fn``
+* fp8 e4m3fn / e5m2 decode/encode .. all 256 codes and all rounding midpoints
+                                     against ``torch.float8_e4m3fn`` / ``torch.float8_e5m2``
 * bf16 rounding .................... against ``torch.bfloat16`` casts
 * quantize / dequantize ............ closed forms of lyra/nn/quant.py:68-72
 * sink softmax attention ........... ``torch`` SDPA / softmax with one extra
@@ -78,6 +78,71 @@ def fp8_e4m3fn_decode_table() -> np.ndarray:
 
 
 _FP8_TABLE = fp8_e4m3fn_decode_table()
+
+FP8_E5M2_MAX = 57344.0  # jnp.finfo(float8_e5m2).max: the other format of FP8_DTYPES, lyra/nn/quant.py:10
+
+
+def fp8_e5m2_decode_table() -> np.ndarray:
+    """float32 value of each of the 256 OCP FP8 E5M2 codes.
+
+    Layout s.eeeee.mm, bias 15, IEEE-like: exponent field 0 is subnormal (m/4 * 2^-14), exponent field 31 is
+    infinity (m = 0) or NaN; max finite 57344 = 1.75 * 2^15.  The code is the upper byte of the float16 with the same value.
+    """
+    table = np.empty(256, dtype=np.float32)
+    for code in range(256):
+        sign = -1.0 if code & 0x80 else 1.0
+        e = (code >> 2) & 0x1F
+        m = code & 0x3
+        if e == 0x1F:
+            val = float("nan") if m else sign * float("inf")
+        elif e == 0:
+            val = sign * (m / 4.0) * 2.0**-14
+        else:
+            val = sign * (1.0 + m / 4.0) * 2.0 ** (e - 15)
+        table[code] = val
+    return table
+
+
+_FP8_E5M2_TABLE = fp8_e5m2_decode_table()
+FP8_FORMATS = {1: "e4m3fn", 2: "e5m2"}  # the format numbers the C oracle and the device library use for 1-byte arrays
+
+
+def fp8_max(fmt: int = 1) -> float:
+    return {1: FP8_E4M3FN_MAX, 2: FP8_E5M2_MAX}[fmt]
+
+
+def fp8_decode(codes: np.ndarray, fmt: int = 1) -> np.ndarray:
+    return {1: _FP8_TABLE, 2: _FP8_E5M2_TABLE}[fmt][np.asarray(codes, dtype=np.uint8)]
+
+
+def fp8_e5m2_encode(x: np.ndarray) -> np.ndarray:
+    """float32 -> e5m2 code, round-to-nearest-even, as ``astype(float8_e5m2)``: magnitudes that round above 57344 become
+    infinity (0x7c), NaN becomes 0x7f.  The reference clips to +-57344 first (lyra/nn/quant.py:72)."""
+    x = np.asarray(x, dtype=np.float32)
+    sign = np.signbit(x).astype(np.uint8) << 7
+    a = np.abs(x).astype(np.float64)
+    nan = np.isnan(a)
+    inf = np.isinf(a)
+    a = np.where(nan | inf, 1.0, a)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+    e = np.clip(e, -14, 15)
+    ulp = 2.0 ** (e - 2)  # 2 mantissa bits
+    val = np.rint(a / ulp) * ulp  # numpy rint = round half to even; exact in float64
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e2 = np.floor(np.log2(np.where(val > 0, val, 1.0)))
+    e2 = np.clip(e2, -14, 16)
+    sub = val < 2.0**-14
+    mant = np.where(sub, val / 2.0**-16, (val / 2.0**e2 - 1.0) * 4.0)
+    expf = np.where(sub, 0, e2 + 15)
+    code = (expf.astype(np.int64) << 2) | np.rint(mant).astype(np.int64)
+    code = np.where((val > FP8_E5M2_MAX) | inf, 0x7C, code)
+    code = np.where(nan, 0x7F, code)
+    return ((code.astype(np.uint8) & 0x7F) | sign).astype(np.uint8)
+
+
+def fp8_encode(x: np.ndarray, fmt: int = 1) -> np.ndarray:
+    return fp8_e5m2_encode(x) if fmt == 2 else fp8_e4m3fn_encode(x)
 
 
 def fp8_e4m3fn_decode(codes: np.ndarray) -> np.ndarray:
@@ -162,8 +227,8 @@ def _block_axes(ldim: int, sdim: int) -> tuple[int, ...]:
     return tuple(ldim + 2 * i + 1 for i in range(sdim))
 
 
-def quantize(x: np.ndarray, block: tuple[int, ...]) -> tuple[np.ndarray, np.ndarray]:
-    """lyra/nn/quant.py:48-75 for dtype=float8_e4m3fn, scale_dtype=float32.
+def quantize(x: np.ndarray, block: tuple[int, ...], fmt: int = 1) -> tuple[np.ndarray, np.ndarray]:
+    """lyra/nn/quant.py:48-75 for dtype=float8_e4m3fn (``fmt`` 1) or float8_e5m2 (``fmt`` 2), scale_dtype=float32.
 
     Returns (qval uint8 codes with x.shape, scale float32 of shape lead x (dim/block)).
     """
@@ -172,21 +237,21 @@ def quantize(x: np.ndarray, block: tuple[int, ...]) -> tuple[np.ndarray, np.ndar
     ldim = x.ndim - sdim
     axes = _block_axes(ldim, sdim)
     tiled = _tile(x, block)
-    fmax = np.float32(FP8_E4M3FN_MAX)
+    fmax = np.float32(fp8_max(fmt))
     amax = np.max(np.abs(tiled), axis=axes).astype(np.float32)
     scale = np.where(amax > 0, amax / fmax, np.float32(1.0)).astype(np.float32)  # :70
     qinv = np.expand_dims((np.float32(1.0) / scale).astype(np.float32), axes)  # :71
     scaled = np.clip((tiled * qinv).astype(np.float32), -fmax, fmax)  # :72
-    qval = fp8_e4m3fn_encode(scaled).reshape(x.shape)
+    qval = fp8_encode(scaled, fmt).reshape(x.shape)
     return qval, scale
 
 
-def dequantize(qval: np.ndarray, scale: np.ndarray, block: tuple[int, ...], *, to_bf16: bool = True) -> np.ndarray:
+def dequantize(qval: np.ndarray, scale: np.ndarray, block: tuple[int, ...], *, to_bf16: bool = True, fmt: int = 1) -> np.ndarray:
     """lyra/nn/quant.py:78-86: f32(qval) * scale, then cast (bf16 by default)."""
     sdim = len(block)
     ldim = qval.ndim - sdim
     axes = _block_axes(ldim, sdim)
-    tiled = _tile(fp8_e4m3fn_decode(qval), block)
+    tiled = _tile(fp8_decode(qval, fmt), block)
     s = np.expand_dims(np.asarray(scale, dtype=np.float32), axes)
     x = (tiled * s).astype(np.float32).reshape(qval.shape)
     return bf16_round(x) if to_bf16 else x
@@ -289,12 +354,13 @@ def decode_attention_reference(
     *,
     mode: str = "fp32",
     gate: np.ndarray | None = None,
+    fp8_format: int = 1,
 ) -> np.ndarray:
     """decode_attention.py:311-361 (+ :263-308 slab path, :392-395 dequantise-first).
 
     q        [B,N,1,H] float32 holding bf16-representable values
     k, v     [B,K,S,H] float32 (bf16 cache)  or  (qval uint8, scale f32 [B,K,S,1]) for an
-             FP8 cache quantised with block (1,H)
+             FP8 cache quantised with block (1,H); ``fp8_format`` names the codes (1 e4m3fn, 2 e5m2)
     sinks    [N] float32; head n belongs to KV head n // G, slot n % G   (:349-350)
     position scalar or [B] int - index of the newest token; the reference takes one
              scalar, a vector is the ragged-batch extension (each row on its own scalar)
@@ -310,8 +376,8 @@ def decode_attention_reference(
         kq, ks = k
         vq, vs = v
         # decode_attention.py:393-394 - the whole cache is dequantised to bf16 first
-        k = dequantize(kq, ks, (1, H), to_bf16=(mode == "ref"))
-        v = dequantize(vq, vs, (1, H), to_bf16=(mode == "ref"))
+        k = dequantize(kq, ks, (1, H), to_bf16=(mode == "ref"), fmt=fp8_format)
+        v = dequantize(vq, vs, (1, H), to_bf16=(mode == "ref"), fmt=fp8_format)
     k = np.asarray(k, dtype=np.float32)
     v = np.asarray(v, dtype=np.float32)
     _, K, S, _ = k.shape
@@ -428,12 +494,13 @@ def decode_gemm_reference(
     swiglu_limit: float = 7.0,
     mode: str = "fp32",
     dequant_bf16: bool | None = None,
+    fp8_format: int = 1,
 ) -> np.ndarray:
     """decode_gemm.py:368-401 / :419-449.
 
     rhs is either float32 [G,K,N] (dense weights; the reference casts them to
     lhs.dtype = bf16, :437) or (qval uint8 [G,K,N], scale f32 [G,K/bk,N/bn]) with
-    ``block=(bk,bn)``, dequantised to lhs.dtype before the grouped product (:431).
+    ``block=(bk,bn)`` (codes of ``fp8_format``: 1 e4m3fn, 2 e5m2), dequantised to lhs.dtype before the grouped product (:431).
     The lhs is never quantised on this path (quant_dtype=None at :398).
     ``dequant_bf16`` overrides what ``mode`` says about the dequantised weights alone: True rounds them to bf16 as the
     reference does (quant.py:85) while the product, bias and SwiGLU stay in float32 when mode="fp32".
@@ -441,7 +508,7 @@ def decode_gemm_reference(
     if isinstance(rhs, tuple):
         qval, scale = rhs
         assert block is not None
-        w = dequantize(qval, scale, block, to_bf16=(mode == "ref") if dequant_bf16 is None else dequant_bf16)
+        w = dequantize(qval, scale, block, to_bf16=(mode == "ref") if dequant_bf16 is None else dequant_bf16, fmt=fp8_format)
     else:
         w = np.asarray(rhs, dtype=np.float32)
         if mode == "ref":

@@ -23,33 +23,36 @@ def t_f32(x: np.ndarray) -> torch.Tensor:
     return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(dev())
 
 
-def t_fp8(codes: np.ndarray) -> torch.Tensor:
-    return torch.from_numpy(np.ascontiguousarray(codes, dtype=np.uint8)).to(dev()).view(torch.float8_e4m3fn)
+def t_fp8(codes: np.ndarray, fmt: int = 1) -> torch.Tensor:
+    """Device tensor of 1-byte codes; fmt 1: e4m3fn, 2: e5m2 (the format numbers of the oracle)."""
+    dt = torch.float8_e5m2 if fmt == 2 else torch.float8_e4m3fn
+    return torch.from_numpy(np.ascontiguousarray(codes, dtype=np.uint8)).to(dev()).view(dt)
 
 
 def to_np(t: torch.Tensor) -> np.ndarray:
     return t.detach().to(torch.float32).cpu().numpy()
 
 
-def quantize_rows(x: np.ndarray):
+def quantize_rows(x: np.ndarray, fmt: int = 1):
     """Block (1,H) quantiser through the C oracle (bit-identical to oracle.quantize, much faster on big caches)."""
     from oracle import clib
 
-    return clib.quantize_rows(x)
+    return clib.quantize_rows(x, fp8_format=fmt)
 
 
-def attention_case(seed, B, N, K, S, H, *, fp8, q_scale=1.0):
-    """Q/K/V ~ N(0,1) rounded to bf16, sinks ~ N(0,1); FP8 cache quantised per token and kv head (block (1,H))."""
+def attention_case(seed, B, N, K, S, H, *, fp8, q_scale=1.0, fmt=1):
+    """Q/K/V ~ N(0,1) rounded to bf16, sinks ~ N(0,1); FP8 cache quantised per token and kv head (block (1,H)) to format
+    ``fmt`` (1: e4m3fn, 2: e5m2)."""
     rng = np.random.default_rng(seed)
     q = O.bf16_round((rng.standard_normal((B, N, 1, H)) * q_scale).astype(np.float32))
     k = O.bf16_round(rng.standard_normal((B, K, S, H), dtype=np.float32))
     v = O.bf16_round(rng.standard_normal((B, K, S, H), dtype=np.float32))
     sinks = rng.standard_normal(N).astype(np.float32)
-    case = {"q": q, "sinks": sinks, "fp8": fp8}
+    case = {"q": q, "sinks": sinks, "fp8": fp8, "fmt": fmt}
     if fp8:
         big = k.size > (1 << 22)
-        kq, ks = quantize_rows(k) if big else O.quantize(k, (1, H))
-        vq, vs = quantize_rows(v) if big else O.quantize(v, (1, H))
+        kq, ks = quantize_rows(k, fmt) if big else O.quantize(k, (1, H), fmt)
+        vq, vs = quantize_rows(v, fmt) if big else O.quantize(v, (1, H), fmt)
         case.update(k=(kq, ks), v=(vq, vs))
     else:
         case.update(k=k, v=v)
@@ -64,8 +67,8 @@ def attention_torch_inputs(case):
     if case["fp8"]:
         (kq, ks), (vq, vs) = case["k"], case["v"]
         H = kq.shape[-1]
-        k = QArray(t_fp8(kq), t_f32(ks), (1, H))
-        v = QArray(t_fp8(vq), t_f32(vs), (1, H))
+        k = QArray(t_fp8(kq, case.get("fmt", 1)), t_f32(ks), (1, H))
+        v = QArray(t_fp8(vq, case.get("fmt", 1)), t_f32(vs), (1, H))
     else:
         k, v = t_bf16(case["k"]), t_bf16(case["v"])
     return q, k, v, sinks

@@ -35,8 +35,10 @@ def _case(seed, M, G, K, N, sizes, *, kind, block=(256, 256), bias=False, w_std=
     w = _weights(rng, G, K, N, w_std)
     c = {"lhs": lhs, "sizes": np.asarray(sizes, np.int32), "kind": kind, "block": block}
     c["bias"] = rng.standard_normal((G, N)).astype(np.float32) if bias else None
-    if kind == "fp8":
-        c["w"] = clib.quantize_blocks(w, block)  # bit-identical to O.quantize (tests/test_oracle_formats.py)
+    c["fmt"] = 2 if kind == "e5m2" else 1  # the 1-byte format of the codes: e4m3fn unless the case says e5m2
+    if kind in ("fp8", "e5m2"):
+        c["w"] = clib.quantize_blocks(w, block, fp8_format=c["fmt"])  # bit-identical to O.quantize (tests/test_oracle_formats.py)
+        c["kind"] = "fp8"
     else:
         c["w"] = O.bf16_round(w)
     return c
@@ -51,11 +53,11 @@ def _want(c, swiglu, big=False):
         if c["kind"] == "fp8":
             q, s = c["w"]
             return clib.decode_gemm(O.bf16_bits(c["lhs"]), q, s, c["block"], c["sizes"], c["bias"], fused_swiglu=swiglu,
-                                    dequant_bf16=like_reference)
+                                    dequant_bf16=like_reference, fp8_format=c["fmt"])
         return clib.decode_gemm(O.bf16_bits(c["lhs"]), O.bf16_bits(c["w"]), None, None, c["sizes"], c["bias"], fused_swiglu=swiglu)
     if c["kind"] == "fp8":
         return O.decode_gemm_reference(c["lhs"], c["w"], c["sizes"], block=c["block"], bias=c["bias"], fused_swiglu=swiglu,
-                                       dequant_bf16=like_reference)
+                                       dequant_bf16=like_reference, fp8_format=c["fmt"])
     return O.decode_gemm_reference(c["lhs"], c["w"], c["sizes"], bias=c["bias"], fused_swiglu=swiglu)
 
 
@@ -68,8 +70,8 @@ def _run(c, swiglu, *, out_f32=False, implementation="pallas"):
         lhs = lhs.to(torch.float32)
     if c["kind"] == "fp8":
         q, s = c["w"]
-        rhs = QArray(U.t_fp8(q), U.t_f32(s), tuple(c["block"]))
-        qd = torch.float8_e4m3fn
+        rhs = QArray(U.t_fp8(q, c["fmt"]), U.t_f32(s), tuple(c["block"]))
+        qd = torch.float8_e5m2 if c["fmt"] == 2 else torch.float8_e4m3fn
     else:
         rhs = U.t_bf16(c["w"])
         qd = None
@@ -80,7 +82,8 @@ def _run(c, swiglu, *, out_f32=False, implementation="pallas"):
     return U.to_np(out)
 
 
-@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", (512, 1)), ("fp8", (512, 128)), ("fp8", (64, 64))])
+@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", (512, 1)), ("fp8", (512, 128)), ("fp8", (64, 64)),
+                                        ("e5m2", (256, 256)), ("e5m2", (512, 1))])
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_small_grouped_shapes(kind, block, swiglu):
     M, G, K, N = 11, 4, 512, 512
@@ -224,7 +227,7 @@ def test_config5_lyra_max_expert_shape_b128():
     U.assert_close(_run(down, False), _want(down, False, big=True), what="down")
 
 
-@pytest.mark.parametrize("kind,block", [("fp8", (512, 1)), ("fp8", (128, 128)), ("bf16", None)])
+@pytest.mark.parametrize("kind,block", [("fp8", (512, 1)), ("fp8", (128, 128)), ("bf16", None), ("e5m2", (512, 1))])
 def test_down_projection_with_many_units_takes_256_column_units(kind, block):
     """Without SwiGLU and with at least 1.75 rounds of 256-column units (here 34 row blocks x 16 = 544 for 256 workgroups)
     the grouped kernel picks the wider units on the device; the result must not depend on that choice."""
@@ -301,6 +304,9 @@ def test_quantize_on_the_fly_and_dispatch_contract():
     (37, 512, 256, "bf16", None, False),          # bf16 weights, one slice of 512 rows
     (64, 4096, 1024, "fp8", (128, 128), False),   # 128-row scale blocks, 8 slices
     (16, 128, 128, "fp8", (128, 1), False),       # the smallest split shape
+    (100, 1024, 512, "e5m2", (256, 256), False),  # e5m2 codes: scale blocks that change along K
+    (64, 2048, 2048, "e5m2", (2048, 1), True),    # ... per-channel scales, SwiGLU
+    (16, 2048, 512, "e5m2", (128, 128), False),   # ... 16-row blocks
 ])
 def test_split_k_dense_variants(M, K, N, kind, block, swiglu):
     """One group with a few MB of weights runs split over K: bias, padding rows (group size < M) and SwiGLU included."""
@@ -345,6 +351,7 @@ def test_units_listed_by_cost_over_several_rounds(K, N, swiglu):
 
 @pytest.mark.parametrize("kind,block,swiglu", [
     ("fp8", (2048, 1), True), ("fp8", (2048, 1), False), ("fp8", (256, 256), True), ("bf16", None, False),
+    ("e5m2", (2048, 1), True), ("e5m2", (256, 256), False),
 ])
 def test_few_units_are_cut_into_k_slices(kind, block, swiglu):
     """Fewer (row block, column span) units than compute units: every unit is cut along K, the slices meet in the
@@ -367,6 +374,8 @@ def test_few_units_are_cut_into_k_slices(kind, block, swiglu):
     (40, 6144, 4096, "fp8", (6144, 1), False),   # their down projection: 8 slices of 768 rows
     (64, 4096, 4096, "fp8", (256, 256), True),   # scale blocks along K in slices of 1024 rows
     (16, 4096, 2048, "bf16", None, False),       # bf16 weights, two register sets refilled
+    (64, 4096, 6144, "e5m2", (4096, 1), False),  # e5m2 codes in the looping variant
+    (64, 4096, 4096, "e5m2", (256, 256), True),
 ])
 def test_long_k_slices_of_larger_projections(M, K, N, kind, block, swiglu):
     """One group with tens of MB of weights: K is cut only as far as needed for one round of workgroups, so a slice is
@@ -404,7 +413,8 @@ def test_many_experts_with_scale_blocks_along_k(block, swiglu):
 
 
 @pytest.mark.parametrize("M,K,N,kind,block", [(5, 416, 131968, "bf16", None), (64, 416, 131200, "bf16", None), (33, 416, 132096, "fp8", (416, 1)),
-                                             (64, 288, 204800, "bf16", None), (17, 480, 131328, "fp8", (96, 128))])
+                                             (64, 288, 204800, "bf16", None), (17, 480, 131328, "fp8", (96, 128)),
+                                             (33, 416, 132096, "e5m2", (416, 1))])
 def test_very_wide_projection_one_workgroup_per_compute_unit(M, K, N, kind, block):
     """A single projection with more than 1024 spans of 128 columns (the LM head): one workgroup per compute unit, the
     spans dealt out evenly.  Span counts that do not divide by the number of workgroups, with bias, 1 to 4 row tiles
@@ -448,6 +458,10 @@ def test_zero_and_extreme_block_scales(G, M):
     (70, 5, 256, 200, "fp8", (64, 8), False, False),
     (33, 1, 512, 72, "fp8", (512, 8), False, True),
     (16, 1, 8192, 8200, "fp8", (8192, 1), False, False),     # large enough for K slices across workgroups + the finish kernel
+    (64, 8, 2880, 5760, "e5m2", (2880, 1), True, True),      # e5m2 codes: expert kernel at a width that is not whole spans
+    (300, 8, 2880, 2880, "e5m2", (96, 64), False, True),
+    (33, 1, 512, 72, "e5m2", (512, 8), False, True),         # ... the general kernel
+    (16, 1, 8192, 8200, "e5m2", (8192, 1), False, False),    # ... with K slices across workgroups
 ])
 def test_widths_that_are_not_whole_spans(M, G, K, N, kind, block, swiglu, bias):
     """N % 8 == 0 (N % 16 == 0 with SwiGLU) is enough: in the expert kernel and in the general kernel the lanes past the
@@ -476,7 +490,7 @@ def _run_packed(c, swiglu, *, out_f32=False, bias=True, row_map=None, rows=None)
 
     if c["kind"] == "fp8":
         q, s = c["w"]
-        rhs = QArray(U.t_fp8(q), U.t_f32(s), tuple(c["block"]))
+        rhs = QArray(U.t_fp8(q, c["fmt"]), U.t_f32(s), tuple(c["block"]))
     else:
         rhs = U.t_bf16(c["w"])
     G = len(c["sizes"])
@@ -527,7 +541,7 @@ def test_span_major_copy_is_the_documented_permutation():
                 np.testing.assert_array_equal(got.reshape(want.shape), want, err_msg=f"G{G} K{K} N{N} es{es} glu{glu}")
 
 
-@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", "channel"), ("fp8", (64, 64))])
+@pytest.mark.parametrize("kind,block", [("bf16", None), ("fp8", (256, 256)), ("fp8", "channel"), ("fp8", (64, 64)), ("e5m2", "channel")])
 @pytest.mark.parametrize("swiglu", [False, True])
 @pytest.mark.parametrize("M,G,K,N,sizes", [
     (11, 4, 512, 512, [3, 0, 7, 1]),                    # fewer units than workgroups: units cut into K slices
@@ -553,7 +567,7 @@ def test_span_major_weights_match_oracle_and_row_major_call(kind, block, swiglu,
         sizes[0] = 64  # a full block first in lhs order, last in the kernel's list
         M = int(sum(sizes)) + 3  # three rows past the last group
     blk = (K, 1) if block == "channel" else block
-    if kind == "fp8" and blk is not None and (K % blk[0] or N % blk[1]):
+    if kind != "bf16" and blk is not None and (K % blk[0] or N % blk[1]):
         pytest.skip("block does not tile the shape")
     c = _case(7, M, G, K, N, sizes, kind=kind, block=blk, bias=True, w_std=0.05)
     _note(f"span-major kind={kind} block={blk} swiglu={swiglu} M={M} G={G} K={K} N={N}")
@@ -580,12 +594,12 @@ def test_span_major_untouched_experts_are_never_read():
     U.assert_close(_run_packed(dict(c, w=(q, s)), True), want, what="poisoned idle experts, span-major")
 
 
-@pytest.mark.parametrize("kind", ["bf16", "fp8"])
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "e5m2"])
 @pytest.mark.parametrize("M,K,N,swiglu", [(64, 2048, 2048, False), (64, 2048, 6144, True), (33, 4096, 2880, False), (8, 2880, 5120, False)])
 def test_span_major_dense_projection_runs_split_over_k(kind, M, K, N, swiglu):
     """One group: the K-split kernel reads layout 1 (also under a fused SwiGLU, which its finish step applies); bit-identical
     to the row-major call, whose slices hold the same sums."""
-    block = (K, 1) if kind == "fp8" else None
+    block = (K, 1) if kind != "bf16" else None
     c = _case(9, M, 1, K, N, [M], kind=kind, block=block, bias=False)
     _note(f"span-major dense kind={kind} M={M} K={K} N={N} swiglu={swiglu}")
     got = _run_packed(c, swiglu, out_f32=True)

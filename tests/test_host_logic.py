@@ -42,6 +42,20 @@ def test_quantize_dequantize_bit_exact_with_oracle():
         quantize(_bf16(x), torch.bfloat16, (1, 64))
 
 
+def test_quantize_to_e5m2_bit_exact_with_oracle():
+    """The host-side producer of QArrays with dtype=float8_e5m2 (the other member of FP8_DTYPES, lyra/nn/quant.py:10)."""
+    from lyra_amd.nn.quant import dequantize, quantize
+
+    rng = np.random.default_rng(5)
+    x = O.bf16_round((rng.standard_normal((3, 256, 128)) * np.exp(rng.standard_normal((3, 1, 1)) * 3)).astype(np.float32))
+    for block in ((1, 128), (256, 1), (64, 64)):
+        qa = quantize(torch.from_numpy(x), torch.float8_e5m2, block)
+        wq, ws = O.quantize(x, block, fmt=2)
+        assert np.array_equal(qa.qval.view(torch.uint8).numpy(), wq)
+        assert np.array_equal(qa.scale.numpy(), ws)
+        assert np.array_equal(dequantize(qa, torch.bfloat16).float().numpy(), O.dequantize(wq, ws, block, fmt=2))
+
+
 def test_dispatch_contract():
     from lyra_amd.kernels.common import dispatch_kernel
 

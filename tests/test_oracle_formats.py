@@ -158,3 +158,99 @@ def test_qupdate_writes_one_token():
     keep[5] = False
     np.testing.assert_array_equal(q2[:, :, keep], q[:, :, keep])
     np.testing.assert_array_equal(s2[:, :, keep], s[:, :, keep])
+
+
+# ---- the second 1-byte format of the reference's FP8_DTYPES (lyra/nn/quant.py:10): e5m2 -------------------------------
+def _torch_e5m2_decode(codes: np.ndarray) -> np.ndarray:
+    return torch.from_numpy(codes.astype(np.uint8)).view(torch.float8_e5m2).to(torch.float32).numpy()
+
+
+def _torch_e5m2_encode(x: np.ndarray) -> np.ndarray:
+    return torch.from_numpy(x.astype(np.float32)).to(torch.float8_e5m2).view(torch.uint8).numpy()
+
+
+def test_e5m2_decode_all_256_codes_match_torch_and_float16():
+    codes = np.arange(256, dtype=np.uint8)
+    want = _torch_e5m2_decode(codes)
+    got = O.fp8_decode(codes, 2)
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+    # the format is the upper byte of IEEE float16: a second, independent definition
+    half = (codes.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+    np.testing.assert_array_equal(got[~np.isnan(want)], half[~np.isnan(want)])
+    lib = clib.load()
+    got_c = np.array([lib.lyra_oracle_fp8_e5m2_to_f32(int(c)) for c in codes], dtype=np.float32)
+    np.testing.assert_array_equal(got_c[~np.isnan(want)], want[~np.isnan(want)])
+    assert got[0x7B] == 57344.0 and np.isinf(got[0x7C]) and np.isnan(got[0x7D])  # finfo(float8_e5m2).max, then inf / NaN
+    assert O.fp8_max(2) == float(torch.finfo(torch.float8_e5m2).max) and O.fp8_max(1) == float(torch.finfo(torch.float8_e4m3fn).max)
+
+
+def test_e5m2_encode_values_midpoints_and_neighbours_match_torch():
+    table = O.fp8_decode(np.arange(0x7C, dtype=np.uint8), 2)  # positive finite codes, ascending
+    mids = (table[:-1].astype(np.float64) + table[1:].astype(np.float64)) / 2  # exact ties
+    eps = np.float32(1e-3)
+    pts = np.concatenate([table, mids.astype(np.float32), np.nextafter(mids.astype(np.float32), np.float32(0)),
+                          np.nextafter(mids.astype(np.float32), np.float32(1e9)), table * (1 + eps), table * (1 - eps)])
+    pts = np.concatenate([pts, -pts, [0.0, -0.0, 2.0**-17, 2.0**-18, 3 * 2.0**-18, 57343.0, 57344.0]]).astype(np.float32)
+    pts = pts[np.abs(pts) <= 57344.0]
+    want = _torch_e5m2_encode(pts)
+    got = O.fp8_encode(pts, 2)
+    np.testing.assert_array_equal(got, want)
+    lib = clib.load()
+    got_c = np.array([lib.lyra_oracle_f32_to_fp8_e5m2(float(p)) for p in pts], dtype=np.uint8)
+    np.testing.assert_array_equal(got_c, want)
+    rng = np.random.default_rng(10)
+    x = (rng.standard_normal(20000) * rng.choice([1e-5, 1e-3, 1.0, 300.0, 20000.0], 20000)).astype(np.float32)
+    x = np.clip(x, -57344, 57344)
+    np.testing.assert_array_equal(O.fp8_encode(x, 2), _torch_e5m2_encode(x))
+
+
+def test_e5m2_quantize_matches_torch_elementwise_and_c():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((4, 7, 128)).astype(np.float32)
+    x[2, 3] = 0.0
+    q, s = O.quantize(x, (1, 128), fmt=2)
+    amax = np.abs(x).max(-1, keepdims=True)
+    np.testing.assert_array_equal(s[amax > 0], (amax[amax > 0] / np.float32(57344.0)).astype(np.float32))
+    assert s[2, 3, 0] == 1.0 and (q[2, 3] == 0).all()
+    inv = (np.float32(1.0) / s).astype(np.float32)
+    scaled = np.clip((x * inv).astype(np.float32), -57344, 57344)
+    np.testing.assert_array_equal(q, _torch_e5m2_encode(scaled))
+    d = O.dequantize(q, s, (1, 128), fmt=2)
+    want = torch.from_numpy(_torch_e5m2_decode(q) * s).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(d, want)
+    qc, sc = clib.quantize_rows(x, fp8_format=2)
+    np.testing.assert_array_equal(qc, q)
+    np.testing.assert_array_equal(sc, s)
+    # round-trip error: half an ulp of 2 mantissa bits (2^-3 relative) in the normal range
+    err = np.abs(O.dequantize(q, s, (1, 128), to_bf16=False, fmt=2) - x)
+    assert (err <= np.maximum(np.abs(x) * 2.0**-3, s * 2.0**-17) * (1 + 1e-6)).all()
+    w = (rng.standard_normal((2, 256, 256)) * 0.02).astype(np.float32)
+    for block in ((256, 256), (256, 1), (64, 128)):
+        qn, sn = O.quantize(w, block, fmt=2)
+        qb, sb = clib.quantize_blocks(w, block, fp8_format=2)
+        np.testing.assert_array_equal(qb, qn)
+        np.testing.assert_array_equal(sb, sn)
+
+
+def test_e5m2_operators_of_the_c_oracle_match_numpy():
+    """The C attention and matmul read e5m2 codes through the table pinned above: same results as the numpy forms."""
+    rng = np.random.default_rng(12)
+    B, N, K, S, H = 2, 4, 2, 96, 64
+    q = O.bf16_round(rng.standard_normal((B, N, 1, H)).astype(np.float32))
+    kq, ks = O.quantize(rng.standard_normal((B, K, S, H)).astype(np.float32), (1, H), fmt=2)
+    vq, vs = O.quantize(rng.standard_normal((B, K, S, H)).astype(np.float32), (1, H), fmt=2)
+    sinks = rng.standard_normal(N).astype(np.float32)
+    pos = np.array([S - 1, 40])
+    want = O.decode_attention_reference(q, (kq, ks), (vq, vs), sinks, H**-0.5, 0, pos, fp8_format=2)
+    got = clib.decode_attention(O.bf16_bits(q), kq, vq, ks, vs, sinks, pos, None, H**-0.5, 0, fp8_format=2)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+    other = clib.decode_attention(O.bf16_bits(q), kq, vq, ks, vs, sinks, pos, None, H**-0.5, 0, fp8_format=1)
+    assert np.abs(other - want).max() > 1e-2  # (the format argument is not ignored)
+    M, G, Kd, Nd = 12, 3, 64, 32
+    lhs = O.bf16_round(rng.standard_normal((M, Kd)).astype(np.float32))
+    wq, wsc = O.quantize((rng.standard_normal((G, Kd, Nd)) * 0.05).astype(np.float32), (32, 16), fmt=2)
+    sizes = np.array([5, 0, 7], dtype=np.int32)
+    want = O.decode_gemm_reference(lhs, (wq, wsc), sizes, block=(32, 16), fp8_format=2)
+    got = clib.decode_gemm(O.bf16_bits(lhs), wq, wsc, (32, 16), sizes, None, fp8_format=2)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
