@@ -9,6 +9,7 @@ the threaded C restatement when ``use_c`` is set (bench baseline, large parity c
 """
 from __future__ import annotations
 
+import functools
 import math
 
 import numpy as np
@@ -19,18 +20,20 @@ from oracle import lyra_oracle as O
 R = O.bf16_round
 
 
-def _gemm(lhs, w, sizes, *, swiglu=False, beta=1.702, limit=7.0, use_c=False, out_bf16=True, bias=None, inner="ref"):
+def _gemm(lhs, w, sizes, *, swiglu=False, beta=1.702, limit=7.0, use_c=False, out_bf16=True, bias=None, inner="ref", fmt=1):
     """decode_gemm / quant.dot: w is float32 [G,K,N] (bf16 weights) or (qval, scale, block); bias [G,N] float32 or None.
     inner="ref": dequantised weights are rounded to bf16 before the product, as the JAX code holds them (quant.py:85);
-    inner="fp32": the product is taken on the exact dequantised values; either way the result is one bf16 array."""
+    inner="fp32": the product is taken on the exact dequantised values; either way the result is one bf16 array.
+    fmt: the 1-byte format of quantised weights (1 e4m3fn, 2 e5m2)."""
     ref = inner == "ref"
     if isinstance(w, tuple):
         q, s, block = w
         if use_c:
-            y = clib.decode_gemm(O.bf16_bits(lhs), q, s, block, sizes, bias, fused_swiglu=swiglu, beta=beta, limit=limit, ref_rounding=ref)
+            y = clib.decode_gemm(O.bf16_bits(lhs), q, s, block, sizes, bias, fused_swiglu=swiglu, beta=beta, limit=limit, ref_rounding=ref,
+                                 fp8_format=fmt)
         else:
             y = O.decode_gemm_reference(lhs, (q, s), sizes, block=block, bias=bias, fused_swiglu=swiglu, swiglu_beta=beta, swiglu_limit=limit,
-                                        mode="ref" if ref else "fp32")
+                                        mode="ref" if ref else "fp32", fp8_format=fmt)
         return R(y) if out_bf16 else y
     if use_c:
         y = clib.decode_gemm(O.bf16_bits(lhs), O.bf16_bits(w), None, None, sizes, bias, fused_swiglu=swiglu, beta=beta, limit=limit, ref_rounding=out_bf16)
@@ -59,6 +62,8 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
     layer_offset: index, in the whole model, of the first layer of ``weights["layers"]`` (even layers have the sliding
     window, model.py:337): lets a caller run a few layers of a deep model on their own, fed that layer's input as "emb".
     """
+    fmt = 2 if str(getattr(cfg, "gemm_dtype", "")).endswith("e5m2") else 1  # the format of every FP8 array of the model (one config field)
+    gemm = functools.partial(_gemm, fmt=fmt)
     B = tokens.shape[0]
     C, H, N, K = cfg.n_embd, cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads
     cos_t, sin_t = O.rope_tables(cfg.seq_len, H, cfg.rope_base, cfg.rope_scale, cfg.ntk_alpha, cfg.ntk_beta)
@@ -71,7 +76,7 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
         # ---- attention_apply ----
         a = lw["attn"]
         hn = R(O.rms_norm(h, a["norm_scale"], cfg.norm_eps))
-        qkv = _gemm(hn, a["qkv"], one, use_c=use_c, inner=inner)
+        qkv = gemm(hn, a["qkv"], one, use_c=use_c, inner=inner)
         if a.get("qkv_bias") is not None:  # model.py:310-313
             qkv = R(qkv + _bias(a["qkv_bias"]))
         q, k, v = np.split(qkv, [N * H, (N + K) * H], axis=-1)
@@ -83,7 +88,7 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
         ck, cv = cache["k"][idx - layer_offset], cache["v"][idx - layer_offset]
         if isinstance(ck, tuple):  # qupdate: quantise the new token with block (1, H) and write it at pos
             for (cq, cs), new in ((ck, k), (cv, v)):
-                nq, ns = O.quantize(new[:, :, None, :], (1, H))
+                nq, ns = O.quantize(new[:, :, None, :], (1, H), fmt)
                 cq[:, :, pos : pos + 1] = nq
                 cs[:, :, pos : pos + 1] = ns
         else:
@@ -98,18 +103,19 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
         if use_c:
             if isinstance(ck, tuple):
                 t = clib.decode_attention(O.bf16_bits(q[:, :, None, :]), ck[0], cv[0], ck[1][..., 0], cv[1][..., 0], a["sinks"],
-                                          pos, g_in, H**-0.5, sw, ref_rounding=ref)
+                                          pos, g_in, H**-0.5, sw, ref_rounding=ref, fp8_format=fmt)
             else:
                 t = clib.decode_attention(O.bf16_bits(q[:, :, None, :]), O.bf16_bits(ck), O.bf16_bits(cv), None, None, a["sinks"],
                                           pos, g_in, H**-0.5, sw, ref_rounding=ref)
         else:
-            t = O.decode_attention_reference(q[:, :, None, :], ck, cv, a["sinks"], H**-0.5, sw, pos, mode="ref" if ref else "fp32", gate=g_in)
+            t = O.decode_attention_reference(q[:, :, None, :], ck, cv, a["sinks"], H**-0.5, sw, pos, mode="ref" if ref else "fp32", gate=g_in,
+                                             fp8_format=fmt)
         if not ref and gate is not None:
             t = R(R(t) * gate[:, :, None, None])
         t = R(t.reshape(B, N, H))
         if a.get("xsa_alpha") is not None:  # model.py:351-363, on the new token's value rows as projected (not as cached)
             t = O.xsa(t, v, a["xsa_alpha"], mode="ref")
-        t = _gemm(t.reshape(B, N * H), a["out"], one, use_c=use_c, inner=inner)
+        t = gemm(t.reshape(B, N * H), a["out"], one, use_c=use_c, inner=inner)
         if a.get("out_bias") is not None:  # model.py:367-368
             t = R(t + _bias(a["out_bias"]))
         t = R(t * np.float32(cfg.residual_scale))
@@ -129,9 +135,9 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
             topk = cfg.n_active_experts
             perm, dest = O.bpermute(active_map, groups, cfg.n_experts)
             t = xn[perm // topk]
-            t = _gemm(t, m["mlp_up"], groups, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
+            t = gemm(t, m["mlp_up"], groups, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
                       bias=_bias(m.get("mlp_up_bias")), inner=inner)
-            t = _gemm(R(t), m["mlp_down"], groups, use_c=use_c, bias=_bias(m.get("mlp_down_bias")), inner=inner)
+            t = gemm(R(t), m["mlp_down"], groups, use_c=use_c, bias=_bias(m.get("mlp_down_bias")), inner=inner)
             t = R(O.combine(R(t), scores, dest))
             t = R(t * np.float32(cfg.residual_scale))
             h = R(h + t)
@@ -139,13 +145,13 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
             if ref and m.get("mlp_up_bias") is not None:
                 # model.py:613-616: the product is a bf16 array, the bias is added to it in bf16, SwiGLU follows
                 # (inner="fp32", like the kernels, adds the bias to the float32 product inside the fused epilogue)
-                t = _gemm(xn, m["mlp_up"], one, use_c=use_c, inner=inner)
+                t = gemm(xn, m["mlp_up"], one, use_c=use_c, inner=inner)
                 t = R(t + _bias(m["mlp_up_bias"])[0])
                 t = R(O.swiglu(t, cfg.swiglu_beta, cfg.swiglu_limit))
             else:
-                t = _gemm(xn, m["mlp_up"], one, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
+                t = gemm(xn, m["mlp_up"], one, swiglu=True, beta=cfg.swiglu_beta, limit=cfg.swiglu_limit, use_c=use_c,
                           bias=_bias(m.get("mlp_up_bias")), inner=inner)
-            t = _gemm(R(t), m["mlp_down"], one, use_c=use_c, inner=inner)
+            t = gemm(R(t), m["mlp_down"], one, use_c=use_c, inner=inner)
             if m.get("mlp_down_bias") is not None:  # model.py:629-630
                 t = R(t + _bias(m["mlp_down_bias"])[0])
             t = R(t * np.float32(cfg.dense_residual_scale))
@@ -153,7 +159,7 @@ def decode_step(tokens, weights, cache, pos, cfg, *, use_c=False, router_margins
     if hidden_out is not None:
         hidden_out.append(h.copy())
     h = R(O.rms_norm(h, weights["norm_scale"], cfg.norm_eps))
-    logits = _gemm(h, weights["unemb_t"], one, use_c=use_c, out_bf16=False)
+    logits = gemm(h, weights["unemb_t"], one, use_c=use_c, out_bf16=False)
     logits[:, cfg.vocab_size :] = -np.inf
     return logits
 

@@ -61,13 +61,15 @@ def _run_steps(cfg, B, S, steps, start, use_c=False):
                 kq = ck.qval.view(torch.uint8)[:, :, start + s].cpu().numpy()
                 ks = ck.scale[:, :, start + s].float().cpu().numpy()
                 oq, osc = cn["k"][l][0][:, :, start + s], cn["k"][l][1][:, :, start + s]
-                np.testing.assert_allclose(O.fp8_e4m3fn_decode(kq) * ks, O.fp8_e4m3fn_decode(oq) * osc, atol=0.08, rtol=0.08)
+                fmt = 2 if ck.qval.dtype == torch.float8_e5m2 else 1
+                step = 0.16 if fmt == 2 else 0.08  # one code step: 2 mantissa bits for e5m2, 3 for e4m3fn
+                np.testing.assert_allclose(O.fp8_decode(kq, fmt) * ks, O.fp8_decode(oq, fmt) * osc, atol=step, rtol=step)
                 if l == 0:
                     assert (kq == oq).mean() > 0.8  # the rest sits one FP8 step away (checked by value above)
     assert int(cache.pos.item()) == start + steps
 
 
-@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("fp8", [False, True, "e5m2"])
 def test_dev_model_decode_steps_match_oracle(fp8):
     from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides
 
@@ -75,6 +77,8 @@ def test_dev_model_decode_steps_match_oracle(fp8):
     cfg = replace(cfg, sliding_window=128, use_sdpa_output_gate=True, seq_len=512, implementation="pallas")
     if fp8:
         cfg = apply_inference_overrides(cfg, fp8=True, fp8_attn=True)
+    if fp8 == "e5m2":  # every FP8 array of the model (weights, cache) in the other format of FP8_DTYPES
+        cfg = replace(cfg, gemm_dtype=torch.float8_e5m2)
     _run_steps(cfg, B=3, S=512, steps=3, start=200)
 
 

@@ -155,14 +155,17 @@ def test_routing_and_permutation_match_oracle():
     assert np.array_equal(perm.numpy(), o_perm) and np.array_equal(dest.numpy(), o_dest)
 
 
-@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("fp8", [False, True, "e5m2"])
 def test_decode_step_driver_on_cpu_matches_oracle(fp8):
-    """model_apply with the plain-framework operators on CPU tensors: the same op sequence as the oracle's decode step."""
+    """model_apply with the plain-framework operators on CPU tensors: the same op sequence as the oracle's decode step
+    ("e5m2": FP8 weights and cache in the other format of FP8_DTYPES, lyra/nn/quant.py:10)."""
     from lyra_amd.model import MODEL_VARIANTS, apply_inference_overrides, init_cache, init_weights, model_apply
 
     cfg = replace(MODEL_VARIANTS["dev"], implementation="xla", seq_len=128, use_sdpa_output_gate=True, sliding_window=128)
     if fp8:
         cfg = apply_inference_overrides(cfg, fp8=True)
+    if fp8 == "e5m2":
+        cfg = replace(cfg, gemm_dtype=torch.float8_e5m2)
     dev = torch.device("cpu")
     w = init_weights(cfg, dev, seed=1)
     cache = init_cache(cfg, 2, 128, dev)
