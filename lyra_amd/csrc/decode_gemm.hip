@@ -1979,6 +1979,7 @@ int launch_planned(GemmParams p, const GemmPlan& pl, int layout, int fused_swigl
     return LYRA_OK;
 }
 #if LYRA_GEMM_PART == 1
+extern template int launch_planned<2>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);  // (pass 3 has it)
 template int launch_planned<0>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);
 template int launch_planned<1>(GemmParams, const GemmPlan&, int, int, float*, hipStream_t);
 #elif LYRA_GEMM_PART == 3
