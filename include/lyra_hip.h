@@ -251,7 +251,9 @@ int lyra_decode_gemm_ex(const void* lhs, const int32_t* lhs_row_map, const void*
  *                                                                                            s < ceil(N / 2 / 64)
  * with zeros where the column does not exist (a last span that N does not fill).  Scales, biases and outputs keep the
  * reference's column order.  lyra_decode_gemm_ex takes layout 2 for several groups with fused_swiglu, layout 1 for
- * several groups without and for the K-split projections of one group (with or without fused_swiglu), and answers
+ * several groups without, for the K-split projections of one group (with or without fused_swiglu) and for the
+ * general kernel without fused_swiglu (the LM head, also through lyra_decode_gemm_tile_max: bit-identical results; a
+ * wavefront then walks one contiguous run instead of K pieces N elements apart), and answers
  * LYRA_E_UNSUPPORTED for any other combination; lyra_decode_gemm_partials takes layout 1.  Results are the same
  * function of the same weights; the float32 summation order over K may differ from the row-major call's.
  *   lyra_gemm_packed_bytes  size of the packed copy (0 for bad arguments)

@@ -330,10 +330,13 @@ void decode_gemm_kernel(GemmParams p) {
     if (!span_ok) ncol = out_col = 0;  // idle wavefront of the last workgroup, lanes past the last column: keep pace, store nothing
 
     const int k0 = ks * p.kpart, k1 = min(p.K, k0 + p.kpart);
-    const int row_bytes = p.N * ES;
+    // row-major weights: a row of the group's matrix is N elements; span-major (GemmParams::packed, layout 1): this
+    // wavefront's span is K contiguous rows of 128 elements, and the spans of a group follow each other
+    const int row_bytes = p.packed ? 128 * ES : p.N * ES;
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.rhs) + (size_t)g * p.K * row_bytes, 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
-    const int wvoff = 8 * kb * row_bytes + ncol * ES;
+        const_cast<uint8_t*>(p.rhs) + (size_t)g * (p.packed ? p.pspans * 128 : p.N) * p.K * ES, 0,
+        (uint32_t)p.K * (uint32_t)((p.packed ? p.pspans * 128 : p.N) * ES), 0x00020000);
+    const int wvoff = p.packed ? ((span < end_span ? span : 0) * p.K + 8 * kb) * row_bytes + 8 * x * ES : 8 * kb * row_bytes + ncol * ES;
     const float* sc_lane = nullptr;
     if (FP8 && p.scale_mode == 1) sc_lane = p.scale + (size_t)g * p.KB * p.NB + (ncol >> p.bn_shift);
 
@@ -2119,9 +2122,10 @@ static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const vo
         else return LYRA_E_UNSUPPORTED;
     }
     const GemmPlan pl = plan_gemm(M, G, K, N, fp8 ? bk : 0, fused_swiglu);
-    // the packed copy exists for the kernels that stream whole spans: several groups (layout 2 with SwiGLU, else 1) and
-    // the K-split projections of one group (layout 1)
-    if (layout && !((pl.grouped && layout == (fused_swiglu ? 2 : 1)) || (!pl.grouped && pl.split_k && layout == 1))) return LYRA_E_UNSUPPORTED;
+    // the packed copy exists for the kernels that stream whole spans: several groups (layout 2 with SwiGLU, else 1), the
+    // K-split projections of one group (layout 1) and the general kernel without SwiGLU (layout 1; offsets below 2 GB)
+    if (layout && !((pl.grouped && layout == (fused_swiglu ? 2 : 1)) || (!pl.grouped && pl.split_k && layout == 1) ||
+                    (!pl.grouped && !pl.split_k && !pl.one_pass && layout == 1 && !fused_swiglu && (size_t)G * packed_spans(N, 1) * K * 256 < (1ull << 31)))) return LYRA_E_UNSUPPORTED;
     if (layout && ((uintptr_t)rhs % 128)) return LYRA_E_BADARG;
     p.packed = layout;
     p.pspans = layout ? packed_spans(N, layout) : 0;

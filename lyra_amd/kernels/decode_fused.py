@@ -130,18 +130,20 @@ _SPAN_MAJOR: dict = {}
 _SPAN_MAJOR_MODE = __import__("os").environ.get("LYRA_SPAN_MAJOR", "auto")  # tuning override: "0" never, "1" every weight
 
 
-def span_major(rhs, glu: bool = False):
+def span_major(rhs, glu: bool = False, always: bool = False):
     """The weight operand a fused decode step should hand to ``gemm``: the span-major copy (made once per weight array and
     kept) when the rows of the reference's array do not start on 128-byte lines - FP8 weights whose width, or whose linear
     half under a fused SwiGLU, is not a multiple of 128 columns, as with gpt-oss-20b's 2880: every 128-byte piece a
-    workgroup reads from such an array straddles two lines and the launch fetches half as much again - else ``rhs``."""
+    workgroup reads from such an array straddles two lines and the launch fetches half as much again - else ``rhs``.
+    ``always``: the copy whatever the width (the LM head: a wavefront then walks one contiguous 512 KB run instead of 2048
+    pieces 400 KB apart, 2-3 % of that launch)."""
     if isinstance(rhs, SpanMajor) or _SPAN_MAJOR_MODE == "0":
         return rhs
     fp8 = isinstance(rhs, QArray)
     rv = rhs.qval if fp8 else rhs
     N = rv.shape[-1]
     row = N * rv.element_size()
-    if _SPAN_MAJOR_MODE != "1" and row % 128 == 0 and not (glu and (row // 2) % 128):
+    if _SPAN_MAJOR_MODE != "1" and not always and row % 128 == 0 and not (glu and (row // 2) % 128):
         return rhs
     if N % (16 if glu else 8) or not rv.is_cuda:
         return rhs
@@ -439,7 +441,7 @@ def gemm_tile_max(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, bias: torch
     with the maximum of every 128-column tile of every result row, which ``argmax`` / ``sample_topk`` take as
     ``tile_max``.  Returns (out [M, N], tile_max [M, ceil(N / 128)]) or None for a shape the launch does not take."""
     rv, rs, bk, bn, rd, (G, K, N) = _rhs_args(rhs)
-    if G != 1 or isinstance(rhs, SpanMajor) or not isinstance(lhs, torch.Tensor):
+    if G != 1 or not isinstance(lhs, torch.Tensor):
         return None
     M = lhs.shape[0]
     assert lhs.dtype == torch.bfloat16 and lhs.is_contiguous() and lhs.shape[1] == K
@@ -455,6 +457,8 @@ def gemm_tile_max(lhs: torch.Tensor, rhs, group_sizes: torch.Tensor, bias: torch
                                       out.data_ptr(), tmax.data_ptr(), ws.data_ptr(), ws.numel(), M, 1, K, N, rd, _lib.DTYPE_F32,
                                       stream)
     if rc == _lib.E_UNSUPPORTED:
+        if isinstance(rhs, SpanMajor) and rhs.fallback is not None:  # (a shape whose kernel does not read this layout)
+            return gemm_tile_max(lhs, rhs.fallback, group_sizes, bias=bias)
         return None
     _lib.check(rc, "lyra_decode_gemm_tile_max")
     return out, tmax

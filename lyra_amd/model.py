@@ -612,11 +612,12 @@ def model_apply_fused(tokens: torch.Tensor, model: ModelWeights, cache: ModelCac
     # The LM head also leaves the maximum of every 128-column tile of the logits; they travel with the tensor (with the
     # version it had when they were taken) and `sample_token` hands them to a sampler that reads a few tiles per row instead
     # of the whole vocabulary - unless the logits have been written to since.
-    with_max = F.gemm_tile_max(h, model.unemb_t, _one_group(h.shape[0], h.device), bias=model.vocab_mask) if _LOGIT_TILE_MAX else None
+    w_head = F.span_major(model.unemb_t, always=True)  # (the span-major copy, made on the first step and kept)
+    with_max = F.gemm_tile_max(h, w_head, _one_group(h.shape[0], h.device), bias=model.vocab_mask) if _LOGIT_TILE_MAX else None
     if with_max is not None:
         logits = with_max[0]
     else:
-        logits = F.gemm(h, model.unemb_t, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
+        logits = F.gemm(h, w_head, _one_group(h.shape[0], h.device), out_f32=True, bias=model.vocab_mask)
     if model.vocab_mask is None:
         logits[:, cfg.vocab_size :] = float("-inf")
     elif with_max is not None:

@@ -605,3 +605,42 @@ def test_span_major_dense_projection_runs_split_over_k(kind, M, K, N, swiglu):
     got = _run_packed(c, swiglu, out_f32=True)
     np.testing.assert_array_equal(got, _run(c, swiglu, out_f32=True))
     U.assert_close(got, _want(c, swiglu, big=True), atol=2e-3, rtol=2e-3, what="span-major dense")
+
+
+@pytest.mark.parametrize("M,K,N,kind,block", [
+    (64, 2048, 204800, "bf16", None),        # the LM head: one workgroup per compute unit, 6 or 7 spans each
+    (5, 1248, 131968, "bf16", None),         # 1031 spans, one 16-row tile
+    (33, 1248, 132096, "fp8", (1248, 1)),    # FP8 with per-column scales
+    (17, 1440, 131328, "e5m2", (96, 128)),   # scale blocks along K
+    (16, 32768, 8200, "fp8", (32768, 1)),    # K split across workgroups + the finish kernel; a last span that N does not fill
+    (40, 262144, 1024, "bf16", None),        # few spans, many K slices
+])
+def test_span_major_weights_in_the_general_kernel(M, K, N, kind, block):
+    """One group whose weights are too large for the K-split kernel (the LM head above all): the general kernel reads
+    layout 1 as well - every wavefront one contiguous run of K rows of 128 weights - with results bit-identical to the
+    row-major call (same products, same order), logits and tile maxima alike."""
+    from lyra_amd import _lib
+    from lyra_amd.kernels import decode_fused as F
+    from lyra_amd.nn.quant import QArray
+
+    c = _case(43, M, 1, K, N, [M - 1], kind=kind, block=block, bias=True, w_std=0.05)
+    _note(f"span-major general kernel M={M} K={K} N={N} kind={kind} block={block}")
+    assert _lib.lib.lyra_decode_gemm_splits(M, K, N, block[0] if block else 0) == 0, "not a shape of the K-split kernel"
+    got = _run_packed(c, False, out_f32=True)
+    np.testing.assert_array_equal(got, _run(c, False, out_f32=True))
+    U.assert_close(got, _want(c, False, big=True), atol=2e-3, rtol=2e-3, what="span-major general f32")
+    U.assert_close(_run_packed(c, False), _want(c, False, big=True), what="span-major general bf16")
+    # with the tile maxima (the launch of the LM head inside a decode step)
+    if c["kind"] == "fp8":
+        rhs = QArray(U.t_fp8(c["w"][0], c["fmt"]), U.t_f32(c["w"][1]), tuple(block))
+    else:
+        rhs = U.t_bf16(c["w"])
+    gs = torch.from_numpy(c["sizes"]).to(U.dev())
+    bias = U.t_f32(c["bias"]).reshape(-1)
+    plain = F.gemm_tile_max(U.t_bf16(c["lhs"]), rhs, gs, bias=bias)
+    packed = F.gemm_tile_max(U.t_bf16(c["lhs"]), F.pack_weights(rhs), gs, bias=bias)
+    if plain is None:  # (a plan with K slices leaves no tile maxima, in either layout)
+        assert packed is None
+    else:
+        assert torch.equal(plain[0], packed[0]) and torch.equal(plain[1], packed[1])
+        np.testing.assert_array_equal(U.to_np(packed[0]), got)
