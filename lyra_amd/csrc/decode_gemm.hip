@@ -1524,6 +1524,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
                         *(f32x4*)(dst + 3 * TS) = f32x4{0.f, 0.f, 0.f, 0.f};
                     }
                 }
+                // The epilogue of a span-major SwiGLU unit below reads the tile by another thread mapping than the one that
+                // just wrote the sums (every other epilogue reads what the same thread wrote): the writes must have landed.
+                // (`finish` is the same in every thread of the workgroup, so all of them arrive here.)
+                if (PACKED && p.swiglu) lds_barrier();
             }
         }
         if (finish && PACKED && p.swiglu) {

@@ -552,6 +552,8 @@ def test_span_major_copy_is_the_documented_permutation():
     (300, 16, 64, 8192, None),                          # ... and with it (64 spans of 64 + 64 columns)
     (40, 3, 320, 2880, [20, 0, 20]),                    # a width that fills no whole number of spans (22.5)
     (7, 5, 64, 48, [2, 1, 0, 3, 1]),                    # narrower than one span, padding rows (sum < M is drawn below)
+    (100, 8, 2048, 1024, [3, 2, 5, 27, 11, 17, 22, 0]),  # K slices of SwiGLU units with two row tiles: the summed tile is read by
+    (23, 3, 2048, 4096, [6, 9, 5]),                     # other threads than wrote it (once a race, found by drawn shapes)
 ])
 def test_span_major_weights_match_oracle_and_row_major_call(kind, block, swiglu, M, G, K, N, sizes):
     """Every grouped-matmul case through the span-major copy: against the oracle at the acceptance bound, float32 output at
