@@ -65,6 +65,7 @@ struct GemmParams {
     int bias_post;      // one group, no SwiGLU: the bias is added to the bf16-rounded product, in bf16 (then scale / residual)
     int max_slices;     // grouped kernel: most K slices a left-over unit is cut into
     int snake;          // grouped kernel: odd rounds of units run over the workgroups in the opposite direction (-1: if >= 4 rounds)
+    int touch_last;     // grouped kernel: touch the first weights of the last group's units before the unit list is known
     int even_spans;     // plain kernel: spans dealt out evenly over one workgroup per compute unit
     int row_block;      // K-split kernel: rows per workgroup (64 or 32)
     const int32_t* row_map;    // lhs row that feeds sorted row r (gather fused into the activation load), or null
@@ -1123,10 +1124,32 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
 
     // ---- unit list: thread t looks at group G-1-t ----
     const int t = threadIdx.x;
+    [[maybe_unused]] uint32_t touched[2] = {0u, 0u};  // (what the touch below reads: looked at once, at the very end)
     int my_cnt = 0, my_before = 0;  // rows of "my" group and rows of all groups before it (in lhs order)
     int total_rows;
     {
         const int v = t < p.G ? p.group_sizes[t] : 0;
+        // The list starts with the row blocks of the last group, which is where a model keeps its shared expert: every
+        // token has a row there, so the units with the most rows - the ones that decide how long the launch lasts - are
+        // known before the group sizes are.  The workgroups that own them if that holds touch the lines of their first
+        // DEPTH steps now (one lane per 128-byte line, behind the request for the group sizes so that nothing waits for
+        // them): the real requests, two round trips later, then meet them in L2.  Where it does not hold, a few
+        // workgroups have fetched 64 KB each for nothing.
+        if constexpr (!WIDE_DYN && !PACKED) {
+            const int blk0 = (int)blockIdx.x / spans, span0 = (int)blockIdx.x - blk0 * spans;
+            const bool guess = p.touch_last && blk0 * (16 * MTM) < p.M;
+            const __amdgpu_buffer_rsrc_t trsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint8_t*>(p.rhs) + (size_t)(p.G - 1) * p.K * row_bytes, 0, (uint32_t)p.K * (uint32_t)row_bytes, 0x00020000);
+            const int col0 = (half * half_stride + span0 * span_cols) * ES;  // first byte of this wavefront's columns in a row
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int line = lane + 64 * j;                  // 128 lines: DEPTH steps x 32 rows x ES lines
+                const int rowi = line / ES, sub = line - rowi * ES;
+                const int idx = rowi >> 5, r = rowi & 31;
+                const int off = ((wslot + kw * idx) * 32 + r) * row_bytes + col0 + 128 * sub;
+                touched[j] = __builtin_amdgcn_raw_buffer_load_b32(trsrc, guess && idx < n_my ? off : kNoLoad, 0, 0);
+            }
+        }
         const int before = wg_scan_exclusive(v, sm_scan, lane, wave, total_rows);
         // hand (before, size) of natural group t to the thread that owns it in heavy-first order: thread G-1-t
         int* tmp = (int*)sm_part;  // scratch before the tiles are used
@@ -1615,6 +1638,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void decode_gemm_group_kernel(Gem
         lds_barrier();  // the tiles are free for the next unit
     }
     wait_all_memory();  // (requests of an item past the end return nothing, but must not outlive the wavefront's registers)
+    if constexpr (!WIDE_DYN && !PACKED) asm volatile("" ::"v"(touched[0]), "v"(touched[1]));  // (the touch above is a real request)
 
     // rows at or beyond sum(group_sizes): zero product, bias of the last group (lax.ragged_dot semantics)
     const int total = total_rows;
@@ -2173,6 +2197,8 @@ static int run_decode_gemm(const void* lhs, const int32_t* lhs_row_map, const vo
         return e ? atoi(e) : -1;
     }();
     p.snake = snake_env;
+    static const bool no_touch = getenv("LYRA_GEMM_NO_TOUCH") != nullptr;  // tuning override
+    p.touch_last = no_touch ? 0 : 1;
     p.even_spans = 0;
     p.residual = (const uint16_t*)residual;
     p.out_scale = out_scale;
