@@ -110,8 +110,20 @@ def test_decode_attention_at_drawn_shapes(seed):
     if gate is not None:
         want = want * gate[:, :, None, None]
     if d["f32"]:
+        # float32 output: held to what the kernel's one rounding allows - the probabilities enter the second product as
+        # bf16, so an element may be off by 2^-9 * A with A = sum_j p_j |v_j| (the oracle on the absolute values gives A);
+        # a gate adds one bf16 rounding of the result.  (With hundreds of keys this is the flat 4e-3 of the other tests;
+        # with a handful of keys nothing averages out and A is the size of a single value.)
+        v_abs = (case["v"][0] & np.uint8(0x7F), case["v"][1]) if d["fp8"] else np.abs(case["v"])
+        a = O.decode_attention_reference(case["q"], case["k"], v_abs, case["sinks"], sm_scale, d["sw"], d["pos"])
+        bound = 1e-3 + 2.0**-8 * a
+        if gate is not None:
+            bound = bound * gate[:, :, None, None] + 2.0**-8 * np.abs(want)
         got = run_attention(case, sm_scale, d["sw"], d["pos"], gate=gate, dtype=torch.float32)
-        U.assert_close(got, want, atol=4e-3 if gate is None else 8e-3, rtol=4e-3, what=f"draw {seed} f32")
+        err = np.abs(np.asarray(got, np.float32).reshape(want.shape) - want)
+        worst = int(np.argmax(err - bound))
+        assert np.isfinite(got).all() and (err <= bound).all(), \
+            f"draw {seed} f32: err {err.flat[worst]:.4g} > bound {bound.flat[worst]:.4g} at {worst}"
     else:
         got = run_attention(case, sm_scale, d["sw"], d["pos"], gate=gate)
         U.assert_close(got, want, what=f"draw {seed}")
