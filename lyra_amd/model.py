@@ -458,6 +458,11 @@ _SEPARATE_COMBINE = os.environ.get("LYRA_MOE_COMBINE_KERNEL") is not None  # tun
 _SEPARATE_QKV_POST = os.environ.get("LYRA_QKV_POST_KERNEL") is not None  # tuning override: QK norm + RoPE + cache append in a launch of its own
 _TILED_ACTIVATIONS = os.environ.get("LYRA_ROW_MAJOR_ACTIVATIONS") is None  # tuning override: expert matmuls read row-major activations
 _LOGIT_TILE_MAX = os.environ.get("LYRA_NO_LOGIT_TILE_MAX") is None  # tuning override: samplers read the whole vocabulary
+# Dense projections (q/k/v, output, MLP up and down) are handed to the kernels in the span-major copy whatever their width:
+# a K-split workgroup then reads one contiguous run per wavefront instead of pieces a weight row apart (0.2-0.3 us of each
+# 5-10 us launch).  Expert weights keep the reference's array unless their rows straddle cache lines (the copy costs the
+# expert kernel more than it gains there).  LYRA_SPAN_MAJOR_DENSE=0: the alignment rule for every array.
+_DENSE_SPAN_MAJOR = os.environ.get("LYRA_SPAN_MAJOR_DENSE", "1") != "0"
 
 
 @dataclass
@@ -497,7 +502,7 @@ def attention_apply_fused(x, w: AttentionWeights, idx: int, pos, cos_t, sin_t, c
         h, gate = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, w.sdpa_gate, None, gate=True, tiled=tiled)
     B = x.shape[0]
     one = _one_group(B, x.device)
-    w_qkv, w_out = F.span_major(w.qkv), F.span_major(w.out)  # (the arrays themselves unless their rows straddle cache lines)
+    w_qkv, w_out = F.span_major(w.qkv, always=_DENSE_SPAN_MAJOR), F.span_major(w.out, always=_DENSE_SPAN_MAJOR)
     # (:310-313: a bias is added to the projection's bf16 result, in bf16: by the attention launch that sums the slices when
     # that launch is certain to take them - one position for the batch, no learned exclusive self attention - else inside
     # the matmul's epilogue, which costs the launch that sums the slices)
@@ -568,7 +573,7 @@ def dense_mlp_apply_fused(x, w: DenseMLPWeights, cfg: ModelConfig):
     else:
         t, _ = F.rmsnorm_proj(x, w.norm_scale, cfg.norm_eps, tiled=tiled)
     one = _one_group(x.shape[0], x.device)
-    w_up, w_down = F.span_major(w.mlp_up), F.span_major(w.mlp_down)
+    w_up, w_down = F.span_major(w.mlp_up, always=_DENSE_SPAN_MAJOR), F.span_major(w.mlp_down, always=_DENSE_SPAN_MAJOR)
     t = F.gemm(t, w_up, one, fused_swiglu=True, swiglu_beta=cfg.swiglu_beta, swiglu_limit=cfg.swiglu_limit,
                bias=_bf16_bias(w.mlp_up_bias), out_tiled=tiled)
     # :628-636: projection, + bias, * residual scale, + residual, each a bf16 result - left to the norm that sums the slices
